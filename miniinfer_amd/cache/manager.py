@@ -1,0 +1,289 @@
+"""The cache manager: pages of keys and values with a block table per request, and slots of
+fixed-size per-request state.
+
+Layers are put into groups by what they need.  All layers that keep every key with the same
+geometry form one group; layers that keep a window of keys form another; each group has a page
+pool, a free list and block tables of its own, because its pages come back at other times (a
+window group gives a page back as soon as the window has passed it).  Layers whose mixer keeps
+a state of fixed size get a row in a state tensor, indexed by the request's slot.
+
+Everything here is host-side bookkeeping on Python lists; the only device memory is the page
+and state storage itself.  The reference keeps a token-granular table on the device and derives
+page tables from it at every step (miniinfer/kvcache/memory_pool.py:245-499,
+miniinfer/kvcache/kv_cache_manager.py:211-328,601-662); the rules kept from it are: a new page is
+opened exactly when a token crosses a page edge (memory_pool.py:217-242), a partial page is filled
+before a new one is opened, page 0 is never handed out (memory_pool.py:422-426), and a finished
+request gives everything back (kv_cache_manager.py:718-750).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..parts.base import FixedState, PagedKV
+
+
+class OutOfPages(RuntimeError):
+  pass
+
+
+class OutOfSlots(RuntimeError):
+  pass
+
+
+class CacheError(RuntimeError):
+  pass
+
+
+class PagePool:
+  """Free list of page ids 1..num_pages (page 0 is a scratch page that is never handed out).
+  Pages freed last are handed out first, so reuse shows early."""
+
+  def __init__(self, num_pages: int):
+    if num_pages <= 0:
+      raise ValueError("a page pool needs at least one page")
+    self.num_pages = num_pages
+    self._free: List[int] = list(range(num_pages, 0, -1))
+    self._held = bytearray(num_pages + 1)
+
+  @property
+  def num_free(self) -> int:
+    return len(self._free)
+
+  def alloc(self, n: int) -> List[int]:
+    if n > len(self._free):
+      raise OutOfPages(f"{n} pages wanted, {len(self._free)} free of {self.num_pages}")
+    out = [self._free.pop() for _ in range(n)]
+    for p in out:
+      if self._held[p]:
+        raise CacheError(f"page {p} was on the free list while held")
+      self._held[p] = 1
+    return out
+
+  def free(self, pages: Sequence[int]) -> None:
+    for p in pages:
+      if p <= 0 or p > self.num_pages:
+        raise CacheError(f"page id {p} does not exist")
+      if not self._held[p]:
+        raise CacheError(f"page {p} freed twice")
+      self._held[p] = 0
+      self._free.append(p)
+
+  def held(self) -> List[int]:
+    return [p for p in range(1, self.num_pages + 1) if self._held[p]]
+
+
+@dataclass
+class PagedGroup:
+  need: PagedKV
+  layers: List[int]
+  pool: PagePool
+  k: Optional[torch.Tensor] = None     # [len(layers), num_pages + 1, nkv, page_size, d]
+  v: Optional[torch.Tensor] = None
+  tables: Dict[Hashable, List[int]] = field(default_factory=dict)   # per request: page id per page index, 0 = given back
+
+
+@dataclass
+class StateGroup:
+  need: FixedState
+  layers: List[int]
+  state: Optional[torch.Tensor] = None  # [len(layers), max_requests, *shape]
+
+
+@dataclass
+class LayerCache:
+  """What one layer's mixer sees of the cache."""
+  kind: str                              # "paged" | "state" | "none"
+  group: int = -1
+  k: Optional[torch.Tensor] = None       # [num_pages + 1, nkv, page_size, d]
+  v: Optional[torch.Tensor] = None
+  state: Optional[torch.Tensor] = None   # [max_requests, *shape]
+  page_size: int = 0
+  window: Optional[int] = None
+
+
+class CacheManager:
+  def __init__(self, layer_needs: Sequence[object], page_size: int, num_pages: int, max_requests: int,
+               max_model_len: int, dtype: torch.dtype, device, allocate: bool = True):
+    """layer_needs[i] is the PagedKV / FixedState / None of layer i."""
+    if page_size <= 0 or page_size & (page_size - 1):
+      raise ValueError(f"page_size must be a power of two, got {page_size}")
+    self.page_size = page_size
+    self.num_pages = num_pages
+    self.max_requests = max_requests
+    self.max_model_len = max_model_len
+    self.max_pages_per_request = -(-max_model_len // page_size)
+    self.dtype = dtype
+    self.device = torch.device(device)
+    self.paged: List[PagedGroup] = []
+    self.states: List[StateGroup] = []
+    self._layer_map: List[Tuple[str, int, int]] = []
+    for i, need in enumerate(layer_needs):
+      if need is None:
+        self._layer_map.append(("none", -1, -1))
+      elif isinstance(need, PagedKV):
+        for gi, g in enumerate(self.paged):
+          if g.need == need:
+            break
+        else:
+          gi = len(self.paged)
+          self.paged.append(PagedGroup(need=need, layers=[], pool=PagePool(num_pages)))
+        self._layer_map.append(("paged", gi, len(self.paged[gi].layers)))
+        self.paged[gi].layers.append(i)
+      elif isinstance(need, FixedState):
+        for si, s in enumerate(self.states):
+          if s.need == need:
+            break
+        else:
+          si = len(self.states)
+          self.states.append(StateGroup(need=need, layers=[]))
+        self._layer_map.append(("state", si, len(self.states[si].layers)))
+        self.states[si].layers.append(i)
+      else:
+        raise TypeError(f"layer {i}: unknown cache need {need!r}")
+    self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
+    self._slot: Dict[Hashable, int] = {}
+    self._length: Dict[Hashable, int] = {}
+    if allocate:
+      self._allocate()
+
+  # ------------------------------------------------------------------ storage
+  @staticmethod
+  def bytes_per_page(layer_needs: Sequence[object], page_size: int, dtype: torch.dtype) -> int:
+    """Device bytes that one more page in every group costs."""
+    esize = torch.empty((), dtype=dtype).element_size()
+    return sum(2 * n.num_kv_heads * n.head_dim * page_size * esize for n in layer_needs if isinstance(n, PagedKV))
+
+  def _allocate(self) -> None:
+    for g in self.paged:
+      shape = (len(g.layers), self.num_pages + 1, g.need.num_kv_heads, self.page_size, g.need.head_dim)
+      g.k = torch.zeros(shape, dtype=self.dtype, device=self.device)
+      g.v = torch.zeros(shape, dtype=self.dtype, device=self.device)
+    for s in self.states:
+      shape = (len(s.layers), self.max_requests) + tuple(s.need.shape)
+      s.state = torch.zeros(shape, dtype=s.need.dtype or self.dtype, device=self.device)
+
+  def layer_cache(self, layer: int) -> LayerCache:
+    kind, gi, li = self._layer_map[layer]
+    if kind == "paged":
+      g = self.paged[gi]
+      return LayerCache(kind="paged", group=gi, k=None if g.k is None else g.k[li], v=None if g.v is None else g.v[li],
+                        page_size=self.page_size, window=g.need.window)
+    if kind == "state":
+      s = self.states[gi]
+      return LayerCache(kind="state", group=gi, state=None if s.state is None else s.state[li])
+    return LayerCache(kind="none")
+
+  # ------------------------------------------------------------------ requests
+  def has(self, req) -> bool:
+    return req in self._slot
+
+  def num_free_slots(self) -> int:
+    return len(self._free_slots)
+
+  def num_free_pages(self) -> int:
+    """Free pages of the tightest group."""
+    return min((g.pool.num_free for g in self.paged), default=self.num_pages)
+
+  def length(self, req) -> int:
+    return self._length[req]
+
+  def slot(self, req) -> int:
+    return self._slot[req]
+
+  def admit(self, req) -> int:
+    """A slot for a new request; its fixed-size state starts at zero."""
+    if req in self._slot:
+      raise CacheError(f"request {req!r} is admitted already")
+    if not self._free_slots:
+      raise OutOfSlots(f"all {self.max_requests} request slots are taken")
+    slot = self._free_slots.pop()
+    self._slot[req] = slot
+    self._length[req] = 0
+    for g in self.paged:
+      g.tables[req] = []
+    for s in self.states:
+      if s.state is not None:
+        s.state[:, slot].zero_()
+    return slot
+
+  def _first_needed_page(self, g: PagedGroup, next_pos: int) -> int:
+    """Index of the first page that the token at `next_pos` can still see."""
+    if g.need.window is None:
+      return 0
+    lo = max(0, next_pos - g.need.window + 1)
+    return lo // self.page_size
+
+  def pages_needed(self, req, new_len: int) -> int:
+    """Pages the tightest group must still hand out so that `req` can hold new_len tokens."""
+    have = len(self.paged[0].tables[req]) if self.paged else 0
+    return max(0, -(-new_len // self.page_size) - have)
+
+  def can_grow(self, req, new_len: int) -> bool:
+    return self.pages_needed(req, new_len) <= self.num_free_pages()
+
+  def grow(self, req, new_len: int) -> None:
+    """Make room for tokens up to position new_len - 1 in every group (all or nothing)."""
+    if new_len > self.max_model_len:
+      raise CacheError(f"request {req!r}: {new_len} tokens exceed max_model_len={self.max_model_len}")
+    if new_len < self._length[req]:
+      raise CacheError(f"request {req!r} cannot shrink from {self._length[req]} to {new_len}")
+    need = self.pages_needed(req, new_len)
+    if need > self.num_free_pages():
+      raise OutOfPages(f"request {req!r} needs {need} more pages, {self.num_free_pages()} are free")
+    for g in self.paged:
+      g.tables[req].extend(g.pool.alloc(need))
+
+  def commit(self, req, new_len: int) -> None:
+    """The step that wrote tokens up to new_len - 1 is done: record the length and give back
+    the pages of window groups that no later token can see."""
+    if new_len > len(self.paged[0].tables[req]) * self.page_size if self.paged else False:
+      raise CacheError(f"request {req!r}: commit of {new_len} tokens beyond its pages")
+    self._length[req] = new_len
+    for g in self.paged:
+      if g.need.window is None:
+        continue
+      table = g.tables[req]
+      first = min(self._first_needed_page(g, new_len), len(table))
+      gone = [p for p in table[:first] if p != 0]
+      if gone:
+        g.pool.free(gone)
+        for i in range(first):
+          table[i] = 0
+
+  def release(self, req) -> None:
+    """Everything the request holds comes back: its pages in every group and its slot."""
+    if req not in self._slot:
+      raise CacheError(f"request {req!r} is not admitted (released twice?)")
+    for g in self.paged:
+      g.pool.free([p for p in g.tables.pop(req) if p != 0])
+    self._free_slots.append(self._slot.pop(req))
+    del self._length[req]
+
+  def table(self, group: int, req) -> List[int]:
+    return self.paged[group].tables[req]
+
+  def live_requests(self) -> List[Hashable]:
+    return list(self._slot)
+
+  # ------------------------------------------------------------------ invariants (tests, debug)
+  def check(self) -> None:
+    """No page lost, none held twice, none both free and held; slots likewise."""
+    for gi, g in enumerate(self.paged):
+      held = [p for t in g.tables.values() for p in t if p != 0]
+      if len(held) != len(set(held)):
+        raise CacheError(f"group {gi}: a page is in two block tables")
+      if sorted(held) != g.pool.held():
+        raise CacheError(f"group {gi}: tables hold {sorted(held)}, the pool says {g.pool.held()}")
+      if len(held) + g.pool.num_free != g.pool.num_pages:
+        raise CacheError(f"group {gi}: {len(held)} held + {g.pool.num_free} free != {g.pool.num_pages}")
+      if len(set(g.pool._free)) != len(g.pool._free) or set(g.pool._free) & set(held):
+        raise CacheError(f"group {gi}: free list is inconsistent")
+    slots = list(self._slot.values())
+    if len(slots) != len(set(slots)) or set(slots) & set(self._free_slots):
+      raise CacheError("a request slot is held twice")
+    if len(slots) + len(self._free_slots) != self.max_requests:
+      raise CacheError("a request slot was lost")

@@ -1,0 +1,152 @@
+// Causal grouped-query attention over a paged cache, any dtype, any head size that is a
+// multiple of 8 up to 256, any number of new tokens per request (prompt portions and single
+// decoded tokens in one launch).  32-bit scores, softmax and accumulation, no matrix
+// instruction: this is the attention of the true 32-bit path and the any-shape fallback of
+// the bfloat16 path.
+//
+// For request b with q_len new tokens and kv_len keys after this step, new token i sits at
+// position p = kv_len - q_len + i and sees keys j with max(0, p - window + 1) <= j <= p
+// (window 0 = all): the bottom-right aligned causal mask of
+// miniinfer/layers/attention.py:112-128; query head h reads kv head h / (nq / nkv)
+// (miniinfer/layers/attention.py:131-191); softmax(scale * q.k) v.
+//
+// One wave per (token, query head).  A tile is 64 keys: each lane scores one key (the query
+// is broadcast from LDS), the wave reduces max and sum for the running softmax, then the lanes
+// switch to output columns and add the tile's probability-weighted value rows.
+#include "common.h"
+
+template <typename T, int VEC>
+__device__ __forceinline__ float dot_row(const float* __restrict__ qs, const T* __restrict__ row, int d);
+
+template <>
+__device__ __forceinline__ float dot_row<float, 4>(const float* __restrict__ qs, const float* __restrict__ row, int d) {
+  float acc = 0.f;
+  for (int e = 0; e < d; e += 4) {
+    const float4 kv = *reinterpret_cast<const float4*>(row + e);
+    acc = fmaf(qs[e], kv.x, acc);
+    acc = fmaf(qs[e + 1], kv.y, acc);
+    acc = fmaf(qs[e + 2], kv.z, acc);
+    acc = fmaf(qs[e + 3], kv.w, acc);
+  }
+  return acc;
+}
+
+template <>
+__device__ __forceinline__ float dot_row<bf16, 8>(const float* __restrict__ qs, const bf16* __restrict__ row, int d) {
+  float acc = 0.f;
+  for (int e = 0; e < d; e += 8) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(row + e);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      acc = fmaf(qs[e + 2 * i], __uint_as_float(w[i] << 16), acc);
+      acc = fmaf(qs[e + 2 * i + 1], __uint_as_float(w[i] & 0xffff0000u), acc);
+    }
+  }
+  return acc;
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void paged_attention_kernel(
+    const T* __restrict__ q, int64_t q_row_stride, T* __restrict__ out, int64_t out_row_stride,
+    const T* __restrict__ k_pages, const T* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
+    const int* __restrict__ token_req, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int num_tokens,
+    int nq, int nkv, int d, int page_shift, float scale, int window) {
+  extern __shared__ float smem[];
+  const int lane = threadIdx.x & (MI_WAVE - 1);
+  const int wave = threadIdx.x / MI_WAVE;
+  float* qs = smem + wave * d;
+  const int64_t wid = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + wave;
+  const bool live = wid < (int64_t)num_tokens * nq;
+  int t = 0, h = 0;
+  if (live) {
+    t = (int)(wid / nq);
+    h = (int)(wid - (int64_t)t * nq);
+    const T* qr = q + (int64_t)t * q_row_stride + (int64_t)h * d;
+    for (int e = lane; e < d; e += MI_WAVE) qs[e] = to_float(qr[e]);
+  }
+  __syncthreads();
+  if (!live) return;
+
+  const int b = token_req[t];
+  const int q_begin = cu_q[b];
+  const int q_len = cu_q[b + 1] - q_begin;
+  const int pos = kv_len[b] - q_len + (t - q_begin);
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int g = h / (nq / nkv);
+  const int P = 1 << page_shift;
+  const int* bt = block_table + (int64_t)b * table_width;
+
+  float m = -INFINITY, l = 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+
+  for (int j0 = lo; j0 <= pos; j0 += MI_WAVE) {
+    const int j = j0 + lane;
+    float s = -INFINITY;
+    if (j <= pos) {
+      const int64_t page = bt[j >> page_shift];
+      const T* row = k_pages + ((page * nkv + g) * P + (j & (P - 1))) * d;
+      s = dot_row<T, VEC>(qs, row, d) * scale;
+    }
+    const float m_new = fmaxf(m, wave_max(s));   // the tile's first key is visible, so m_new is finite
+    const float p = (j <= pos) ? expf(s - m_new) : 0.f;
+    const float alpha = expf(m - m_new);         // 0 on the first tile (m = -inf)
+    l = l * alpha + wave_sum(p);
+    m = m_new;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] *= alpha;
+    const int n = (pos - j0 + 1 < MI_WAVE) ? pos - j0 + 1 : MI_WAVE;
+    for (int i = 0; i < n; ++i) {
+      const float pi = __shfl(p, i, MI_WAVE);
+      const int jj = j0 + i;
+      const int64_t page = bt[jj >> page_shift];
+      const T* vrow = v_pages + ((page * nkv + g) * P + (jj & (P - 1))) * d;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int e = lane + c * MI_WAVE;
+        if (e < d) acc[c] = fmaf(pi, to_float(vrow[e]), acc[c]);
+      }
+    }
+  }
+  T* o = out + (int64_t)t * out_row_stride + (int64_t)h * d;
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int e = lane + c * MI_WAVE;
+    if (e < d) o[e] = from_float<T>(acc[c] * inv);
+  }
+}
+
+MI_EXPORT int mi_paged_attention(int dtype, const void* q, int64_t q_row_stride, void* out, int64_t out_row_stride,
+                                 const void* k_pages, const void* v_pages, const int* block_table, int table_width,
+                                 const int* token_req, const int* cu_q, const int* kv_len, int num_tokens,
+                                 int num_requests, int nq, int nkv, int d, int page_size, float scale, int window,
+                                 hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && num_requests >= 0 && nq > 0 && nkv > 0, "paged_attention: bad sizes");
+  MI_REQUIRE(nq % nkv == 0, "paged_attention: %d query heads are no multiple of %d kv heads", nq, nkv);
+  MI_REQUIRE(d > 0 && d % 8 == 0 && d <= 256, "paged_attention: head size %d is not a multiple of 8 up to 256", d);
+  MI_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0, "paged_attention: page size %d is no power of two",
+             page_size);
+  MI_REQUIRE(q_row_stride >= (int64_t)nq * d && out_row_stride >= (int64_t)nq * d, "paged_attention: row strides too small");
+  MI_REQUIRE(q_row_stride % 8 == 0, "paged_attention: query row stride %lld is not a multiple of 8", (long long)q_row_stride);
+  MI_REQUIRE(window >= 0 && table_width > 0, "paged_attention: bad window or table width");
+  if (num_tokens == 0) return 0;
+  int shift = 0;
+  while ((1 << shift) < page_size) ++shift;
+  const int waves_per_block = 4;
+  const int64_t waves = (int64_t)num_tokens * nq;
+  const int blocks = (int)((waves + waves_per_block - 1) / waves_per_block);
+  const size_t lds = (size_t)waves_per_block * d * sizeof(float);
+  if (dtype == MI_DTYPE_F32)
+    paged_attention_kernel<float, 4><<<blocks, waves_per_block * MI_WAVE, lds, stream>>>(
+        (const float*)q, q_row_stride, (float*)out, out_row_stride, (const float*)k_pages, (const float*)v_pages,
+        block_table, table_width, token_req, cu_q, kv_len, num_tokens, nq, nkv, d, shift, scale, window);
+  else if (dtype == MI_DTYPE_BF16)
+    paged_attention_kernel<bf16, 8><<<blocks, waves_per_block * MI_WAVE, lds, stream>>>(
+        (const bf16*)q, q_row_stride, (bf16*)out, out_row_stride, (const bf16*)k_pages, (const bf16*)v_pages,
+        block_table, table_width, token_req, cu_q, kv_len, num_tokens, nq, nkv, d, shift, scale, window);
+  else
+    MI_FAIL("paged_attention: unknown dtype %d", dtype);
+  MI_CHECK_LAUNCH("paged_attention");
+  return 0;
+}

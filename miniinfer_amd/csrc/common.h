@@ -1,0 +1,98 @@
+// Shared device helpers for the gfx950 (CDNA4, wave64) kernels of this library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#define MI_WAVE 64
+
+// ---------------------------------------------------------------- error reporting (host)
+// Every entry point returns 0 on success; otherwise the message is read with mi_last_error().
+static thread_local char g_mi_error[512] = {0};
+
+#define MI_FAIL(...)                                            \
+  do {                                                          \
+    snprintf(g_mi_error, sizeof(g_mi_error), __VA_ARGS__);      \
+    return 1;                                                   \
+  } while (0)
+
+#define MI_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) MI_FAIL(__VA_ARGS__); \
+  } while (0)
+
+#define MI_CHECK_LAUNCH(name)                                                   \
+  do {                                                                          \
+    hipError_t e_ = hipGetLastError();                                          \
+    if (e_ != hipSuccess) MI_FAIL("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+  } while (0)
+
+#define MI_EXPORT extern "C" __attribute__((visibility("default")))
+
+// ---------------------------------------------------------------- bfloat16 as raw bits
+struct bf16 {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16 x) { return bf16_bits_to_float(x.bits); }
+
+template <typename T>
+__device__ __forceinline__ T from_float(float x);
+template <>
+__device__ __forceinline__ float from_float<float>(float x) { return x; }
+template <>
+__device__ __forceinline__ bf16 from_float<bf16>(float x) {
+  bf16 r;
+  r.bits = float_to_bf16_bits(x);
+  return r;
+}
+
+// ---------------------------------------------------------------- reductions
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = MI_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, MI_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = MI_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MI_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds 16 floats of LDS. Every thread gets the sum.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (MI_WAVE - 1);
+  const int wave = threadIdx.x / MI_WAVE;
+  const int nwaves = (blockDim.x + MI_WAVE - 1) / MI_WAVE;
+  v = wave_sum(v);
+  __syncthreads();  // scratch may still be read from an earlier call
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nwaves; ++i) t += scratch[i];
+  return t;
+}
+
+static inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+// one translation unit per shared object: each exports its own message reader
+MI_EXPORT const char* mi_last_error() { return g_mi_error; }
+
+#define MI_DTYPE_F32 0
+#define MI_DTYPE_BF16 1

@@ -1,0 +1,252 @@
+// Row-wise kernels of the decoder: embedding gather, (residual add +) RMS norm, SiLU*mul,
+// and the fused per-head norm + rotary + cache write.  All arithmetic is 32-bit; values are
+// rounded once, when they are stored in the activation dtype.
+//
+// Formulas restate tom-jerr/MiniInfer: layers/embedding.py:27 (gather), layers/layernorm.py:22-32
+// and kernels/triton/rms_norm.py:84-101 (norm, add + norm), kernels/triton/silu_mul.py:33-37,
+// models/fused_qwen3.py:98-105 with layers/position_encoding.py:91-117 (per-head norm, rotation),
+// kvcache/memory_pool.py:55-56 (cache write).
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
+                             int H, int V) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  const bool ok = id >= 0 && id < V;
+  const T* row = table + (int64_t)(ok ? id : 0) * H;
+  float* o = out + (int64_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ok ? to_float(row[i]) : __builtin_nanf("");
+}
+
+MI_EXPORT int mi_embed(int dtype, const void* table, const int* ids, float* out, int T, int H, int V,
+                       hipStream_t stream) {
+  MI_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+  if (T == 0) return 0;
+  const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+  if (dtype == MI_DTYPE_F32)
+    embed_kernel<float><<<T, threads, 0, stream>>>((const float*)table, ids, out, H, V);
+  else if (dtype == MI_DTYPE_BF16)
+    embed_kernel<bf16><<<T, threads, 0, stream>>>((const bf16*)table, ids, out, H, V);
+  else
+    MI_FAIL("embed: unknown dtype %d", dtype);
+  MI_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------- (add +) RMS norm
+// For output row i (source row s = rows ? rows[i] : i):
+//   v = residual[s] + x[s]      (either may be absent)
+//   residual[s] = v             (when write_back; never with `rows`)
+//   y[i] = v * rsqrt(mean(v^2) + eps) * w
+template <typename TX, typename TY>
+__global__ void add_rmsnorm_kernel(const TX* __restrict__ x, float* __restrict__ residual,
+                                   const float* __restrict__ w, TY* __restrict__ y, const int* __restrict__ rows,
+                                   int N, float eps, int write_back) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const int64_t s = rows ? rows[i] : i;
+  const TX* xr = x ? x + s * N : nullptr;
+  float* rr = residual ? residual + s * N : nullptr;
+  TY* yr = y + (int64_t)i * N;
+
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < N; c += blockDim.x) {
+    float v = 0.f;
+    if (rr) v = rr[c];
+    if (xr) v += to_float(xr[c]);
+    if (write_back) rr[c] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = rsqrtf(ss / (float)N + eps);
+  for (int c = threadIdx.x; c < N; c += blockDim.x) {
+    float v;
+    if (write_back) {
+      v = rr[c];  // this thread wrote it above
+    } else {
+      v = 0.f;
+      if (rr) v = rr[c];
+      if (xr) v += to_float(xr[c]);
+    }
+    yr[c] = from_float<TY>(v * rstd * w[c]);
+  }
+}
+
+// x_dtype: dtype of x (ignored when x is null); y_dtype: dtype of y.
+MI_EXPORT int mi_add_rmsnorm(int x_dtype, int y_dtype, const void* x, float* residual, const float* w, void* y,
+                             const int* rows, int M, int N, float eps, int write_back, hipStream_t stream) {
+  MI_REQUIRE(M >= 0 && N > 0, "add_rmsnorm: bad sizes M=%d N=%d", M, N);
+  MI_REQUIRE(x || residual, "add_rmsnorm: neither x nor residual given");
+  MI_REQUIRE(!(write_back && rows), "add_rmsnorm: write_back with a row selection is not defined");
+  MI_REQUIRE(!(write_back && !residual), "add_rmsnorm: write_back without a residual");
+  if (M == 0) return 0;
+  const int threads = N >= 2048 ? 512 : (N >= 512 ? 256 : (N >= 128 ? 128 : 64));
+#define LAUNCH(TX, TY)                                                                                       \
+  add_rmsnorm_kernel<TX, TY><<<M, threads, 0, stream>>>((const TX*)x, residual, w, (TY*)y, rows, N, eps, \
+                                                        write_back)
+  if (!x) x_dtype = MI_DTYPE_F32;
+  if (x_dtype == MI_DTYPE_F32 && y_dtype == MI_DTYPE_F32) LAUNCH(float, float);
+  else if (x_dtype == MI_DTYPE_BF16 && y_dtype == MI_DTYPE_BF16) LAUNCH(bf16, bf16);
+  else if (x_dtype == MI_DTYPE_F32 && y_dtype == MI_DTYPE_BF16) LAUNCH(float, bf16);
+  else if (x_dtype == MI_DTYPE_BF16 && y_dtype == MI_DTYPE_F32) LAUNCH(bf16, float);
+  else MI_FAIL("add_rmsnorm: unknown dtypes %d %d", x_dtype, y_dtype);
+#undef LAUNCH
+  MI_CHECK_LAUNCH("add_rmsnorm");
+  return 0;
+}
+
+// ---------------------------------------------------------------- SiLU(gate) * up
+// gu [M, 2I]: gate = first I columns, up = last I.  out [M, I].
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int M, int I) {
+  const int64_t total = (int64_t)M * I;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = idx / I;
+    const int c = (int)(idx - m * I);
+    const float g = to_float(gu[m * 2 * I + c]);
+    const float u = to_float(gu[m * 2 * I + I + c]);
+    const float s = g / (1.f + expf(-g));
+    out[idx] = from_float<T>(s * u);
+  }
+}
+
+MI_EXPORT int mi_silu_mul(int dtype, const void* gu, void* out, int M, int I, hipStream_t stream) {
+  MI_REQUIRE(M >= 0 && I > 0, "silu_mul: bad sizes M=%d I=%d", M, I);
+  if (M == 0) return 0;
+  const int64_t total = (int64_t)M * I;
+  const int threads = 256;
+  int64_t blocks = (total + threads - 1) / threads;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == MI_DTYPE_F32)
+    silu_mul_kernel<float><<<(int)blocks, threads, 0, stream>>>((const float*)gu, (float*)out, M, I);
+  else if (dtype == MI_DTYPE_BF16)
+    silu_mul_kernel<bf16><<<(int)blocks, threads, 0, stream>>>((const bf16*)gu, (bf16*)out, M, I);
+  else
+    MI_FAIL("silu_mul: unknown dtype %d", dtype);
+  MI_CHECK_LAUNCH("silu_mul");
+  return 0;
+}
+
+// ---------------------------------------------------------------- per-head norm + rotary + cache write
+// qkv [T, (nq + 2 nkv) d] with heads ordered q | k | v.  One wave per (token, head):
+//   q heads: norm (if qw) and rotation (if cos_sin), written back in place;
+//   k heads: the same with kw, written to the key pages (and back in place);
+//   v heads: copied to the value pages.
+// Pages are [num_pages, nkv, P, d]; token t goes to slot slots[t] = page * P + offset.
+// cos_sin [max_pos, rotary_dim] = cos(pos * inv_freq_j) for j < rotary_dim/2, then sin(...).
+// Pairs are (j, j + rotary_dim/2) within the first rotary_dim elements; the rest pass through.
+template <typename T>
+__global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
+                                          const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+                                          const float* __restrict__ cos_sin, int rotary_dim, int max_pos,
+                                          const int* __restrict__ positions, T* __restrict__ k_pages,
+                                          T* __restrict__ v_pages, const int* __restrict__ slots, int page_shift,
+                                          int num_tokens) {
+  const int lane = threadIdx.x & (MI_WAVE - 1);
+  const int heads = nq + 2 * nkv;
+  const int64_t wid = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + threadIdx.x / MI_WAVE;
+  if (wid >= (int64_t)num_tokens * heads) return;
+  const int t = (int)(wid / heads);
+  const int h = (int)(wid - (int64_t)t * heads);
+  T* src = qkv + (int64_t)t * row_stride + (int64_t)h * d;
+  const int P = 1 << page_shift;
+
+  T* dst = nullptr;  // where the cache copy goes
+  if (h >= nq && k_pages) {
+    const int slot = slots[t];
+    const int64_t page = slot >> page_shift;
+    const int off = slot & (P - 1);
+    const int g = (h - nq) % nkv;
+    T* base = (h < nq + nkv) ? k_pages : v_pages;
+    dst = base + ((page * nkv + g) * P + off) * d;
+  }
+
+  if (h >= nq + nkv) {  // value head: plain copy
+    if (dst)
+      for (int e = lane; e < d; e += MI_WAVE) dst[e] = src[e];
+    return;
+  }
+
+  const float* w = (h < nq) ? qw : kw;
+  float rstd = 1.f;
+  if (w) {
+    float ss = 0.f;
+    for (int e = lane; e < d; e += MI_WAVE) {
+      const float v = to_float(src[e]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    rstd = rsqrtf(ss / (float)d + eps);
+  }
+  const int half = cos_sin ? rotary_dim / 2 : 0;
+  const int rd = cos_sin ? rotary_dim : 0;
+  int pos = positions ? positions[t] : 0;
+  pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+  const float* cs = cos_sin ? cos_sin + (int64_t)pos * rotary_dim : nullptr;
+
+  for (int e = lane; e < d; e += MI_WAVE) {
+    if (e < half) {
+      const int e2 = e + half;
+      float x1 = to_float(src[e]) * rstd;
+      float x2 = to_float(src[e2]) * rstd;
+      if (w) {
+        x1 *= w[e];
+        x2 *= w[e2];
+      }
+      const float c = cs[e], s = cs[half + e];
+      const T o1 = from_float<T>(x1 * c - x2 * s);
+      const T o2 = from_float<T>(x2 * c + x1 * s);
+      src[e] = o1;
+      src[e2] = o2;
+      if (dst) {
+        dst[e] = o1;
+        dst[e2] = o2;
+      }
+    } else if (e >= rd) {
+      float x1 = to_float(src[e]) * rstd;
+      if (w) x1 *= w[e];
+      const T o = from_float<T>(x1);
+      src[e] = o;
+      if (dst) dst[e] = o;
+    }
+  }
+}
+
+MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nq, int nkv, int d,
+                                    const float* qw, const float* kw, float eps, const float* cos_sin,
+                                    int rotary_dim, int max_pos, const int* positions, void* k_pages, void* v_pages,
+                                    const int* slots, int page_size, hipStream_t stream) {
+  MI_REQUIRE(num_tokens >= 0 && nq > 0 && nkv > 0 && d > 0, "qk_norm_rope_cache: bad sizes");
+  MI_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qk_norm_rope_cache: row stride %lld too small",
+             (long long)row_stride);
+  MI_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0, "qk_norm_rope_cache: page size %d is no power of two",
+             page_size);
+  if (cos_sin) {
+    MI_REQUIRE(rotary_dim > 0 && rotary_dim % 2 == 0 && rotary_dim <= d, "qk_norm_rope_cache: rotary_dim %d for head %d",
+               rotary_dim, d);
+    MI_REQUIRE(positions != nullptr && max_pos > 0, "qk_norm_rope_cache: rotation without positions");
+  }
+  MI_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "qk_norm_rope_cache: key and value pages go together");
+  MI_REQUIRE(!k_pages || slots, "qk_norm_rope_cache: cache write without slots");
+  if (num_tokens == 0) return 0;
+  int shift = 0;
+  while ((1 << shift) < page_size) ++shift;
+  const int waves_per_block = 4;
+  const int64_t waves = (int64_t)num_tokens * (nq + 2 * nkv);
+  const int blocks = (int)((waves + waves_per_block - 1) / waves_per_block);
+  if (dtype == MI_DTYPE_F32)
+    qk_norm_rope_cache_kernel<float><<<blocks, waves_per_block * MI_WAVE, 0, stream>>>(
+        (float*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (float*)k_pages,
+        (float*)v_pages, slots, shift, num_tokens);
+  else if (dtype == MI_DTYPE_BF16)
+    qk_norm_rope_cache_kernel<bf16><<<blocks, waves_per_block * MI_WAVE, 0, stream>>>(
+        (bf16*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (bf16*)k_pages,
+        (bf16*)v_pages, slots, shift, num_tokens);
+  else
+    MI_FAIL("qk_norm_rope_cache: unknown dtype %d", dtype);
+  MI_CHECK_LAUNCH("qk_norm_rope_cache");
+  return 0;
+}

@@ -1,0 +1,272 @@
+"""Python face of the HIP kernels: checks shapes, dtypes and devices on the host, then launches
+on the current HIP stream.  Tensors are torch tensors used as plain device buffers.
+
+There is no CPU path and no library fallback: a tensor that is not on the GPU, or a shape a
+kernel does not take, raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+from typing import Optional
+
+import torch
+
+from . import jit
+
+F32, BF16 = 0, 1
+
+
+class KernelError(RuntimeError):
+  pass
+
+
+def dtype_code(dt: torch.dtype) -> int:
+  if dt == torch.float32:
+    return F32
+  if dt == torch.bfloat16:
+    return BF16
+  raise KernelError(f"dtype {dt} is not supported by the HIP kernels (float32 and bfloat16 are)")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+  return None if t is None else t.data_ptr()
+
+
+def _stream():
+  return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(*tensors):
+  for t in tensors:
+    if t is not None and not t.is_cuda:
+      raise KernelError("miniinfer_amd kernels run on the GPU only; got a tensor on " + str(t.device))
+
+
+def _contig(name, t):
+  if t is not None and not t.is_contiguous():
+    raise KernelError(f"{name} must be contiguous")
+
+
+def _i32(name, t, n=None):
+  if t is None:
+    return
+  if t.dtype != torch.int32:
+    raise KernelError(f"{name} must be int32, got {t.dtype}")
+  _contig(name, t)
+  if n is not None and t.numel() < n:
+    raise KernelError(f"{name} has {t.numel()} elements, {n} are needed")
+
+
+def _f32(name, t, n=None):
+  if t is None:
+    return
+  if t.dtype != torch.float32:
+    raise KernelError(f"{name} must be float32, got {t.dtype}")
+  _contig(name, t)
+  if n is not None and t.numel() != n:
+    raise KernelError(f"{name} has {t.numel()} elements, {n} are expected")
+
+
+_SIGS = {
+  "elementwise": {
+    "mi_embed": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "mi_add_rmsnorm": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
+                       c_void_p],
+    "mi_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "mi_qk_norm_rope_cache": [c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
+                              c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+  },
+  "gemm": {
+    "mi_gemm_nt": [c_int, c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int,
+                   c_void_p],
+  },
+  "attention": {
+    "mi_paged_attention": [c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
+                           c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                           c_void_p],
+  },
+}
+
+_libs = {}
+
+
+def _lib(name: str, defines=()):
+  key = (name, tuple(sorted(defines)))
+  lib = _libs.get(key)
+  if lib is None:
+    lib = jit.load_module(name, defines)
+    for fn, sig in _SIGS.get(name, {}).items():
+      f = getattr(lib, fn)
+      f.argtypes = sig
+      f.restype = c_int
+    _libs[key] = lib
+  return lib
+
+
+def _check(lib, rc):
+  if rc != 0:
+    raise KernelError(lib.mi_last_error().decode())
+
+
+def modules_for(spec_kinds=()):
+  """(name, defines) of every shared object the plain kernel set needs."""
+  return [("elementwise", ()), ("gemm", ()), ("attention", ())]
+
+
+# ----------------------------------------------------------------------------- embedding
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+  """out[t, :] = float32(table[ids[t], :]).  An id outside the table gives a row of NaN."""
+  _dev(table, ids, out)
+  V, H = table.shape
+  T = ids.numel()
+  _contig("table", table)
+  _i32("ids", ids)
+  _f32("out", out, T * H)
+  lib = _lib("elementwise")
+  _check(lib, lib.mi_embed(dtype_code(table.dtype), _ptr(table), _ptr(ids), _ptr(out), T, H, V, _stream()))
+  return out
+
+
+# ----------------------------------------------------------------------------- norms
+
+def add_rmsnorm(x: Optional[torch.Tensor], residual: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_back: bool = False) -> torch.Tensor:
+  """out[i] = rmsnorm(residual[s] + x[s]) * weight with s = rows[i] (or i); 32-bit arithmetic.
+  x [M, N] in float32 or bfloat16 (may be None), residual [M, N] float32 (may be None; updated in
+  place to the sum when `write_back`)."""
+  _dev(x, residual, weight, out, rows)
+  N = weight.numel()
+  _f32("weight", weight)
+  src = x if x is not None else residual
+  if src is None:
+    raise KernelError("add_rmsnorm needs x or a residual")
+  if src.shape[-1] != N:
+    raise KernelError(f"add_rmsnorm: rows of {src.shape[-1]} elements, weight of {N}")
+  M_src = src.numel() // N
+  for name, t in (("x", x), ("residual", residual)):
+    if t is not None:
+      _contig(name, t)
+      if t.numel() != M_src * N:
+        raise KernelError(f"add_rmsnorm: {name} has another shape than its partner")
+  if residual is not None and residual.dtype != torch.float32:
+    raise KernelError("add_rmsnorm: the residual stream is float32")
+  if rows is not None:
+    _i32("rows", rows)
+    M = rows.numel()
+  else:
+    M = M_src
+  _contig("out", out)
+  if out.numel() != M * N:
+    raise KernelError(f"add_rmsnorm: out has {out.numel()} elements, {M * N} are expected")
+  lib = _lib("elementwise")
+  _check(lib, lib.mi_add_rmsnorm(dtype_code(x.dtype) if x is not None else F32, dtype_code(out.dtype), _ptr(x),
+                                 _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), M, N, float(eps),
+                                 1 if write_back else 0, _stream()))
+  return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+  """out[m, c] = silu(gate_up[m, c]) * gate_up[m, I + c]."""
+  _dev(gate_up, out)
+  _contig("gate_up", gate_up)
+  _contig("out", out)
+  M, I2 = gate_up.shape
+  if I2 % 2 or out.shape != (M, I2 // 2) or out.dtype != gate_up.dtype:
+    raise KernelError(f"silu_mul: gate_up {tuple(gate_up.shape)} and out {tuple(out.shape)} do not fit")
+  lib = _lib("elementwise")
+  _check(lib, lib.mi_silu_mul(dtype_code(gate_up.dtype), _ptr(gate_up), _ptr(out), M, I2 // 2, _stream()))
+  return out
+
+
+def qk_norm_rope_cache(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: Optional[torch.Tensor],
+                       k_weight: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
+                       positions: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                       v_pages: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> None:
+  """In place on qkv [T, (nq + 2 nkv) d]: per-head RMS norm of q and k (if weights), rotation of q and k
+  (if cos_sin [max_pos, rotary_dim]), and a copy of the new k and v rows into pages
+  [num_pages, nkv, page_size, d] at slots[t] = page * page_size + offset."""
+  _dev(qkv, q_weight, k_weight, cos_sin, positions, k_pages, v_pages, slots)
+  if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] != (nq + 2 * nkv) * d:
+    raise KernelError(f"qk_norm_rope_cache: qkv {tuple(qkv.shape)} does not hold {nq}+2*{nkv} heads of {d}")
+  T = qkv.shape[0]
+  _f32("q_weight", q_weight, d)
+  _f32("k_weight", k_weight, d)
+  rotary_dim, max_pos = 0, 0
+  if cos_sin is not None:
+    _f32("cos_sin", cos_sin)
+    max_pos, rotary_dim = cos_sin.shape
+    _i32("positions", positions, T)
+  if k_pages is not None:
+    for name, p in (("k_pages", k_pages), ("v_pages", v_pages)):
+      _contig(name, p)
+      if p.dtype != qkv.dtype or p.dim() != 4 or tuple(p.shape[1:]) != (nkv, page_size, d):
+        raise KernelError(f"qk_norm_rope_cache: {name} {tuple(p.shape)} {p.dtype} is not [pages, {nkv}, {page_size}, {d}] "
+                          f"of {qkv.dtype}")
+    _i32("slots", slots, T)
+  lib = _lib("elementwise")
+  _check(lib, lib.mi_qk_norm_rope_cache(dtype_code(qkv.dtype), _ptr(qkv), qkv.stride(0), T, nq, nkv, d,
+                                        _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin), rotary_dim,
+                                        max_pos, _ptr(positions), _ptr(k_pages), _ptr(v_pages), _ptr(slots),
+                                        page_size, _stream()))
+
+
+# ----------------------------------------------------------------------------- matrix product
+
+def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+  """out[M, N] = a[M, K] @ w[N, K]^T with 32-bit FMA accumulation (no matrix instruction).
+  a and w share a dtype; out is that dtype or float32.  Rows may be strided, columns are dense."""
+  _dev(a, w, out)
+  if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+    raise KernelError("gemm_nt takes matrices")
+  M, K = a.shape
+  N, K2 = w.shape
+  if K != K2 or tuple(out.shape) != (M, N):
+    raise KernelError(f"gemm_nt: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+  if a.dtype != w.dtype:
+    raise KernelError(f"gemm_nt: a is {a.dtype}, w is {w.dtype}")
+  for name, t in (("a", a), ("w", w), ("out", out)):
+    if t.stride(1) != 1:
+      raise KernelError(f"gemm_nt: {name} must have dense rows")
+  lib = _lib("gemm")
+  _check(lib, lib.mi_gemm_nt(dtype_code(a.dtype), dtype_code(out.dtype), _ptr(a), a.stride(0) if M > 1 else K,
+                             _ptr(w), w.stride(0) if N > 1 else K, _ptr(out), out.stride(0) if M > 1 else N,
+                             M, N, K, _stream()))
+  return out
+
+
+# ----------------------------------------------------------------------------- attention
+
+def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
+                    v_pages: torch.Tensor, block_table: torch.Tensor, token_req: torch.Tensor, cu_q: torch.Tensor,
+                    kv_len: torch.Tensor, scale: float, window: int = 0) -> torch.Tensor:
+  """Causal attention of new tokens over their requests' paged keys and values.
+
+  q: [T, >= nq*d] rows (the q part of a fused qkv buffer is fine), out [T, nq*d];
+  pages [num_pages, nkv, P, d]; block_table [B, W] int32; token_req [T] = request of each token;
+  cu_q [B+1] = first token of each request; kv_len [B] = keys per request including the new tokens."""
+  _dev(q, out, k_pages, v_pages, block_table, token_req, cu_q, kv_len)
+  T = q.shape[0]
+  B = kv_len.numel()
+  if q.stride(1) != 1 or q.shape[1] < nq * d or out.stride(1) != 1 or out.shape != (T, nq * d):
+    raise KernelError(f"paged_attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not hold {nq} heads of {d}")
+  if k_pages.shape != v_pages.shape or k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d:
+    raise KernelError(f"paged_attention: pages {tuple(k_pages.shape)} are not [pages, {nkv}, P, {d}]")
+  if not (q.dtype == out.dtype == k_pages.dtype == v_pages.dtype):
+    raise KernelError("paged_attention: q, out and pages must share a dtype")
+  _contig("k_pages", k_pages)
+  _contig("v_pages", v_pages)
+  _i32("block_table", block_table)
+  if block_table.dim() != 2 or block_table.shape[0] < B:
+    raise KernelError(f"paged_attention: block_table {tuple(block_table.shape)} for {B} requests")
+  _i32("token_req", token_req, T)
+  _i32("cu_q", cu_q, B + 1)
+  _i32("kv_len", kv_len, B)
+  lib = _lib("attention")
+  _check(lib, lib.mi_paged_attention(dtype_code(q.dtype), _ptr(q), q.stride(0), _ptr(out), out.stride(0),
+                                     _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
+                                     _ptr(token_req), _ptr(cu_q), _ptr(kv_len), T, B, nq, nkv, d,
+                                     k_pages.shape[2], float(scale), int(window), _stream()))
+  return out

@@ -1,0 +1,73 @@
+"""Causal grouped-query attention over the paged cache (the mixer of Qwen3).
+
+Order of operations, as miniinfer/models/fused_qwen3.py:95-107: one fused QKV projection
+(rows q | k | v, no bias), per-head RMS norm of q and k, rotation of q and k, the new keys and
+values written to their cache slots before attention (flashinfer_backend.py:341-348), attention
+of the new tokens over all cached keys of their request, output projection.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Tuple
+
+import torch
+
+from ..kernels import ops
+from .base import (BuildContext, NORMS, POSITIONS, PagedKV, ParamSpec, Part, Source, register_mixer)
+from .linear import linear
+
+
+class PagedAttention(Part):
+  def __init__(self, spec, ctx: BuildContext):
+    if spec.num_heads % spec.num_kv_heads:
+      raise ValueError(f"{spec.num_heads} query heads are no multiple of {spec.num_kv_heads} kv heads")
+    if spec.head_dim % 8 or spec.head_dim > 256:
+      raise ValueError(f"head_dim={spec.head_dim} is not supported: the attention kernels take multiples of 8 up to 256")
+    self.spec = spec
+    self.ctx = ctx
+    self.nq, self.nkv, self.d = spec.num_heads, spec.num_kv_heads, spec.head_dim
+    self.hidden = spec.hidden_size
+    self.scale = float(spec.scale)
+    self.window = spec.window
+    self.position = POSITIONS.build(spec.position, ctx)
+    self.q_norm = NORMS.build(spec.qk_norm, ctx) if spec.qk_norm is not None else None
+    self.k_norm = NORMS.build(spec.qk_norm, ctx) if spec.qk_norm is not None else None
+    self.qkv_weight: Optional[torch.Tensor] = None
+    self.o_weight: Optional[torch.Tensor] = None
+
+  # ------------------------------------------------------------------ tensors
+  def param_specs(self) -> List[ParamSpec]:
+    qn, kn, vn, on = self.spec.tensor_names[:4]
+    nq, nkv, d, H = self.nq, self.nkv, self.d, self.hidden
+    return [
+      ParamSpec("qkv_weight", ((nq + 2 * nkv) * d, H),
+                (Source(qn + ".weight", nq * d), Source(kn + ".weight", nkv * d), Source(vn + ".weight", nkv * d))),
+      ParamSpec("o_weight", (H, nq * d), (Source(on + ".weight", H),)),
+    ]
+
+  def children(self) -> List[Tuple[str, Part]]:
+    if self.q_norm is None:
+      return []
+    return [(self.spec.tensor_names[4] + ".", self.q_norm), (self.spec.tensor_names[5] + ".", self.k_norm)]
+
+  def cache_requirement(self):
+    return PagedKV(num_kv_heads=self.nkv, head_dim=self.d, window=self.window)
+
+  # ------------------------------------------------------------------ one step
+  def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+    T = x.shape[0]
+    qkv = linear(x, self.qkv_weight)
+    table = self.position.rotary_table()
+    eps = self.q_norm.eps if self.q_norm is not None else 0.0
+    ops.qk_norm_rope_cache(
+      qkv, self.nq, self.nkv, self.d,
+      self.q_norm.weight if self.q_norm is not None else None,
+      self.k_norm.weight if self.k_norm is not None else None,
+      eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
+    out = torch.empty((T, self.nq * self.d), dtype=x.dtype, device=x.device)
+    ops.paged_attention(qkv, self.nq, self.nkv, self.d, out, cache.k, cache.v, ctx.block_tables[cache.group],
+                        ctx.token_req, ctx.cu_q, ctx.kv_len, self.scale, self.window or 0)
+    return linear(out, self.o_weight)
+
+
+register_mixer("paged_attention", PagedAttention)

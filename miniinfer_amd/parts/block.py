@@ -1,0 +1,42 @@
+"""Arrangement of a mixer and a feed-forward on the residual stream.
+
+"prenorm": x = norm1(r += h_in); a = mixer(x); x = norm2(r += a); h_out = ff(x).
+The add of a branch's output is deferred into the next norm, as the reference defers it
+(miniinfer/models/fused_qwen3.py:176-196); the residual stream `r` itself is kept in 32-bit.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Tuple
+
+import torch
+
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, register_block
+
+
+class PreNormBlock(Part):
+  def __init__(self, spec, ctx: BuildContext):
+    self.spec = spec
+    self.mixer_norm = NORMS.build(spec.mixer_norm, ctx)
+    self.mixer = MIXERS.build(spec.mixer, ctx)
+    self.ff_norm = NORMS.build(spec.feed_forward_norm, ctx)
+    self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, ctx)
+
+  def children(self) -> List[Tuple[str, Part]]:
+    n1, mx, n2, ff = self.spec.part_prefixes
+    return [(n1, self.mixer_norm), (mx, self.mixer), (n2, self.ff_norm), (ff, self.feed_forward)]
+
+  def cache_requirement(self):
+    fn = getattr(self.mixer, "cache_requirement", None)
+    return fn() if fn else None
+
+  def forward(self, h: Optional[torch.Tensor], residual: torch.Tensor, ctx, cache) -> torch.Tensor:
+    """h: the previous block's pending output (None for the first block); residual [T, hidden] float32,
+    updated in place.  Returns this block's pending output."""
+    x = self.mixer_norm.forward_residual(h, residual)
+    a = self.mixer.forward(x, ctx, cache)
+    x = self.ff_norm.forward_residual(a, residual)
+    return self.feed_forward.forward(x, ctx)
+
+
+register_block("prenorm", PreNormBlock)

@@ -1,0 +1,40 @@
+"""Dense gated feed-forward: down( silu(x Wg^T) * (x Wu^T) ) with gate and up fused into one matrix,
+gate rows first (miniinfer/models/fused_qwen3.py:111-138; miniinfer/loader/weight.py:87-93)."""
+
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import BuildContext, ParamSpec, Part, Source, register_feed_forward
+from .linear import linear
+
+
+class GatedMLP(Part):
+  def __init__(self, spec, ctx: BuildContext):
+    if spec.activation != "silu":
+      raise ValueError(f"activation {spec.activation!r} is not supported, only 'silu'")
+    self.spec = spec
+    self.hidden = spec.hidden_size
+    self.inter = spec.intermediate_size
+    self.gate_up_weight: Optional[torch.Tensor] = None
+    self.down_weight: Optional[torch.Tensor] = None
+
+  def param_specs(self) -> List[ParamSpec]:
+    g, u, d = self.spec.tensor_names
+    return [
+      ParamSpec("gate_up_weight", (2 * self.inter, self.hidden),
+                (Source(g + ".weight", self.inter), Source(u + ".weight", self.inter))),
+      ParamSpec("down_weight", (self.hidden, self.inter), (Source(d + ".weight", self.hidden),)),
+    ]
+
+  def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    gu = linear(x, self.gate_up_weight)
+    act = torch.empty((x.shape[0], self.inter), dtype=x.dtype, device=x.device)
+    ops.silu_mul(gu, act)
+    return linear(act, self.down_weight)
+
+
+register_feed_forward("gated_mlp", GatedMLP)

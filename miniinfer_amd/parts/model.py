@@ -1,0 +1,74 @@
+"""A decoder model assembled from a `ModelSpec`: embedding, blocks run in `run_order`, final norm,
+output head.  Nothing here names an architecture.
+
+Flow of one step (miniinfer/models/fused_qwen3.py:242-259,317-344): gather the embedding rows of
+the step's tokens into the 32-bit residual stream; run the blocks; add the last pending output,
+keep only the rows whose logits are wanted, norm them; logits = rows @ head^T in 32-bit.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Tuple
+
+import torch
+
+from ..config.spec import ModelSpec
+from ..kernels import ops
+from .base import BLOCKS, NORMS, BuildContext, ParamSpec, Part, Source
+from .linear import linear
+
+
+class DecoderModel(Part):
+  def __init__(self, spec: ModelSpec, ctx: BuildContext):
+    self.spec = spec
+    self.ctx = ctx
+    self.blocks = [BLOCKS.build(ls, ctx) for ls in spec.layers]
+    for i in spec.run_order:
+      if not 0 <= i < len(self.blocks):
+        raise ValueError(f"run_order names layer {i}, the model has {len(self.blocks)}")
+    self.final_norm = NORMS.build(spec.final_norm, ctx)
+    self.embedding: Optional[torch.Tensor] = None
+    self.head: Optional[torch.Tensor] = None
+
+  # ------------------------------------------------------------------ tensors
+  def param_specs(self) -> List[ParamSpec]:
+    V, H = self.spec.vocab_size, self.spec.hidden_size
+    return [ParamSpec("embedding", (V, H), (Source(self.spec.embedding_name, V),)),
+            ParamSpec("head", (V, H), (Source(self.spec.head_name, V),))]
+
+  def children(self) -> List[Tuple[str, Part]]:
+    out = [(ls.prefix, b) for ls, b in zip(self.spec.layers, self.blocks)]
+    out.append((self.spec.final_norm_prefix, self.final_norm))
+    return out
+
+  def cache_needs(self) -> List[object]:
+    """Per layer: what its mixer keeps between steps; a layer that borrows another's cache keeps nothing."""
+    needs = []
+    for ls, b in zip(self.spec.layers, self.blocks):
+      needs.append(None if ls.cache_of is not None else b.cache_requirement())
+    for i, ls in enumerate(self.spec.layers):
+      if ls.cache_of is not None:
+        if not 0 <= ls.cache_of < len(self.blocks) or self.spec.layers[ls.cache_of].cache_of is not None:
+          raise ValueError(f"layer {i} borrows the cache of layer {ls.cache_of}, which has none of its own")
+        if self.blocks[ls.cache_of].cache_requirement() != self.blocks[i].cache_requirement():
+          raise ValueError(f"layer {i} borrows the cache of layer {ls.cache_of}, whose geometry differs")
+    return needs
+
+  def cache_layer_of(self, layer: int) -> int:
+    co = self.spec.layers[layer].cache_of
+    return layer if co is None else co
+
+  # ------------------------------------------------------------------ one step
+  def forward(self, ctx) -> torch.Tensor:
+    """ctx: StepContext.  Returns float32 logits [len(ctx.logit_rows), vocab]."""
+    T, H = ctx.num_tokens, self.spec.hidden_size
+    residual = torch.empty((T, H), dtype=torch.float32, device=self.ctx.device)
+    ops.embed(self.embedding, ctx.token_ids, residual)
+    h = None
+    for li in self.spec.run_order:
+      h = self.blocks[li].forward(h, residual, ctx, ctx.layer_cache(self.cache_layer_of(li)))
+    R = ctx.num_logit_rows
+    if R == 0:
+      return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.ctx.device)
+    x = self.final_norm.forward_residual(h, residual, rows=ctx.logit_rows)
+    return linear(x, self.head if self.head is not None else self.embedding, out_dtype=torch.float32)

@@ -1,0 +1,218 @@
+"""Each HIP kernel alone against a plain torch statement of the same operation, at sizes other than
+the engine tests use (odd widths, vocabularies and head counts that are no power of two)."""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype):
+  return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,T", [(500, 80, 7), (1000, 1024, 33), (37, 3, 1)])
+def test_embed(dtype, V, H, T):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(0)
+  table = torch.randn(V, H, generator=g).to(dtype).to(DEV)
+  ids = torch.randint(0, V, (T,), generator=g).to(torch.int32).to(DEV)
+  out = torch.empty(T, H, dtype=torch.float32, device=DEV)
+  ops.embed(table, ids, out)
+  assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N", [(5, 80), (3, 1024), (17, 111), (2, 5120), (4, 7)])
+def test_add_rmsnorm(dtype, M, N):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(1)
+  x = (torch.randn(M, N, generator=g) * 3).to(dtype).to(DEV)
+  r = (torch.randn(M, N, generator=g) * 3).to(DEV)
+  w = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+  eps = 1e-5
+  want_r = r + x.float()
+  want = torch.nn.functional.rms_norm(want_r, (N,), w, eps)
+  out = torch.empty(M, N, dtype=dtype, device=DEV)
+  r2 = r.clone()
+  ops.add_rmsnorm(x, r2, w, eps, out, write_back=True)
+  torch.testing.assert_close(r2, want_r, rtol=1e-6, atol=1e-6)
+  torch.testing.assert_close(out.float(), want, **_tol(dtype))
+  # plain norm of x alone, the reference's own check (tests/unittests/test_norm_mlp.py:13-25)
+  out2 = torch.empty(M, N, dtype=dtype, device=DEV)
+  ops.add_rmsnorm(x, None, w, eps, out2)
+  torch.testing.assert_close(out2.float(), torch.nn.functional.rms_norm(x.float(), (N,), w, eps), **_tol(dtype))
+  # selected rows, residual untouched
+  rows = torch.tensor([M - 1, 0], dtype=torch.int32, device=DEV)
+  out3 = torch.empty(2, N, dtype=dtype, device=DEV)
+  r3 = r.clone()
+  ops.add_rmsnorm(x, r3, w, eps, out3, rows=rows)
+  assert torch.equal(r3, r)
+  torch.testing.assert_close(out3.float(), want[rows.long()], **_tol(dtype))
+
+
+def test_rmsnorm_large_values_do_not_overflow():
+  """bfloat16 inputs of magnitude 1e3 (the reference checks fp16 this way: tests/unittests/test_norm_mlp.py:30-43)."""
+  from miniinfer_amd.kernels import ops
+  x = (torch.randn(4, 256) * 1000).to(torch.bfloat16).to(DEV)
+  w = torch.ones(256, device=DEV)
+  out = torch.empty_like(x)
+  ops.add_rmsnorm(x, None, w, 1e-6, out)
+  rms = out.float().pow(2).mean(-1).sqrt()
+  torch.testing.assert_close(rms, torch.ones_like(rms), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I", [(3, 112), (9, 3072), (1, 5)])
+def test_silu_mul(dtype, M, I):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(2)
+  gu = (torch.randn(M, 2 * I, generator=g) * 2).to(dtype).to(DEV)
+  out = torch.empty(M, I, dtype=dtype, device=DEV)
+  ops.silu_mul(gu, out)
+  want = torch.nn.functional.silu(gu.float()[:, :I]) * gu.float()[:, I:]
+  torch.testing.assert_close(out.float(), want, **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 500, 80), (7, 130, 96), (65, 64, 17), (33, 1000, 1024), (128, 257, 300)])
+def test_gemm_nt(dtype, M, N, K):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(3)
+  a = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+  w = torch.randn(N, K, generator=g).to(dtype).to(DEV)
+  want = a.double() @ w.double().T
+  out32 = torch.empty(M, N, dtype=torch.float32, device=DEV)
+  ops.gemm_nt(a, w, out32)
+  torch.testing.assert_close(out32.double(), want, rtol=1e-5, atol=1e-4)
+  out = torch.empty(M, N, dtype=dtype, device=DEV)
+  ops.gemm_nt(a, w, out)
+  torch.testing.assert_close(out.double(), want, rtol=1e-5 if dtype == torch.float32 else 1e-2,
+                             atol=1e-4 if dtype == torch.float32 else 1e-1)
+
+
+def _rope_ref(x, pos, theta, rotary_dim):
+  """Complex multiplication by e^{i pos theta^(-2j/rd)} on pairs (j, j + rd/2): the statement of the
+  reference's test helper (tests/utils.py:12-17,65-116)."""
+  j = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
+  ang = pos.float()[:, None] * (1.0 / theta ** (j / rotary_dim))[None, :]
+  cis = torch.polar(torch.ones_like(ang), ang)[:, None, :]
+  half = rotary_dim // 2
+  z = torch.complex(x[..., :half], x[..., half:rotary_dim]) * cis
+  return torch.cat((z.real, z.imag, x[..., rotary_dim:]), dim=-1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,rd,P", [(6, 3, 48, 48, 16), (4, 4, 128, 128, 8), (5, 1, 16, 16, 4), (2, 2, 80, 32, 16)])
+def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(4)
+  T, pages, max_pos, theta, eps = 11, 9, 300, 12345.0, 1e-5
+  qkv = torch.randn(T, (nq + 2 * nkv) * d, generator=g).to(dtype)
+  qw = 1 + 0.1 * torch.randn(d, generator=g)
+  kw = 1 + 0.1 * torch.randn(d, generator=g)
+  pos = torch.randint(0, max_pos, (T,), generator=g)
+  slots = torch.randperm(pages * P, generator=g)[:T] + P   # never page 0
+  j = torch.arange(0, rd, 2, dtype=torch.float32)
+  ang = torch.outer(torch.arange(max_pos, dtype=torch.float32), 1.0 / theta ** (j / rd))
+  table = torch.cat((ang.cos(), ang.sin()), -1)
+
+  x = qkv.float().view(T, nq + 2 * nkv, d)
+  q, k, v = x[:, :nq], x[:, nq:nq + nkv], x[:, nq + nkv:]
+  qn = torch.nn.functional.rms_norm(q, (d,), qw, eps)
+  kn = torch.nn.functional.rms_norm(k, (d,), kw, eps)
+  q_want, k_want = _rope_ref(qn, pos, theta, rd), _rope_ref(kn, pos, theta, rd)
+
+  dq = qkv.to(DEV)
+  kp = torch.zeros(pages + 1, nkv, P, d, dtype=dtype, device=DEV)
+  vp = torch.zeros_like(kp)
+  ops.qk_norm_rope_cache(dq, nq, nkv, d, qw.to(DEV), kw.to(DEV), eps, table.to(DEV), pos.to(torch.int32).to(DEV),
+                         kp, vp, slots.to(torch.int32).to(DEV), P)
+  got = dq.float().cpu().view(T, nq + 2 * nkv, d)
+  torch.testing.assert_close(got[:, :nq], q_want, **_tol(dtype))
+  torch.testing.assert_close(got[:, nq:nq + nkv], k_want, **_tol(dtype))
+  assert torch.equal(got[:, nq + nkv:], v)
+  kc, vc = kp.float().cpu(), vp.float().cpu()
+  for t in range(T):
+    page, off = int(slots[t]) // P, int(slots[t]) % P
+    assert torch.equal(kc[page, :, off], got[t, nq:nq + nkv])
+    assert torch.equal(vc[page, :, off], v[t])
+  # nothing else was written
+  assert int((kc.abs().sum(-1) > 0).sum()) == T * nkv
+
+
+def _attention_ref(q, k, v, scale, window):
+  """q [L, nq, d], k, v [S, nkv, d]; bottom-right aligned causal mask; float64."""
+  L, nq, d = q.shape
+  S, nkv, _ = k.shape
+  rep = nq // nkv
+  kk = k.repeat_interleave(rep, dim=1).double()
+  vv = v.repeat_interleave(rep, dim=1).double()
+  s = torch.einsum("lhd,shd->hls", q.double(), kk) * scale
+  i = torch.arange(L)[:, None] + (S - L)
+  jj = torch.arange(S)[None, :]
+  mask = jj > i
+  if window:
+    mask = mask | (jj <= i - window)
+  s = s.masked_fill(mask[None], -math.inf)
+  return torch.einsum("hls,shd->lhd", torch.softmax(s, -1), vv)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P,window", [(6, 3, 48, 16, 0), (8, 2, 128, 8, 0), (4, 4, 16, 4, 0), (5, 1, 80, 32, 0),
+                                               (4, 2, 64, 16, 37), (16, 8, 256, 16, 0)])
+def test_paged_attention(dtype, nq, nkv, d, P, window):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(5)
+  # requests: (keys already cached, new tokens)
+  reqs = [(0, 70), (129, 1), (40, 3), (0, 1), (63, 2), (200, 1)]
+  B = len(reqs)
+  kv_lens = [a + n for a, n in reqs]
+  T = sum(n for _, n in reqs)
+  W = max(-(-kv // P) for kv in kv_lens)
+  n_pages = sum(-(-kv // P) for kv in kv_lens)
+  perm = (torch.randperm(n_pages, generator=g) + 1).tolist()
+  kp = torch.randn(n_pages + 1, nkv, P, d, generator=g).to(dtype)
+  vp = torch.randn(n_pages + 1, nkv, P, d, generator=g).to(dtype)
+  q = torch.randn(T, nq * d, generator=g).to(dtype)
+  table = torch.zeros(B, W, dtype=torch.int32)
+  cu = [0]
+  token_req = []
+  want = []
+  for b, (past, n) in enumerate(reqs):
+    npg = -(-kv_lens[b] // P)
+    pages = [perm.pop() for _ in range(npg)]
+    table[b, :npg] = torch.tensor(pages, dtype=torch.int32)
+    kk = torch.cat([kp[p].transpose(0, 1) for p in pages], 0)[:kv_lens[b]]   # [S, nkv, d]
+    vv = torch.cat([vp[p].transpose(0, 1) for p in pages], 0)[:kv_lens[b]]
+    qq = q[cu[-1]:cu[-1] + n].view(n, nq, d)
+    want.append(_attention_ref(qq.float(), kk.float(), vv.float(), d ** -0.5, window).reshape(n, nq * d))
+    token_req += [b] * n
+    cu.append(cu[-1] + n)
+  want = torch.cat(want, 0)
+  out = torch.empty(T, nq * d, dtype=dtype, device=DEV)
+  i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+  ops.paged_attention(q.to(DEV), nq, nkv, d, out, kp.to(DEV), vp.to(DEV), table.to(DEV), i32(token_req), i32(cu),
+                      i32(kv_lens), d ** -0.5, window)
+  torch.testing.assert_close(out.double().cpu(), want, **(_tol(dtype) if dtype == torch.bfloat16
+                                                           else dict(rtol=1e-5, atol=1e-5)))
+
+
+def test_attention_one_key_returns_its_value():
+  """A single visible key: softmax is 1 and the output is that key's value row, for every head of its group."""
+  from miniinfer_amd.kernels import ops
+  nq, nkv, d, P = 4, 2, 32, 8
+  kp = torch.randn(3, nkv, P, d, device=DEV)
+  vp = torch.randn(3, nkv, P, d, device=DEV)
+  q = torch.randn(1, nq * d, device=DEV)
+  out = torch.empty(1, nq * d, device=DEV)
+  i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+  ops.paged_attention(q, nq, nkv, d, out, kp, vp, i32([[2]]), i32([0]), i32([0, 1]), i32([1]), d ** -0.5, 0)
+  for h in range(nq):
+    torch.testing.assert_close(out[0, h * d:(h + 1) * d], vp[2, h // 2, 0])

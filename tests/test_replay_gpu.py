@@ -1,0 +1,151 @@
+"""The engine against the plain implementation, under every way of cutting the work.
+
+The same requests are replayed whole; with the last 32 tokens decoded one by one; in portions of
+changing size down to two tokens; and mixed, up to four live requests with portions of some beside
+decoded tokens of others and so few pages that they are used again.  In 32-bit the logits must
+agree with the plain implementation to 1e-4; in bfloat16 to the rounding of bfloat16 activations.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import tiny_models as tm
+import trace_tools as tt
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [5, 17, 33, 100, 128, 64], "B": [1, 9, 40, 64, 100, 200, 33], "C": [300, 77, 513, 2, 150]}
+FP32_TOL = 1e-4
+
+
+def _requests(name, cfg):
+  return {f"r{i}": tm.random_tokens(cfg, n, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
+
+
+def _plain_logits(cfg_dict, weights, requests):
+  pc = dict(cfg_dict)
+  w = {k: v.float() for k, v in weights.items()}
+  return {rid: plain.qwen3_logits(toks, w, pc).numpy() for rid, toks in requests.items()}
+
+
+def _replay(folder, dtype, steps, requests, page_size, max_tokens):
+  from miniinfer_amd.engine.replay import Replayer
+  rp = Replayer(str(folder), dtype, max_tokens, page_size=page_size)
+  outs = []
+  for st in steps:
+    outs.append(rp.step(st))
+    rp.cache.check()
+  assert rp.cache.num_free_pages() == rp.cache.num_pages, "pages were not all given back"
+  assert not rp.cache.live_requests()
+  return outs
+
+
+def _bf16_check(got, want, what):
+  scale = np.abs(want).max()
+  err = np.abs(got - want)
+  assert err.max() <= 0.04 * scale, f"{what}: max err {err.max():.4g} vs scale {scale:.4g}"
+  assert err.mean() <= 0.006 * scale, f"{what}: mean err {err.mean():.4g} vs scale {scale:.4g}"
+  # the top token agrees wherever the plain margin is clear
+  top = want.argmax(-1)
+  srt = np.sort(want, -1)
+  clear = (srt[:, -1] - srt[:, -2]) > 0.08 * scale
+  assert (got.argmax(-1)[clear] == top[clear]).all(), f"{what}: top token differs at a clear margin"
+
+
+REGIMES = {
+  "whole": lambda r: tt.whole(r),
+  "tail_decoded": lambda r: tt.tail_decoded(r, 32),
+  "portions": lambda r: tt.portions(r),
+  "mixed": lambda r: tt.mixed(r, max_live=4, seed=3),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("regime", list(REGIMES))
+def test_regime(tmp_path, name, dtype, regime):
+  file_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
+  cfg, w = tm.make_model(str(tmp_path / "m"), name, seed=7, dtype=file_dtype, std=0.05)
+  requests = _requests(name, cfg)
+  want = _plain_logits(cfg, w, requests)
+  steps = REGIMES[regime](requests)
+  max_tokens = tt.peak_tokens(steps, requests)
+  print(f"config {name} {dtype} {regime}: {len(steps)} steps, pool for {max_tokens} tokens", flush=True)
+  outs = _replay(tmp_path / "m", dtype, steps, requests, tm.PAGE_SIZE[name], max_tokens)
+  got = tt.gather(steps, outs, requests, cfg["vocab_size"])
+  for rid in requests:
+    assert not np.isnan(got[rid]).any()
+    if dtype == "float32":
+      err = np.abs(got[rid] - want[rid]).max()
+      assert err <= FP32_TOL, f"{name} {regime} request {rid}: max abs err {err:.3g}"
+    else:
+      _bf16_check(got[rid], want[rid], f"{name} {regime} request {rid}")
+
+
+def test_first_tokens_and_single_token_prompt(tmp_path):
+  """The first tokens of a sequence: position 0 sees one key; a one-token prompt; a two-token portion first."""
+  cfg, w = tm.make_model(str(tmp_path / "m"), "B", seed=11, dtype=torch.float32, std=0.05)
+  requests = {"a": tm.random_tokens(cfg, 1, 1), "b": tm.random_tokens(cfg, 2, 2), "c": tm.random_tokens(cfg, 3, 3)}
+  want = _plain_logits(cfg, w, requests)
+  steps = [{"step": 0, "entries": [{"id": r, "tokens": t, "want": list(range(len(t)))} for r, t in requests.items()],
+            "end": list(requests)}]
+  outs = _replay(tmp_path / "m", "float32", steps, requests, 8, 256)
+  got = tt.gather(steps, outs, requests, cfg["vocab_size"])
+  for rid in requests:
+    assert np.abs(got[rid] - want[rid]).max() <= FP32_TOL
+
+
+def test_long_decoding(tmp_path):
+  """A short prompt and then hundreds of single-token steps, across many page edges."""
+  cfg, w = tm.make_model(str(tmp_path / "m"), "C", seed=5, dtype=torch.float32, std=0.05)
+  toks = tm.random_tokens(cfg, 700, 9)
+  requests = {"long": toks}
+  want = _plain_logits(cfg, w, requests)
+  steps = tt.tail_decoded(requests, tail=690)
+  outs = _replay(tmp_path / "m", "float32", steps, requests, 16, 704)
+  got = tt.gather(steps, outs, requests, cfg["vocab_size"])
+  assert np.abs(got["long"] - want["long"]).max() <= FP32_TOL
+
+
+def test_wanted_rows_only(tmp_path):
+  """`want` picks places; an empty `want` writes nothing; the rest of the step is unchanged."""
+  cfg, w = tm.make_model(str(tmp_path / "m"), "A", seed=2, dtype=torch.float32, std=0.05)
+  toks = tm.random_tokens(cfg, 40, 4)
+  want = _plain_logits(cfg, w, {"a": toks})["a"]
+  from miniinfer_amd.engine.replay import Replayer
+  rp = Replayer(str(tmp_path / "m"), "float32", 64, page_size=16)
+  assert rp.step({"step": 0, "entries": [{"id": "a", "tokens": toks[:10], "want": []}], "end": []}) is None
+  out = rp.step({"step": 1, "entries": [{"id": "a", "tokens": toks[10:40], "want": [29, 0, 7]}], "end": ["a"]})
+  assert out.shape == (3, cfg["vocab_size"])
+  for r, p in enumerate([39, 10, 17]):
+    assert np.abs(out[r] - want[p]).max() <= FP32_TOL
+
+
+def test_trace_run_program(tmp_path):
+  """bin/trace_run as a user calls it: JSON lines on stdin, <step>.f32 files, `done <step>` lines."""
+  import json
+  import os
+  import subprocess
+  import sys
+  cfg, w = tm.make_model(str(tmp_path / "m"), "A", seed=3, dtype=torch.float32, std=0.05)
+  requests = {"x": tm.random_tokens(cfg, 50, 1), "y": tm.random_tokens(cfg, 21, 2)}
+  want = _plain_logits(cfg, w, requests)
+  steps = tt.mixed(requests, max_live=2, seed=1)
+  root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+  inp = "".join(json.dumps(s) + "\n" for s in steps)
+  out_dir = tmp_path / "out"
+  proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(tmp_path / "m"),
+                         "--dtype", "float32", "--out", str(out_dir), "--max-tokens", "128"],
+                        input=inp, capture_output=True, text=True, timeout=300)
+  assert proc.returncode == 0, proc.stderr[-2000:]
+  assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+  outs = []
+  for s in steps:
+    n = sum(len(e["want"]) for e in s["entries"])
+    arr = np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4").reshape(n, cfg["vocab_size"]) if n else None
+    outs.append(arr)
+  got = tt.gather(steps, outs, requests, cfg["vocab_size"])
+  for rid in requests:
+    assert np.abs(got[rid] - want[rid]).max() <= FP32_TOL
