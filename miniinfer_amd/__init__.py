@@ -1,3 +1,17 @@
-"""miniinfer_amd: a small, whole inference engine for one MI355X (gfx950)."""
+"""miniinfer_amd: a small, whole inference engine for one MI355X (gfx950).
+
+    from miniinfer_amd import LLMEngine, SamplingParams
+"""
 
 __version__ = "0.1.0"
+
+from .config import EngineConfig
+from .sampling import SamplingParams
+
+
+def __getattr__(name):
+  # the engine pulls in the kernels; keep `import miniinfer_amd` light
+  if name == "LLMEngine":
+    from .engine import LLMEngine
+    return LLMEngine
+  raise AttributeError(name)

@@ -217,10 +217,17 @@ class CacheManager:
     lo = max(0, next_pos - g.need.window + 1)
     return lo // self.page_size
 
+  def held_pages(self, req) -> int:
+    """Page indices `req` has been given so far (0 for a request that is not admitted)."""
+    if not self.paged or req not in self.paged[0].tables:
+      return 0
+    return len(self.paged[0].tables[req])
+
   def pages_needed(self, req, new_len: int) -> int:
-    """Pages the tightest group must still hand out so that `req` can hold new_len tokens."""
-    have = len(self.paged[0].tables[req]) if self.paged else 0
-    return max(0, -(-new_len // self.page_size) - have)
+    """Pages each group must still hand out so that `req` can hold new_len tokens."""
+    if not self.paged:
+      return 0
+    return max(0, -(-new_len // self.page_size) - self.held_pages(req))
 
   def can_grow(self, req, new_len: int) -> bool:
     return self.pages_needed(req, new_len) <= self.num_free_pages()

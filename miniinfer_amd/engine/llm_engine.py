@@ -1,0 +1,208 @@
+"""The Python entry point, in the manner of the reference's `LLMEngine`
+(miniinfer/engine/llm_engine.py:87-141 constructor, :898-1015 generate, :465-557 step, :1309 add_request,
+:1271 is_finished, :1301-1306 context manager; examples/minimal_engine.py:60-90).
+
+    with LLMEngine(model="/path/to/folder", max_num_seqs=4, max_model_len=512) as engine:
+      outs = engine.generate(prompts, SamplingParams(temperature=0.7, max_tokens=64))
+      outs[0]["token_ids"], outs[0]["text"]
+
+Prompts are lists of token ids (always) or strings (when the model folder holds a tokenizer.json).
+One synchronous loop: schedule, step, sample, update; no processes, no server.
+"""
+
+from __future__ import annotations
+
+import os
+import sys
+import time
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..config import EngineConfig, load_model_config, model_spec_of
+from ..sampling import Sampler, SamplingParams, request_seed
+from ..weights import build_model, fill_random, load_weights
+from .runner import ModelRunner, StepEntry
+from .scheduler import Request, ScheduledStep, Scheduler
+
+TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+@dataclass
+class StepOutput:
+  """What one engine step did (miniinfer/engine/llm_engine.py:62-75)."""
+  finished: List[Request] = field(default_factory=list)
+  num_prefill_tokens: int = 0
+  num_decode_tokens: int = 0
+  num_preempted: int = 0
+
+
+class LLMEngine:
+  def __init__(self, model: str, model_config=None, random_weights_seed: Optional[int] = None, **kwargs):
+    """model: a folder with config.json and *.safetensors.  With `model_config` (a typed configuration)
+    and `random_weights_seed`, no folder is read and the weights are drawn on the device."""
+    kwargs.pop("use_multiprocess", None)   # the reference's examples pass it; there is one process here
+    self.config = EngineConfig.from_kwargs(model, **kwargs)
+    if not torch.cuda.is_available():
+      raise RuntimeError("miniinfer_amd needs a GPU: torch.cuda.is_available() is False and there is no CPU path")
+    cfg = self.config
+    self.dtype = TORCH_DTYPES[cfg.dtype]
+    self.device = torch.device(cfg.device)
+    torch.cuda.set_device(self.device)
+    self.model_config = model_config if model_config is not None else load_model_config(cfg.model_path)
+    self.model = build_model(model_spec_of(self.model_config), self.dtype, self.device)
+    if random_weights_seed is not None:
+      fill_random(self.model, random_weights_seed)
+    else:
+      load_weights(self.model, cfg.model_path)
+    spec = self.model.spec
+    self.max_model_len = min(cfg.max_model_len or spec.max_positions, spec.max_positions)
+    needs = self.model.cache_needs()
+    self.num_pages = cfg.num_pages if cfg.num_pages is not None else self._pages_from_memory(needs)
+    self.cache = CacheManager(needs, page_size=cfg.page_size, num_pages=self.num_pages, max_requests=cfg.max_num_seqs,
+                              max_model_len=self.max_model_len, dtype=self.dtype, device=self.device)
+    self.runner = ModelRunner(self.model, self.cache)
+    eos = cfg.eos if cfg.eos is not None else getattr(self.model_config, "eos_token_id", None)
+    self.eos_token_id = eos
+    self.scheduler = Scheduler(self.cache, max_num_seqs=cfg.max_num_seqs,
+                               max_num_batched_tokens=cfg.max_num_batched_tokens, max_model_len=self.max_model_len,
+                               enable_chunked_prefill=cfg.enable_chunked_prefill, eos_token_id=eos)
+    self.sampler = Sampler(self.device)
+    self.tokenizer = self._load_tokenizer(cfg.model_path)
+    self._next_number = 0
+    self._requests: Dict[str, Request] = {}
+    self.num_steps = 0
+
+  # ------------------------------------------------------------------ set-up helpers
+  def _pages_from_memory(self, needs) -> int:
+    """Pages from the device memory left after the weights (the reference: utils/memory_utils.py:85-144,
+    which also holds a share back for activations)."""
+    cfg = self.config
+    per_page = CacheManager.bytes_per_page(needs, cfg.page_size, self.dtype)
+    cap = cfg.max_num_seqs * (-(-self.max_model_len // cfg.page_size))
+    if per_page == 0:
+      return max(1, cap)
+    free, total = torch.cuda.mem_get_info(self.device)
+    usable = free - int(total * (1.0 - cfg.gpu_memory_utilization))
+    usable = int(usable * 0.8)
+    pages = usable // per_page - 1
+    if pages < 2:
+      raise RuntimeError(f"not enough device memory for a cache: {free >> 20} MiB free, a page costs {per_page} bytes")
+    return int(min(pages, cap))
+
+  @staticmethod
+  def _load_tokenizer(path: str):
+    tj = os.path.join(path, "tokenizer.json") if path and os.path.isdir(path) else None
+    if tj and os.path.isfile(tj):
+      try:
+        from tokenizers import Tokenizer
+        return Tokenizer.from_file(tj)
+      except Exception:
+        return None
+    return None
+
+  # ------------------------------------------------------------------ context manager (llm_engine.py:1301-1306)
+  def __enter__(self):
+    return self
+
+  def __exit__(self, *exc):
+    self.stop()
+    return False
+
+  def start(self):
+    return self
+
+  def stop(self):
+    pass
+
+  # ------------------------------------------------------------------ requests
+  def _encode(self, prompt) -> List[int]:
+    if isinstance(prompt, str):
+      if self.tokenizer is None:
+        raise ValueError("a text prompt needs a tokenizer.json in the model folder; pass token ids instead")
+      return list(self.tokenizer.encode(prompt).ids)
+    return [int(t) for t in prompt]
+
+  def add_request(self, prompt: Union[str, Sequence[int]], sampling_params: Optional[SamplingParams] = None,
+                  request_id: Optional[str] = None) -> str:
+    params = sampling_params or SamplingParams()
+    ids = self._encode(prompt)
+    V = self.model.spec.vocab_size
+    if any(t < 0 or t >= V for t in ids):
+      raise ValueError(f"prompt holds a token id outside [0, {V})")
+    number = self._next_number
+    self._next_number += 1
+    rid = request_id or f"req-{number}"
+    req = Request(number=number, request_id=rid, prompt=ids, params=params,
+                  seed=request_seed(self.config.seed, number, params.seed))
+    self.scheduler.add(req)
+    self._requests[rid] = req
+    return rid
+
+  def is_finished(self) -> bool:
+    return not self.scheduler.has_unfinished()
+
+  has_unfinished = property(lambda self: self.scheduler.has_unfinished())
+
+  # ------------------------------------------------------------------ one step
+  def step(self) -> StepOutput:
+    """schedule -> run the batch -> sample -> update (miniinfer/engine/llm_engine.py:465-557)."""
+    plan = self.scheduler.schedule()
+    out = StepOutput()
+    if plan is None:
+      return out
+    entries = []
+    sampling = []
+    for e in plan.entries:
+      toks = e.request.tokens[e.start:e.start + e.num_tokens]
+      entries.append(StepEntry(req=e.request.number, tokens=toks, want=[e.num_tokens - 1] if e.samples else []))
+      if e.samples:
+        sampling.append(e.request)
+    logits = self.runner.step(entries)
+    sampled: Dict[int, int] = {}
+    if sampling:
+      toks = self.sampler.sample(logits, [r.params for r in sampling], [r.seed for r in sampling],
+                                 [len(r.outputs) for r in sampling])
+      sampled = {r.number: t for r, t in zip(sampling, toks)}
+    out.finished = self.scheduler.update(plan, sampled)
+    out.num_prefill_tokens = plan.num_prefill_tokens
+    out.num_decode_tokens = plan.num_decode_tokens
+    out.num_preempted = len(plan.preempted)
+    self.num_steps += 1
+    return out
+
+  # ------------------------------------------------------------------ generate
+  def generate(self, prompts, sampling_params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+               use_tqdm: bool = True) -> List[dict]:
+    """prompts: a string, a list of strings, a list of token ids, or a list of such lists; sampling_params: one
+    for all or one per prompt.  Returns, in the order of the prompts, dicts with "text", "token_ids",
+    "request_id" (miniinfer/engine/llm_engine.py:898-1015) and "finish_reason"."""
+    if isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], int)):
+      prompts = [prompts]
+    if sampling_params is None:
+      sampling_params = SamplingParams()
+    if isinstance(sampling_params, SamplingParams):
+      sampling_params = [sampling_params] * len(prompts)
+    if len(sampling_params) != len(prompts):
+      raise ValueError("one SamplingParams for all prompts, or one per prompt")
+    rids = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+    t0 = time.time()
+    decoded = 0
+    last = t0
+    while not self.is_finished():
+      so = self.step()
+      decoded += so.num_decode_tokens
+      if use_tqdm and time.time() - last > 1.0:
+        last = time.time()
+        print(f"\r[miniinfer_amd] step {self.num_steps}: {decoded / (last - t0):.1f} decoded tok/s", end="",
+              file=sys.stderr, flush=True)
+    if use_tqdm:
+      print(file=sys.stderr)
+    results = []
+    for rid in rids:
+      r = self._requests.pop(rid)
+      text = self.tokenizer.decode(r.outputs) if self.tokenizer is not None else ""
+      results.append({"text": text, "token_ids": list(r.outputs), "request_id": rid, "finish_reason": r.finish_reason})
+    return results

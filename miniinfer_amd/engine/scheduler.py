@@ -1,0 +1,231 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token budget, decodes, finishes
+and frees.  Host-only; it talks to the cache manager through a handful of calls, so tests drive it
+with the real manager on the CPU.
+
+Policy (Sarathi-style, like the reference with `enable_chunked_prefill`,
+miniinfer/scheduler/scheduler.py:242-286,417-434): every step carries one token for each running
+request that is decoding, and the rest of the token budget is filled with prompt portions, first of
+requests already running, then of waiting requests in arrival order
+(miniinfer/scheduler/prefill_adder.py:39-421 plays this role there, with page-rounded chunks; here a
+portion is any length >= 1).
+
+When pages run out (the reference retracts from the tail of the running list and drops the generated
+tokens, scheduler.py:519-610): the most recently admitted running request is preempted: its pages
+and slot are given back and it returns to the head of the waiting queue, keeping its generated tokens;
+when it is admitted again it recomputes prompt + outputs as one prompt.  Admission of new requests
+stops while running requests cannot grow.  A request that could never fit the pool alone is refused
+when it is added.
+"""
+
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional, Sequence
+
+from ..sampling.params import SamplingParams
+
+
+@dataclass
+class Request:
+  number: int                     # arrival order; also the handle in the cache manager
+  request_id: str
+  prompt: List[int]
+  params: SamplingParams
+  seed: int = 0
+  outputs: List[int] = field(default_factory=list)
+  num_computed: int = 0           # tokens whose keys and values are in the cache
+  finish_reason: Optional[str] = None
+  num_preemptions: int = 0
+
+  @property
+  def tokens(self) -> List[int]:
+    return self.prompt + self.outputs
+
+  @property
+  def num_tokens(self) -> int:
+    return len(self.prompt) + len(self.outputs)
+
+  @property
+  def remaining(self) -> int:
+    return self.num_tokens - self.num_computed
+
+  @property
+  def finished(self) -> bool:
+    return self.finish_reason is not None
+
+
+@dataclass
+class ScheduledEntry:
+  request: Request
+  start: int                      # position of the first token of this portion
+  num_tokens: int
+  samples: bool                   # the portion ends the known tokens: its last logits pick the next token
+
+
+@dataclass
+class ScheduledStep:
+  entries: List[ScheduledEntry]
+  preempted: List[Request] = field(default_factory=list)
+
+  @property
+  def num_tokens(self) -> int:
+    return sum(e.num_tokens for e in self.entries)
+
+  @property
+  def num_decode_tokens(self) -> int:
+    return sum(1 for e in self.entries if e.num_tokens == 1 and e.start > 0)
+
+  @property
+  def num_prefill_tokens(self) -> int:
+    return self.num_tokens - self.num_decode_tokens
+
+
+class Scheduler:
+  def __init__(self, cache, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
+               enable_chunked_prefill: bool = True, eos_token_id: Optional[int] = None):
+    self.cache = cache
+    self.max_num_seqs = max_num_seqs
+    self.max_num_batched_tokens = max_num_batched_tokens
+    self.max_model_len = max_model_len
+    self.enable_chunked_prefill = enable_chunked_prefill
+    self.eos_token_id = eos_token_id
+    self.waiting: Deque[Request] = deque()
+    self.running: List[Request] = []      # in order of admission
+    self.finished: List[Request] = []
+    self.num_preemptions = 0
+
+  # ------------------------------------------------------------------ requests in
+  def add(self, req: Request) -> None:
+    n = len(req.prompt)
+    if n == 0:
+      raise ValueError("a request needs at least one prompt token")
+    if n + req.params.max_tokens > self.max_model_len:
+      # the reference never checks this and would index past its table (kvcache/memory_pool.py:476-478)
+      raise ValueError(f"prompt of {n} tokens plus max_tokens={req.params.max_tokens} exceeds "
+                       f"max_model_len={self.max_model_len}")
+    P = self.cache.page_size
+    if -(-(n + req.params.max_tokens) // P) > self.cache.num_pages:
+      raise ValueError(f"request of up to {n + req.params.max_tokens} tokens can never fit the cache of "
+                       f"{self.cache.num_pages} pages of {P} tokens")
+    if not self.enable_chunked_prefill and n + req.params.max_tokens > self.max_num_batched_tokens:
+      raise ValueError(f"without chunked prefill a request of up to {n + req.params.max_tokens} tokens must fit the "
+                       f"step budget of {self.max_num_batched_tokens}")
+    self.waiting.append(req)
+
+  def has_unfinished(self) -> bool:
+    return bool(self.waiting or self.running)
+
+  # ------------------------------------------------------------------ one step's plan
+  def _pages_for(self, req: Request, new_len: int) -> int:
+    return self.cache.pages_needed(req.number, new_len)
+
+  def _preempt(self, req: Request) -> None:
+    self.cache.release(req.number)
+    self.running.remove(req)
+    req.num_computed = 0
+    req.num_preemptions += 1
+    self.num_preemptions += 1
+    self.waiting.appendleft(req)
+
+  def schedule(self) -> Optional[ScheduledStep]:
+    if not self.has_unfinished():
+      return None
+    budget = self.max_num_batched_tokens
+    free = self.cache.num_free_pages()
+    entries: List[ScheduledEntry] = []
+    preempted: List[Request] = []
+
+    # 1. decodes: one token for every running request whose known tokens are all but one in the cache
+    decoding = [r for r in self.running if r.remaining == 1 and r.num_computed > 0]
+    while True:
+      need = sum(self._pages_for(r, r.num_tokens) for r in decoding)
+      if need <= free or not decoding:
+        break
+      victim = self.running[-1]
+      self._preempt(victim)
+      preempted.append(victim)
+      decoding = [r for r in decoding if r is not victim]
+      free = self.cache.num_free_pages()
+    for r in decoding[:budget]:
+      entries.append(ScheduledEntry(r, r.num_computed, 1, True))
+      free -= self._pages_for(r, r.num_tokens)
+      budget -= 1
+    scheduled = {id(e.request) for e in entries}
+
+    # 2. prompt portions of running requests (a preempted-and-readmitted request included)
+    for r in self.running:
+      if budget <= 0:
+        break
+      if id(r) in scheduled or r.remaining <= 0 or (r.remaining == 1 and r.num_computed > 0):
+        continue
+      n = self._portion(r, budget, free)
+      if n <= 0:
+        continue
+      entries.append(ScheduledEntry(r, r.num_computed, n, r.num_computed + n == r.num_tokens))
+      free -= self._pages_for(r, r.num_computed + n)
+      budget -= n
+
+    # 3. admissions, in arrival order; none while a request had to be preempted in this step
+    while self.waiting and budget > 0 and not preempted and len(self.running) < self.max_num_seqs \
+        and self.cache.num_free_slots() > 0:
+      r = self.waiting[0]
+      # watermark: its whole known sequence must fit, with one spare page for each request already running,
+      # so that an admission does not at once force a preemption
+      if self._pages_for(r, r.num_tokens) + len(self.running) > free:
+        break
+      n = self._portion(r, budget, free)
+      if n <= 0:
+        break
+      self.waiting.popleft()
+      self.cache.admit(r.number)
+      self.running.append(r)
+      entries.append(ScheduledEntry(r, 0, n, n == r.num_tokens))
+      free -= self._pages_for(r, n)
+      budget -= n
+
+    if not entries:
+      if self.running or self.waiting:
+        # nothing fits: every running request is stuck on pages and none can be preempted further
+        if len(self.running) > 1:
+          victim = self.running[-1]
+          self._preempt(victim)
+          return self.schedule()
+        raise RuntimeError("the scheduler cannot make progress: no request fits the cache")
+      return None
+    return ScheduledStep(entries, preempted)
+
+  def _portion(self, r: Request, budget: int, free_pages: int) -> int:
+    """How many of r's remaining tokens run in this step: bounded by the budget and by the tokens that fit
+    the pages r holds plus the free ones.  Without chunked prefill it is all of them or none."""
+    P = self.cache.page_size
+    capacity = (self.cache.held_pages(r.number) + free_pages) * P
+    n = min(r.remaining, budget, capacity - r.num_computed)
+    if not self.enable_chunked_prefill and n < r.remaining:
+      return 0
+    return max(n, 0)
+
+  # ------------------------------------------------------------------ results in
+  def update(self, step: ScheduledStep, sampled: Dict[int, int]) -> List[Request]:
+    """After the step ran: `sampled[request.number]` is the next token of every entry that samples.
+    Returns the requests that finished; their pages and slots are given back here."""
+    done = []
+    for e in step.entries:
+      r = e.request
+      r.num_computed += e.num_tokens
+      if not e.samples:
+        continue
+      tok = int(sampled[r.number])
+      r.outputs.append(tok)
+      if not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id:
+        r.finish_reason = "eos"
+      elif len(r.outputs) >= r.params.max_tokens:
+        r.finish_reason = "max_tokens"
+      elif r.num_tokens >= self.max_model_len:
+        r.finish_reason = "length"
+      if r.finished:
+        self.cache.release(r.number)
+        self.running.remove(r)
+        self.finished.append(r)
+        done.append(r)
+    return done

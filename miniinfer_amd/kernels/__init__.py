@@ -5,7 +5,7 @@ from typing import List
 from . import jit
 
 # every shared object of the library: (source name, defines)
-ALL_MODULES = [("elementwise", ()), ("gemm", ()), ("attention", ())]
+ALL_MODULES = [("elementwise", ()), ("gemm", ()), ("attention", ()), ("sampling", ())]
 
 
 def build_all(force: bool = False) -> List[str]:

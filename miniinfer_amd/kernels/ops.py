@@ -89,6 +89,10 @@ _SIGS = {
   },
 }
 
+_SIGS["sampling"] = {
+  "mi_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+}
+
 _libs = {}
 
 
@@ -269,4 +273,30 @@ def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tenso
                                      _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
                                      _ptr(token_req), _ptr(cu_q), _ptr(kv_len), T, B, nq, nkv, d,
                                      k_pages.shape[2], float(scale), int(window), _stream()))
+  return out
+
+
+# ----------------------------------------------------------------------------- sampling
+
+def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_k: Optional[torch.Tensor],
+           top_p: Optional[torch.Tensor], seeds: Optional[torch.Tensor], steps: Optional[torch.Tensor],
+           out: torch.Tensor) -> torch.Tensor:
+  """out[r] = next token of row r of float32 logits [R, V].  temperature[r] == 0 (or no temperatures) is
+  argmax with the lowest index winning ties; otherwise a draw from softmax(logits / temperature), limited to
+  the top_k[r] most probable tokens (0 = all) and then to the top_p[r] mass (1 = all), from the counter-based
+  generator keyed by (seeds[r], steps[r], token index)."""
+  _dev(logits, temperature, top_k, top_p, seeds, steps, out)
+  if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+    raise KernelError("sample: logits must be float32 [R, V] with dense rows")
+  R, V = logits.shape
+  _f32("temperature", temperature, R)
+  _i32("top_k", top_k, R)
+  _f32("top_p", top_p, R)
+  for name, t in (("seeds", seeds), ("steps", steps)):
+    if t is not None and (t.dtype != torch.int64 or t.numel() != R or not t.is_contiguous()):
+      raise KernelError(f"sample: {name} must be int64 [R]")
+  _i32("out", out, R)
+  lib = _lib("sampling")
+  _check(lib, lib.mi_sample(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature), _ptr(top_k),
+                            _ptr(top_p), _ptr(seeds), _ptr(steps), _ptr(out), _stream()))
   return out

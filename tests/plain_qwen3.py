@@ -197,8 +197,9 @@ def greedy_generate(prompt: List[int], n: int, w: Dict[str, torch.Tensor], cfg: 
 # ----------------------------------------------------------------------------
 
 def sampling_distribution(logits: torch.Tensor, temperature: float, top_k: int = 0, top_p: float = 1.0) -> torch.Tensor:
-  """The distribution a token is drawn from: softmax(logits / T), then keep the top_k most
-  probable (0 = all) and the smallest most-probable set whose mass reaches top_p, renormalised.
+  """The distribution a token is drawn from: softmax(logits / T); keep the top_k most probable
+  (0 = all) and renormalise; then keep the smallest most-probable set whose mass reaches top_p and
+  renormalise (top-k first, as the reference's fused call applies them).
   temperature 0 is argmax.  miniinfer/layers/sample.py:107-128; utils/sampling_params.py:5-23."""
   x = logits.to(torch.float64)
   V = x.numel()
@@ -207,14 +208,14 @@ def sampling_distribution(logits: torch.Tensor, temperature: float, top_k: int =
     p[int(torch.argmax(x))] = 1.0
     return p
   p = torch.softmax(x / temperature, dim=-1)
-  order = torch.argsort(p, descending=True, stable=True)
-  keep = torch.ones(V, dtype=torch.bool)
   if top_k and top_k < V:
-    keep[order[top_k:]] = False
+    kth = torch.sort(p, descending=True).values[top_k - 1]
+    p = torch.where(p >= kth, p, torch.zeros_like(p))
+    p = p / p.sum()
   if top_p < 1.0:
-    sp = p[order]
+    sp, order = torch.sort(p, descending=True, stable=True)
     before = torch.cumsum(sp, 0) - sp  # mass strictly ahead of each token
-    drop = before >= top_p
-    keep[order[drop]] = False
-  p = torch.where(keep, p, torch.zeros_like(p))
+    keep = torch.zeros(V, dtype=torch.bool)
+    keep[order[before < top_p]] = True
+    p = torch.where(keep, p, torch.zeros_like(p))
   return p / p.sum()

