@@ -1,0 +1,163 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X, Qwen3-0.6B shape, random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--preset qwen3-0.6b]
+
+A step is one decode step of the whole engine (schedule, batch building, model, sampling) with `batch`
+requests that each hold `context` tokens in the cache.  Prints ONE JSON line: decoded tokens a second, the
+2,048-token prefill, the decode step's HBM roofline, and decode at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+
+def model_numbers(cfg, layers):
+  H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+  nq, nkv, d = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+  per_layer = (nq + 2 * nkv) * d * H + nq * d * H + 3 * H * I
+  return dict(linear_params=per_layer * layers, head_params=V * H, kv_per_token=2 * layers * nkv * d)
+
+
+def decode_bytes(cfg, layers, batch, context, esize):
+  n = model_numbers(cfg, layers)
+  return (n["linear_params"] + n["head_params"]) * esize + batch * context * n["kv_per_token"] * esize
+
+
+def prefill_flops(cfg, layers, T):
+  n = model_numbers(cfg, layers)
+  attn = layers * 4 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) // 2)
+  return 2 * T * n["linear_params"] + attn + 2 * n["head_params"]
+
+
+def time_decode(engine, batch, context, steps, warmup, seed):
+  """`batch` requests with `context` random tokens each, prefilled through the engine; then `warmup` untimed and
+  `steps` timed decode steps.  Returns seconds per step."""
+  import torch
+  from random import Random
+  from miniinfer_amd import SamplingParams
+  rnd = Random(seed)
+  V = engine.model.spec.vocab_size
+  # requests whose prompts go first decode while the others are still prefilled: leave room for that
+  stagger = -(-batch * context // engine.config.max_num_batched_tokens) + 1
+  sp = SamplingParams(temperature=0.0, max_tokens=warmup + steps + stagger + 2, ignore_eos=True)
+  for _ in range(batch):
+    engine.add_request([rnd.randrange(V) for _ in range(context)], sp)
+  # prefill until every request is decoding
+  while any(r.remaining != 1 or r.num_computed == 0 for r in engine.scheduler.running) or engine.scheduler.waiting:
+    engine.step()
+  for _ in range(warmup):
+    engine.step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(steps):
+    so = engine.step()
+    assert so.num_decode_tokens == batch and so.num_prefill_tokens == 0
+  torch.cuda.synchronize()
+  dt = (time.perf_counter() - t0) / steps
+  while not engine.is_finished():
+    engine.step()
+  engine._requests.clear()
+  return dt
+
+
+def time_prefill(engine, T, reps, seed):
+  import torch
+  from random import Random
+  from miniinfer_amd import SamplingParams
+  rnd = Random(seed)
+  V = engine.model.spec.vocab_size
+  sp = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
+  times = []
+  for i in range(reps + 1):
+    engine.add_request([rnd.randrange(V) for _ in range(T)], sp)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    so = engine.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert so.num_prefill_tokens == T and len(so.finished) == 1
+    if i > 0:
+      times.append(dt)
+    engine._requests.clear()
+  return min(times)
+
+
+def main() -> int:
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=64)
+  ap.add_argument("--warmup", type=int, default=8)
+  ap.add_argument("--batch", type=int, default=8)
+  ap.add_argument("--context", type=int, default=2048)
+  ap.add_argument("--preset", default="qwen3-0.6b")
+  ap.add_argument("--layers", type=int, default=None, help="fewer layers than the preset (named in the record)")
+  ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+  ap.add_argument("--eager", action="store_true")
+  ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+    return 2
+
+  import torch
+  from miniinfer_amd import LLMEngine
+  from miniinfer_amd.presets import preset
+
+  full = preset(args.preset)
+  cfg = preset(args.preset, args.layers) if args.layers else full
+  layers = cfg.num_hidden_layers
+  max_batch = max(args.batch, 1 if args.no_points else 64)
+  page_size = 16
+  room = args.context + args.steps + args.warmup + (-(-max_batch * args.context // 8192)) + 16
+  max_len = max(4096, room)
+  pages = max_batch * (-(-room // page_size)) + 16
+  engine = LLMEngine(model="", model_config=cfg, random_weights_seed=0, dtype=args.dtype, page_size=page_size,
+                     num_pages=pages, max_num_seqs=max_batch, max_model_len=max_len, max_num_batched_tokens=8192,
+                     enforce_eager=args.eager)
+  esize = 2 if args.dtype == "bfloat16" else 4
+
+  sec = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
+  value = args.batch / sec
+  mid_context = args.context + args.warmup + args.steps // 2
+  bytes_step = decode_bytes(cfg, layers, args.batch, mid_context, esize)
+  achieved = bytes_step / sec / 1e9
+  rec = {
+    "metric": "decode tok/s @ batch 8, 2,048-token contexts, Qwen3-0.6B shape", "value": round(value, 2),
+    "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4),
+    "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+    "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (seeded random token ids, random weights)",
+    "config": {
+      "model": args.preset, "layers": layers, "layers_full": full.num_hidden_layers, "hidden": cfg.hidden_size,
+      "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+      "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": cfg.tie_word_embeddings,
+      "global_batch": args.batch, "seq_len": args.context, "max_model_len": max_len, "page_size": page_size,
+      "parallelism": "1 GPU", "graphs": not args.eager, "prefill_tokens": 2048,
+    },
+    "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                 "frac": round(achieved / PEAK_HBM_GBS, 4)},
+  }
+  if not args.no_points:
+    T = 2048
+    psec = time_prefill(engine, T, reps=3, seed=2)
+    fl = prefill_flops(cfg, layers, T)
+    rec["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
+                      "frac": round(fl / psec / PEAK_FLOPS[args.dtype], 4)}
+    points = {}
+    for b in (1, 64):
+      s = time_decode(engine, b, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), seed=10 + b)
+      points[f"decode_b{b}"] = round(b / s, 2)
+    rec["points"] = points
+  print(json.dumps(rec))
+  return 0
+
+
+if __name__ == "__main__":
+  sys.exit(main())

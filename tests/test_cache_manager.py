@@ -1,0 +1,128 @@
+"""The cache manager on the host: no page lost, held twice or freed twice, under random orders of requests;
+groups with a window give pages back as the window passes; state slots start at zero."""
+
+import random
+
+import pytest
+import torch
+
+from miniinfer_amd.cache import CacheError, CacheManager, OutOfPages, OutOfSlots, PagePool
+from miniinfer_amd.parts import FixedState, PagedKV
+
+
+def _mgr(needs=None, P=16, pages=8, slots=4, max_len=4096):
+  needs = needs if needs is not None else [PagedKV(2, 8)] * 2
+  return CacheManager(needs, page_size=P, num_pages=pages, max_requests=slots, max_model_len=max_len,
+                      dtype=torch.float32, device="cpu")
+
+
+def test_pool_never_hands_out_page_zero_and_catches_double_free():
+  pool = PagePool(5)
+  got = pool.alloc(5)
+  assert sorted(got) == [1, 2, 3, 4, 5]
+  with pytest.raises(OutOfPages):
+    pool.alloc(1)
+  pool.free([3])
+  with pytest.raises(CacheError, match="twice"):
+    pool.free([3])
+  with pytest.raises(CacheError):
+    pool.free([0])
+  assert pool.alloc(1) == [3]        # freed last, handed out first: reuse shows early
+
+
+def test_pages_open_exactly_at_page_edges():
+  # the reference's rules (tests/unittests/test_kv_cache_manager.py:300-373): a partial page is filled before a new
+  # one opens; decoding opens a page exactly when it crosses an edge
+  m = _mgr(P=16, pages=8)
+  m.admit("a")
+  m.grow("a", 10); m.commit("a", 10)
+  assert m.held_pages("a") == 1
+  m.grow("a", 16); m.commit("a", 16)
+  assert m.held_pages("a") == 1 and m.pages_needed("a", 16) == 0 and m.pages_needed("a", 17) == 1
+  m.grow("a", 17); m.commit("a", 17)
+  assert m.held_pages("a") == 2
+  # numbers of the reference's backend test (test_flashinfer_backend.py:50-71): lengths 10 and 20 at P=16 -> 1 and 2 pages
+  m.admit("b"); m.grow("b", 20)
+  assert m.held_pages("b") == 2
+  m.check()
+  m.release("a"); m.release("b")
+  assert m.num_free_pages() == 8 and m.num_free_slots() == 4
+  with pytest.raises(CacheError, match="not admitted"):
+    m.release("a")
+
+
+def test_grow_is_all_or_nothing_and_errors_are_typed():
+  m = _mgr(P=8, pages=4, slots=2)
+  m.admit(1); m.admit(2)
+  with pytest.raises(OutOfSlots):
+    m.admit(3)
+  m.grow(1, 24)
+  with pytest.raises(OutOfPages):
+    m.grow(2, 17)
+  assert m.held_pages(2) == 0 and m.num_free_pages() == 1
+
+
+def test_max_model_len_is_enforced():
+  m = _mgr(max_len=32)
+  m.admit("x")
+  with pytest.raises(CacheError, match="max_model_len"):
+    m.grow("x", 33)
+
+
+def test_groups_have_pages_of_their_own_and_windows_give_pages_back():
+  full, win = PagedKV(2, 8), PagedKV(2, 8, window=20)
+  m = _mgr(needs=[full, win, full, win, FixedState((4,), torch.float32)], P=8, pages=10)
+  assert len(m.paged) == 2 and m.paged[0].layers == [0, 2] and m.paged[1].layers == [1, 3]
+  assert m.paged[0].k.shape == (2, 11, 2, 8, 8)
+  assert m.layer_cache(3).group == 1 and m.layer_cache(3).window == 20 and m.layer_cache(4).kind == "state"
+  m.admit("r")
+  m.grow("r", 40); m.commit("r", 40)
+  # next token is at 40 and sees keys 21..40: pages 0 and 1 (keys 0..15) of the window group are gone
+  assert len(m.table(0, "r")) == 5 and all(p > 0 for p in m.table(0, "r"))
+  assert m.table(1, "r")[:2] == [0, 0] and all(p > 0 for p in m.table(1, "r")[2:])
+  assert m.paged[0].pool.num_free == 5 and m.paged[1].pool.num_free == 7
+  m.check()
+  for n in range(41, 80):
+    m.grow("r", n); m.commit("r", n); m.check()
+  assert sum(1 for p in m.table(1, "r") if p) <= 4      # a window of 20 keys touches at most 4 pages of 8
+  m.release("r")
+  assert m.paged[0].pool.num_free == 10 and m.paged[1].pool.num_free == 10
+
+
+def test_state_slots_are_zero_on_admission():
+  m = _mgr(needs=[FixedState((3,), torch.float32), PagedKV(1, 8)], slots=2)
+  s = m.admit("a")
+  m.states[0].state[0, s] = 7.0
+  m.release("a")
+  s2 = m.admit("b")
+  assert s2 == s and float(m.states[0].state[0, s2].abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_orders_keep_the_books(seed):
+  rnd = random.Random(seed)
+  m = _mgr(needs=[PagedKV(1, 8), PagedKV(1, 8, window=24)], P=8, pages=24, slots=5, max_len=400)
+  live = {}
+  next_id = 0
+  for _ in range(600):
+    op = rnd.random()
+    if op < 0.25 and m.num_free_slots() > 0:
+      m.admit(next_id); live[next_id] = 0; next_id += 1
+    elif op < 0.85 and live:
+      r = rnd.choice(list(live))
+      new_len = min(400, live[r] + rnd.choice([1, 1, 1, 2, 7, 30]))
+      if m.can_grow(r, new_len):
+        m.grow(r, new_len); m.commit(r, new_len); live[r] = new_len
+      else:
+        with pytest.raises(OutOfPages):
+          m.grow(r, new_len)
+    elif live:
+      r = rnd.choice(list(live))
+      m.release(r); del live[r]
+    m.check()
+    for r, n in live.items():
+      assert m.length(r) == n and m.held_pages(r) == -(-n // 8)
+  for r in list(live):
+    m.release(r)
+  m.check()
+  assert m.num_free_pages() == 24 and m.num_free_slots() == 5

@@ -1,0 +1,156 @@
+"""The scheduler's decisions on the host, with the real cache manager and a fake model whose next token is a
+function of the request's whole history (so recomputation after a preemption must give the same tokens)."""
+
+import random
+
+import pytest
+import torch
+
+from miniinfer_amd.cache import CacheManager
+from miniinfer_amd.engine.scheduler import Request, Scheduler
+from miniinfer_amd.parts import PagedKV
+from miniinfer_amd.sampling import SamplingParams
+
+V = 1000
+
+
+def fake_next(tokens):
+  h = 1469598103934665603
+  for t in tokens:
+    h = ((h ^ t) * 1099511628211) & ((1 << 64) - 1)
+  return h % V
+
+
+def make(pages, P=8, max_seqs=4, budget=32, max_len=512, chunked=True, eos=None):
+  cache = CacheManager([PagedKV(1, 8)], page_size=P, num_pages=pages, max_requests=max_seqs, max_model_len=max_len,
+                       dtype=torch.float32, device="cpu")
+  return cache, Scheduler(cache, max_num_seqs=max_seqs, max_num_batched_tokens=budget, max_model_len=max_len,
+                          enable_chunked_prefill=chunked, eos_token_id=eos)
+
+
+def run(cache, sched, reqs, max_steps=100000, on_step=None):
+  """Drives the scheduler like the engine does; the 'model' checks that it is fed contiguous portions."""
+  for r in reqs:
+    sched.add(r)
+  steps = 0
+  while sched.has_unfinished():
+    plan = sched.schedule()
+    assert plan is not None and plan.entries
+    assert plan.num_tokens <= sched.max_num_batched_tokens
+    assert len({id(e.request) for e in plan.entries}) == len(plan.entries)
+    sampled = {}
+    for e in plan.entries:
+      r = e.request
+      assert e.start == r.num_computed == cache.length(r.number), "a portion must continue where the cache ends"
+      assert 1 <= e.num_tokens <= r.remaining
+      cache.grow(r.number, e.start + e.num_tokens)       # what runner.step does
+      cache.commit(r.number, e.start + e.num_tokens)
+      assert e.samples == (e.start + e.num_tokens == r.num_tokens)
+      if e.samples:
+        sampled[r.number] = fake_next(r.tokens)
+    if on_step:
+      on_step(plan)
+    sched.update(plan, sampled)
+    cache.check()
+    steps += 1
+    assert steps < max_steps
+  return steps
+
+
+def expected(prompt, n):
+  toks = list(prompt)
+  for _ in range(n):
+    toks.append(fake_next(toks))
+  return toks[len(prompt):]
+
+
+def _req(i, n_prompt, max_tokens, seed=0, **kw):
+  rnd = random.Random(seed * 1000 + i)
+  return Request(number=i, request_id=f"r{i}", prompt=[rnd.randrange(V) for _ in range(n_prompt)],
+                 params=SamplingParams(temperature=0.0, max_tokens=max_tokens, ignore_eos=True, **kw))
+
+
+def test_prompts_are_cut_under_the_budget_and_decodes_ride_along():
+  cache, sched = make(pages=100, budget=32)
+  reqs = [_req(0, 70, 5), _req(1, 9, 8), _req(2, 40, 3)]
+  seen = []
+  run(cache, sched, reqs, on_step=lambda p: seen.append([(e.request.number, e.start, e.num_tokens) for e in p.entries]))
+  assert seen[0] == [(0, 0, 32)]                       # first portion takes the whole budget
+  assert seen[1] == [(0, 32, 32)]
+  assert seen[2] == [(0, 64, 6), (1, 0, 9), (2, 0, 17)]  # the rest of r0, all of r1, the start of r2
+  assert seen[3][:2] == [(0, 70, 1), (1, 9, 1)]          # decodes first, then r2's next portion
+  assert seen[3][2] == (2, 17, 23)
+  for r in reqs:
+    assert r.outputs == expected(r.prompt, r.params.max_tokens) and r.finish_reason == "max_tokens"
+  assert cache.num_free_pages() == 100 and cache.num_free_slots() == 4
+
+
+def test_without_chunked_prefill_prompts_run_whole():
+  cache, sched = make(pages=100, budget=64, chunked=False)
+  reqs = [_req(0, 40, 4), _req(1, 30, 4), _req(2, 20, 4)]
+  seen = []
+  run(cache, sched, reqs, on_step=lambda p: seen.append([(e.request.number, e.num_tokens) for e in p.entries]))
+  assert seen[0] == [(0, 40), (2, 20)] or seen[0] == [(0, 40)]   # r1 does not fit beside r0; nothing is cut
+  assert all(n in (1, 40, 30, 20) for step in seen for _, n in step)
+  with pytest.raises(ValueError, match="chunked"):
+    sched.add(_req(9, 100, 4))
+
+
+def test_batch_size_cap_and_fcfs():
+  cache, sched = make(pages=200, max_seqs=2, budget=64)
+  reqs = [_req(i, 10, 6) for i in range(5)]
+  live = []
+  run(cache, sched, reqs, on_step=lambda p: live.append(len(sched.running)))
+  assert max(live) <= 2
+  order = [r.number for r in sched.finished]
+  assert order == sorted(order)
+
+
+def test_pages_run_out_newest_is_preempted_and_recomputes():
+  # 4 requests that each grow to 30 + 50 = 80 tokens (10 pages) in a pool of 22 pages
+  cache, sched = make(pages=22, P=8, max_seqs=4, budget=48)
+  reqs = [_req(i, 30, 50) for i in range(4)]
+  preempted = []
+  run(cache, sched, reqs, on_step=lambda p: preempted.extend(r.number for r in p.preempted))
+  assert sched.num_preemptions > 0 and preempted
+  for r in reqs:
+    assert len(r.outputs) == 50 and r.outputs == expected(r.prompt, 50)     # exactly max_tokens, same tokens
+  assert reqs[0].num_preemptions == 0                  # the oldest running request is never the victim
+  assert cache.num_free_pages() == 22
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_starvation_level_pools_still_finish_everything(seed):
+  rnd = random.Random(seed)
+  P = 8
+  reqs = [_req(i, rnd.randint(1, 60), rnd.randint(1, 40), seed=seed) for i in range(12)]
+  biggest = max(-(-(len(r.prompt) + r.params.max_tokens) // P) for r in reqs)
+  cache, sched = make(pages=biggest + rnd.randint(0, 3), P=P, max_seqs=3, budget=rnd.choice([8, 16, 64]))
+  run(cache, sched, reqs)
+  for r in reqs:
+    assert r.outputs == expected(r.prompt, r.params.max_tokens)
+  assert cache.num_free_pages() == cache.num_pages and cache.num_free_slots() == 3
+
+
+def test_requests_that_can_never_fit_are_refused_when_added():
+  cache, sched = make(pages=4, P=8, max_len=64)
+  with pytest.raises(ValueError, match="never fit"):
+    sched.add(_req(0, 30, 10))
+  with pytest.raises(ValueError, match="max_model_len"):
+    sched.add(_req(1, 60, 10))
+  with pytest.raises(ValueError, match="at least one"):
+    sched.add(Request(number=2, request_id="e", prompt=[], params=SamplingParams()))
+
+
+def test_eos_and_length_finish():
+  cache, sched = make(pages=50, eos=None)
+  r = _req(0, 5, 20)
+  want = expected(r.prompt, 20)
+  cache2, sched2 = make(pages=50, eos=want[3])
+  r2 = Request(number=0, request_id="x", prompt=list(r.prompt), params=SamplingParams(temperature=0.0, max_tokens=20))
+  run(cache2, sched2, [r2])
+  assert r2.outputs == want[:want.index(want[3]) + 1] and r2.finish_reason == "eos"
+  r3 = Request(number=1, request_id="y", prompt=list(r.prompt),
+               params=SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True))
+  run(cache2, sched2, [r3])
+  assert r3.outputs == want and r3.finish_reason == "max_tokens"
