@@ -82,7 +82,7 @@ class PagedGroup:
   layers: List[int]
   pool: PagePool
   k: Optional[torch.Tensor] = None     # [len(layers), num_pages + 1, nkv, page_size, d]
-  v: Optional[torch.Tensor] = None
+  v: Optional[torch.Tensor] = None     # [len(layers), num_pages + 1, nkv, d, page_size] (transposed pages)
   tables: Dict[Hashable, List[int]] = field(default_factory=dict)   # per request: page id per page index, 0 = given back
 
 
@@ -99,7 +99,7 @@ class LayerCache:
   kind: str                              # "paged" | "state" | "none"
   group: int = -1
   k: Optional[torch.Tensor] = None       # [num_pages + 1, nkv, page_size, d]
-  v: Optional[torch.Tensor] = None
+  v: Optional[torch.Tensor] = None       # [num_pages + 1, nkv, d, page_size]
   state: Optional[torch.Tensor] = None   # [max_requests, *shape]
   page_size: int = 0
   window: Optional[int] = None
@@ -159,9 +159,10 @@ class CacheManager:
 
   def _allocate(self) -> None:
     for g in self.paged:
-      shape = (len(g.layers), self.num_pages + 1, g.need.num_kv_heads, self.page_size, g.need.head_dim)
-      g.k = torch.zeros(shape, dtype=self.dtype, device=self.device)
-      g.v = torch.zeros(shape, dtype=self.dtype, device=self.device)
+      n, h, d = len(g.layers), g.need.num_kv_heads, g.need.head_dim
+      # keys [.., page_size, d]; values transposed [.., d, page_size]: the MFMA kernels read runs of keys per dim
+      g.k = torch.zeros((n, self.num_pages + 1, h, self.page_size, d), dtype=self.dtype, device=self.device)
+      g.v = torch.zeros((n, self.num_pages + 1, h, d, self.page_size), dtype=self.dtype, device=self.device)
     for s in self.states:
       shape = (len(s.layers), self.max_requests) + tuple(s.need.shape)
       s.state = torch.zeros(shape, dtype=s.need.dtype or self.dtype, device=self.device)

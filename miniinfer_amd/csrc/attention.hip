@@ -13,6 +13,7 @@
 // One wave per (token, query head).  A tile is 64 keys: each lane scores one key (the query
 // is broadcast from LDS), the wave reduces max and sum for the running softmax, then the lanes
 // switch to output columns and add the tile's probability-weighted value rows.
+// Key pages are [num_pages, nkv, P, d]; value pages are stored transposed, [num_pages, nkv, d, P].
 #include "common.h"
 
 template <typename T, int VEC>
@@ -100,11 +101,11 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
       const float pi = __shfl(p, i, MI_WAVE);
       const int jj = j0 + i;
       const int64_t page = bt[jj >> page_shift];
-      const T* vrow = v_pages + ((page * nkv + g) * P + (jj & (P - 1))) * d;
+      const T* vcol = v_pages + (page * nkv + g) * (int64_t)d * P + (jj & (P - 1));   // value pages are [d][P]
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const int e = lane + c * MI_WAVE;
-        if (e < d) acc[c] = fmaf(pi, to_float(vrow[e]), acc[c]);
+        if (e < d) acc[c] = fmaf(pi, to_float(vcol[(int64_t)e * P]), acc[c]);
       }
     }
   }

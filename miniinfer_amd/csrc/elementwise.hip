@@ -135,7 +135,8 @@ MI_EXPORT int mi_silu_mul(int dtype, const void* gu, void* out, int M, int I, hi
 //   q heads: norm (if qw) and rotation (if cos_sin), written back in place;
 //   k heads: the same with kw, written to the key pages (and back in place);
 //   v heads: copied to the value pages.
-// Pages are [num_pages, nkv, P, d]; token t goes to slot slots[t] = page * P + offset.
+// Key pages are [num_pages, nkv, P, d]; value pages are stored transposed, [num_pages, nkv, d, P], so that the
+// attention kernels read runs of consecutive keys for one dim.  Token t goes to slot slots[t] = page * P + offset.
 // cos_sin [max_pos, rotary_dim] = cos(pos * inv_freq_j) for j < rotary_dim/2, then sin(...).
 // Pairs are (j, j + rotary_dim/2) within the first rotary_dim elements; the rest pass through.
 template <typename T>
@@ -160,15 +161,14 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_strid
     const int64_t page = slot >> page_shift;
     const int off = slot & (P - 1);
     const int g = (h - nq) % nkv;
-    T* base = (h < nq + nkv) ? k_pages : v_pages;
-    dst = base + ((page * nkv + g) * P + off) * d;
+    if (h < nq + nkv) {
+      dst = k_pages + ((page * nkv + g) * P + off) * d;
+    } else {  // value head: copy into the transposed page, element e of the head at [e][off]
+      T* vdst = v_pages + (page * nkv + g) * (int64_t)d * P + off;
+      for (int e = lane; e < d; e += MI_WAVE) vdst[(int64_t)e * P] = src[e];
+    }
   }
-
-  if (h >= nq + nkv) {  // value head: plain copy
-    if (dst)
-      for (int e = lane; e < d; e += MI_WAVE) dst[e] = src[e];
-    return;
-  }
+  if (h >= nq + nkv) return;
 
   const float* w = (h < nq) ? qw : kw;
   float rstd = 1.f;

@@ -54,9 +54,32 @@ class StepContext:
     self.max_q_len = 0
     self.max_kv_len = 0
     self._cache: CacheManager = None
+    self._device = None
+    self._work: Dict[int, torch.Tensor] = {}
+    self._scratch: Dict[str, torch.Tensor] = {}
 
   def layer_cache(self, layer: int) -> LayerCache:
     return self._cache.layer_cache(layer)
+
+  def prefill_work(self, tokens_per_block: int) -> torch.Tensor:
+    """[n, 2] int32 = (entry, block of `tokens_per_block` query tokens within it) for every multi-token entry;
+    built once per step and granule, shared by all layers."""
+    w = self._work.get(tokens_per_block)
+    if w is None:
+      items = [(b, i) for b in range(self.num_multi) for i in range(-(-self.q_lens[b] // tokens_per_block))]
+      # the blocks with the most keys first: they take longest
+      items.sort(key=lambda it: -(self.kv_lens[it[0]] - self.q_lens[it[0]] + (it[1] + 1) * tokens_per_block))
+      w = torch.tensor(items, dtype=torch.int32).reshape(-1, 2).to(self._device, non_blocking=True)
+      self._work[tokens_per_block] = w
+    return w
+
+  def scratch(self, name: str, numel: int, dtype: torch.dtype) -> torch.Tensor:
+    """A device buffer that lives for this step (reused by every layer that asks under the same name)."""
+    t = self._scratch.get(name)
+    if t is None or t.numel() < numel or t.dtype != dtype:
+      t = torch.empty(numel, dtype=dtype, device=self._device)
+      self._scratch[name] = t
+    return t
 
 
 class ModelRunner:
@@ -154,6 +177,7 @@ class ModelRunner:
 
     ctx = StepContext()
     ctx._cache = cache
+    ctx._device = self.device
     ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = T, B, R
     ctx.token_ids = dev[offs[0]:offs[0] + T]
     ctx.positions = dev[offs[1]:offs[1] + T]

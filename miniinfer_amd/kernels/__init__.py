@@ -5,7 +5,10 @@ from typing import List
 from . import jit
 
 # every shared object of the library: (source name, defines)
-ALL_MODULES = [("elementwise", ()), ("gemm", ()), ("attention", ()), ("sampling", ())]
+# head sizes the MFMA attention is prebuilt for (others are built at a model's first use)
+PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
+ALL_MODULES = [("elementwise", ()), ("gemm", ()), ("attention", ()), ("sampling", ())] + \
+    [("attention_mfma", (("HEAD_DIM", d),)) for d in PREBUILT_HEAD_DIMS]
 
 
 def build_all(force: bool = False) -> List[str]:

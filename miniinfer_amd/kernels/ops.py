@@ -89,6 +89,14 @@ _SIGS = {
   },
 }
 
+_SIGS["attention_mfma"] = {
+  "mi_attn_prefill": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                      c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
+  "mi_attn_decode": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                     c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
+  "mi_attn_prefill_tokens_per_block": [c_int, c_int],
+}
+
 _SIGS["sampling"] = {
   "mi_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
 }
@@ -117,6 +125,20 @@ def _check(lib, rc):
 def modules_for(spec_kinds=()):
   """(name, defines) of every shared object the plain kernel set needs."""
   return [("elementwise", ()), ("gemm", ()), ("attention", ())]
+
+
+def _check_pages(what, k_pages, v_pages, nkv, d, dtype):
+  """Key pages [pages, nkv, P, d]; value pages transposed [pages, nkv, d, P]."""
+  if k_pages.dim() != 4 or v_pages.dim() != 4:
+    raise KernelError(f"{what}: pages must have 4 dims")
+  n, h, P, dd = k_pages.shape
+  if h != nkv or dd != d or tuple(v_pages.shape) != (n, nkv, d, P):
+    raise KernelError(f"{what}: key pages {tuple(k_pages.shape)} / value pages {tuple(v_pages.shape)} are not "
+                      f"[pages, {nkv}, P, {d}] / [pages, {nkv}, {d}, P]")
+  if k_pages.dtype != dtype or v_pages.dtype != dtype:
+    raise KernelError(f"{what}: pages are {k_pages.dtype}/{v_pages.dtype}, activations {dtype}")
+  _contig("k_pages", k_pages)
+  _contig("v_pages", v_pages)
 
 
 # ----------------------------------------------------------------------------- embedding
@@ -190,8 +212,9 @@ def qk_norm_rope_cache(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: O
                        positions: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
                        v_pages: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> None:
   """In place on qkv [T, (nq + 2 nkv) d]: per-head RMS norm of q and k (if weights), rotation of q and k
-  (if cos_sin [max_pos, rotary_dim]), and a copy of the new k and v rows into pages
-  [num_pages, nkv, page_size, d] at slots[t] = page * page_size + offset."""
+  (if cos_sin [max_pos, rotary_dim]), and a copy of the new k rows into key pages [num_pages, nkv, page_size, d]
+  and of the new v rows into the transposed value pages [num_pages, nkv, d, page_size], at
+  slots[t] = page * page_size + offset."""
   _dev(qkv, q_weight, k_weight, cos_sin, positions, k_pages, v_pages, slots)
   if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] != (nq + 2 * nkv) * d:
     raise KernelError(f"qk_norm_rope_cache: qkv {tuple(qkv.shape)} does not hold {nq}+2*{nkv} heads of {d}")
@@ -204,11 +227,9 @@ def qk_norm_rope_cache(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: O
     max_pos, rotary_dim = cos_sin.shape
     _i32("positions", positions, T)
   if k_pages is not None:
-    for name, p in (("k_pages", k_pages), ("v_pages", v_pages)):
-      _contig(name, p)
-      if p.dtype != qkv.dtype or p.dim() != 4 or tuple(p.shape[1:]) != (nkv, page_size, d):
-        raise KernelError(f"qk_norm_rope_cache: {name} {tuple(p.shape)} {p.dtype} is not [pages, {nkv}, {page_size}, {d}] "
-                          f"of {qkv.dtype}")
+    _check_pages("qk_norm_rope_cache", k_pages, v_pages, nkv, d, qkv.dtype)
+    if k_pages.shape[2] != page_size:
+      raise KernelError(f"qk_norm_rope_cache: pages of {k_pages.shape[2]} tokens, page_size={page_size}")
     _i32("slots", slots, T)
   lib = _lib("elementwise")
   _check(lib, lib.mi_qk_norm_rope_cache(dtype_code(qkv.dtype), _ptr(qkv), qkv.stride(0), T, nq, nkv, d,
@@ -249,19 +270,16 @@ def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tenso
   """Causal attention of new tokens over their requests' paged keys and values.
 
   q: [T, >= nq*d] rows (the q part of a fused qkv buffer is fine), out [T, nq*d];
-  pages [num_pages, nkv, P, d]; block_table [B, W] int32; token_req [T] = request of each token;
+  key pages [num_pages, nkv, P, d], value pages [num_pages, nkv, d, P]; block_table [B, W] int32; token_req [T] = request of each token;
   cu_q [B+1] = first token of each request; kv_len [B] = keys per request including the new tokens."""
   _dev(q, out, k_pages, v_pages, block_table, token_req, cu_q, kv_len)
   T = q.shape[0]
   B = kv_len.numel()
   if q.stride(1) != 1 or q.shape[1] < nq * d or out.stride(1) != 1 or out.shape != (T, nq * d):
     raise KernelError(f"paged_attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not hold {nq} heads of {d}")
-  if k_pages.shape != v_pages.shape or k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d:
-    raise KernelError(f"paged_attention: pages {tuple(k_pages.shape)} are not [pages, {nkv}, P, {d}]")
-  if not (q.dtype == out.dtype == k_pages.dtype == v_pages.dtype):
-    raise KernelError("paged_attention: q, out and pages must share a dtype")
-  _contig("k_pages", k_pages)
-  _contig("v_pages", v_pages)
+  _check_pages("paged_attention", k_pages, v_pages, nkv, d, q.dtype)
+  if q.dtype != out.dtype:
+    raise KernelError("paged_attention: q and out must share a dtype")
   _i32("block_table", block_table)
   if block_table.dim() != 2 or block_table.shape[0] < B:
     raise KernelError(f"paged_attention: block_table {tuple(block_table.shape)} for {B} requests")
@@ -300,3 +318,73 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_k: Opt
   _check(lib, lib.mi_sample(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature), _ptr(top_k),
                             _ptr(top_p), _ptr(seeds), _ptr(steps), _ptr(out), _stream()))
   return out
+
+
+# ----------------------------------------------------------------------------- attention on the matrix cores
+
+def mfma_attention_supported(dtype: torch.dtype, nq: int, nkv: int, d: int, page_size: int) -> bool:
+  """The MFMA attention kernels take bfloat16, head sizes that are multiples of 16 up to 256, up to 16 query
+  heads per kv head, and pages of at least 4 tokens; everything else runs on the plain kernel."""
+  return (dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and nq % nkv == 0 and nq // nkv <= 16
+          and page_size >= 4)
+
+
+def attn_prefill_tokens_per_block(nq: int, nkv: int, d: int) -> int:
+  """Query tokens one wave of the prefill kernel takes (the granule of its work list)."""
+  lib = _lib("attention_mfma", (("HEAD_DIM", d),))
+  return lib.mi_attn_prefill_tokens_per_block(nq, nkv)
+
+
+def _attn_common(what, q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len):
+  _dev(q, out, k_pages, v_pages, block_table, cu_q, kv_len)
+  T = q.shape[0]
+  if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+    raise KernelError(f"{what}: bfloat16 only")
+  if q.stride(1) != 1 or q.shape[1] < nq * d or out.stride(1) != 1 or tuple(out.shape) != (T, nq * d):
+    raise KernelError(f"{what}: q {tuple(q.shape)} / out {tuple(out.shape)} do not hold {nq} heads of {d}")
+  _check_pages(what, k_pages, v_pages, nkv, d, q.dtype)
+  _i32("block_table", block_table)
+  B = kv_len.numel()
+  if block_table.dim() != 2 or block_table.shape[0] < B:
+    raise KernelError(f"{what}: block_table {tuple(block_table.shape)} for {B} requests")
+  _i32("cu_q", cu_q, B + 1)
+  _i32("kv_len", kv_len, B)
+  return B
+
+
+def attn_prefill(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
+                 v_pages: torch.Tensor, block_table: torch.Tensor, work: torch.Tensor, cu_q: torch.Tensor,
+                 kv_len: torch.Tensor, scale: float, window: int = 0) -> None:
+  """MFMA attention of the entries named in `work` [n, 2] = (entry, block of `attn_prefill_tokens_per_block` query
+  tokens within it).  Other arguments as `paged_attention`."""
+  _attn_common("attn_prefill", q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len)
+  _dev(work)
+  _i32("work", work)
+  if work.dim() != 2 or work.shape[1] != 2:
+    raise KernelError("attn_prefill: work must be [n, 2]")
+  lib = _lib("attention_mfma", (("HEAD_DIM", d),))
+  _check(lib, lib.mi_attn_prefill(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages),
+                                  _ptr(block_table), block_table.shape[1], _ptr(work), work.shape[0], _ptr(cu_q),
+                                  _ptr(kv_len), nq, nkv, k_pages.shape[2], float(scale), int(window), _stream()))
+
+
+def attn_decode(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
+                v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor, kv_len: torch.Tensor,
+                first_entry: int, num_entries: int, num_splits: int, part_o: torch.Tensor, part_ml: torch.Tensor,
+                scale: float, window: int = 0) -> None:
+  """MFMA split-key attention of entries first_entry .. first_entry + num_entries - 1, each of which brings exactly
+  one token.  part_o float32 [>= num_entries * nq * num_splits * d], part_ml float32 [>= num_entries * nq *
+  num_splits * 2] are scratch."""
+  B = _attn_common("attn_decode", q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len)
+  if first_entry < 0 or num_entries < 0 or first_entry + num_entries > B:
+    raise KernelError(f"attn_decode: entries {first_entry}..{first_entry + num_entries} of {B}")
+  _dev(part_o, part_ml)
+  need = num_entries * nq * num_splits
+  if part_o.dtype != torch.float32 or part_o.numel() < need * d or part_ml.dtype != torch.float32 \
+      or part_ml.numel() < need * 2 or not part_o.is_contiguous() or not part_ml.is_contiguous():
+    raise KernelError("attn_decode: partial buffers are too small or not float32")
+  lib = _lib("attention_mfma", (("HEAD_DIM", d),))
+  _check(lib, lib.mi_attn_decode(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages),
+                                 _ptr(block_table), block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry,
+                                 num_entries, num_splits, _ptr(part_o), _ptr(part_ml), nq, nkv, k_pages.shape[2],
+                                 float(scale), int(window), _stream()))

@@ -65,9 +65,36 @@ class PagedAttention(Part):
       self.k_norm.weight if self.k_norm is not None else None,
       eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
     out = torch.empty((T, self.nq * self.d), dtype=x.dtype, device=x.device)
-    ops.paged_attention(qkv, self.nq, self.nkv, self.d, out, cache.k, cache.v, ctx.block_tables[cache.group],
-                        ctx.token_req, ctx.cu_q, ctx.kv_len, self.scale, self.window or 0)
+    self._attend(qkv, out, ctx, cache)
     return linear(out, self.o_weight)
+
+  def _attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx, cache) -> None:
+    nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0
+    table = ctx.block_tables[cache.group]
+    if not ops.mfma_attention_supported(qkv.dtype, nq, nkv, d, cache.page_size):
+      ops.paged_attention(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.token_req, ctx.cu_q, ctx.kv_len,
+                          self.scale, window)
+      return
+    # entries with several tokens come first, single tokens last
+    if ctx.num_multi > 0:
+      work = ctx.prefill_work(ops.attn_prefill_tokens_per_block(nq, nkv, d))
+      ops.attn_prefill(qkv, nq, nkv, d, out, cache.k, cache.v, table, work, ctx.cu_q, ctx.kv_len, self.scale, window)
+    n_single = ctx.num_requests - ctx.num_multi
+    if n_single > 0:
+      splits = decode_splits(n_single * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len)
+      need = n_single * nq * splits
+      part_o = ctx.scratch("attn_part_o", need * d, torch.float32)
+      part_ml = ctx.scratch("attn_part_ml", need * 2, torch.float32)
+      ops.attn_decode(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, ctx.num_multi, n_single,
+                      splits, part_o, part_ml, self.scale, window)
+
+
+def decode_splits(num_head_entries: int, max_keys: int, target_waves: int = 2048) -> int:
+  """Into how many key ranges a decoding request is cut: enough waves to fill the chip, at least 4 tiles of 16
+  keys each."""
+  tiles = -(-max_keys // 16)
+  want = -(-target_waves // max(1, num_head_entries))
+  return int(max(1, min(want, max(1, tiles // 4), 256)))
 
 
 register_mixer("paged_attention", PagedAttention)

@@ -73,7 +73,7 @@ def test_groups_have_pages_of_their_own_and_windows_give_pages_back():
   full, win = PagedKV(2, 8), PagedKV(2, 8, window=20)
   m = _mgr(needs=[full, win, full, win, FixedState((4,), torch.float32)], P=8, pages=10)
   assert len(m.paged) == 2 and m.paged[0].layers == [0, 2] and m.paged[1].layers == [1, 3]
-  assert m.paged[0].k.shape == (2, 11, 2, 8, 8)
+  assert m.paged[0].k.shape == (2, 11, 2, 8, 8) and m.paged[0].v.shape == (2, 11, 2, 8, 8)
   assert m.layer_cache(3).group == 1 and m.layer_cache(3).window == 20 and m.layer_cache(4).kind == "state"
   m.admit("r")
   m.grow("r", 40); m.commit("r", 40)

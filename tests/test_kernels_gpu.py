@@ -131,14 +131,14 @@ def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P):
 
   dq = qkv.to(DEV)
   kp = torch.zeros(pages + 1, nkv, P, d, dtype=dtype, device=DEV)
-  vp = torch.zeros_like(kp)
+  vp = torch.zeros(pages + 1, nkv, d, P, dtype=dtype, device=DEV)   # value pages are stored transposed
   ops.qk_norm_rope_cache(dq, nq, nkv, d, qw.to(DEV), kw.to(DEV), eps, table.to(DEV), pos.to(torch.int32).to(DEV),
                          kp, vp, slots.to(torch.int32).to(DEV), P)
   got = dq.float().cpu().view(T, nq + 2 * nkv, d)
   torch.testing.assert_close(got[:, :nq], q_want, **_tol(dtype))
   torch.testing.assert_close(got[:, nq:nq + nkv], k_want, **_tol(dtype))
   assert torch.equal(got[:, nq + nkv:], v)
-  kc, vc = kp.float().cpu(), vp.float().cpu()
+  kc, vc = kp.float().cpu(), vp.float().cpu().transpose(2, 3)
   for t in range(T):
     page, off = int(slots[t]) // P, int(slots[t]) % P
     assert torch.equal(kc[page, :, off], got[t, nq:nq + nkv])
@@ -179,7 +179,7 @@ def test_paged_attention(dtype, nq, nkv, d, P, window):
   n_pages = sum(-(-kv // P) for kv in kv_lens)
   perm = (torch.randperm(n_pages, generator=g) + 1).tolist()
   kp = torch.randn(n_pages + 1, nkv, P, d, generator=g).to(dtype)
-  vp = torch.randn(n_pages + 1, nkv, P, d, generator=g).to(dtype)
+  vp = torch.randn(n_pages + 1, nkv, P, d, generator=g).to(dtype)      # [page, head, key, dim]; the kernel gets it transposed
   q = torch.randn(T, nq * d, generator=g).to(dtype)
   table = torch.zeros(B, W, dtype=torch.int32)
   cu = [0]
@@ -198,8 +198,8 @@ def test_paged_attention(dtype, nq, nkv, d, P, window):
   want = torch.cat(want, 0)
   out = torch.empty(T, nq * d, dtype=dtype, device=DEV)
   i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
-  ops.paged_attention(q.to(DEV), nq, nkv, d, out, kp.to(DEV), vp.to(DEV), table.to(DEV), i32(token_req), i32(cu),
-                      i32(kv_lens), d ** -0.5, window)
+  ops.paged_attention(q.to(DEV), nq, nkv, d, out, kp.to(DEV), vp.transpose(2, 3).contiguous().to(DEV), table.to(DEV),
+                      i32(token_req), i32(cu), i32(kv_lens), d ** -0.5, window)
   torch.testing.assert_close(out.double().cpu(), want, **(_tol(dtype) if dtype == torch.bfloat16
                                                            else dict(rtol=1e-5, atol=1e-5)))
 
@@ -209,10 +209,100 @@ def test_attention_one_key_returns_its_value():
   from miniinfer_amd.kernels import ops
   nq, nkv, d, P = 4, 2, 32, 8
   kp = torch.randn(3, nkv, P, d, device=DEV)
-  vp = torch.randn(3, nkv, P, d, device=DEV)
+  vp = torch.randn(3, nkv, d, P, device=DEV)
   q = torch.randn(1, nq * d, device=DEV)
   out = torch.empty(1, nq * d, device=DEV)
   i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
   ops.paged_attention(q, nq, nkv, d, out, kp, vp, i32([[2]]), i32([0]), i32([0, 1]), i32([1]), d ** -0.5, 0)
   for h in range(nq):
-    torch.testing.assert_close(out[0, h * d:(h + 1) * d], vp[2, h // 2, 0])
+    torch.testing.assert_close(out[0, h * d:(h + 1) * d], vp[2, h // 2, :, 0])
+
+
+def _paged_case(reqs, nq, nkv, d, P, window, seed):
+  """Random pages and queries for requests (keys already cached, new tokens); returns device tensors, the plain
+  result, and the host lists."""
+  g = torch.Generator().manual_seed(seed)
+  B = len(reqs)
+  kv_lens = [a + n for a, n in reqs]
+  T = sum(n for _, n in reqs)
+  W = max(-(-kv // P) for kv in kv_lens)
+  n_pages = sum(-(-kv // P) for kv in kv_lens)
+  perm = (torch.randperm(n_pages, generator=g) + 1).tolist()
+  kp = torch.randn(n_pages + 1, nkv, P, d, generator=g).bfloat16()
+  vp = torch.randn(n_pages + 1, nkv, P, d, generator=g).bfloat16()
+  q = torch.randn(T, (nq + 2 * nkv) * d, generator=g).bfloat16()     # a fused qkv buffer: q is its first part
+  table = torch.zeros(B, W, dtype=torch.int32)
+  cu, token_req, want = [0], [], []
+  for b, (past, n) in enumerate(reqs):
+    npg = -(-kv_lens[b] // P)
+    pages = [perm.pop() for _ in range(npg)]
+    table[b, :npg] = torch.tensor(pages, dtype=torch.int32)
+    kk = torch.cat([kp[p].transpose(0, 1) for p in pages], 0)[:kv_lens[b]]
+    vv = torch.cat([vp[p].transpose(0, 1) for p in pages], 0)[:kv_lens[b]]
+    qq = q[cu[-1]:cu[-1] + n, :nq * d].reshape(n, nq, d)
+    want.append(_attention_ref(qq.float(), kk.float(), vv.float(), d ** -0.5, window).reshape(n, nq * d))
+    token_req += [b] * n
+    cu.append(cu[-1] + n)
+  i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+  return dict(q=q.to(DEV), kp=kp.to(DEV), vp=vp.transpose(2, 3).contiguous().to(DEV), table=table.to(DEV),
+              cu=i32(cu), kv=i32(kv_lens), token_req=i32(token_req), want=torch.cat(want, 0), T=T, B=B, q_lens=[n for _, n in reqs])
+
+
+MFMA_SHAPES = [(16, 8, 128, 16, 0), (6, 3, 48, 16, 0), (8, 2, 32, 8, 0), (4, 4, 16, 4, 0), (5, 1, 80, 32, 0),
+               (16, 1, 64, 16, 0), (12, 4, 96, 64, 0), (4, 2, 256, 16, 0), (8, 4, 128, 16, 50), (6, 2, 64, 8, 17)]
+
+
+@pytest.mark.parametrize("nq,nkv,d,P,window", MFMA_SHAPES)
+def test_mfma_prefill_attention(nq, nkv, d, P, window):
+  from miniinfer_amd.kernels import ops
+  reqs = [(0, 70), (129, 2), (40, 33), (0, 2), (63, 17), (300, 5)]
+  c = _paged_case(reqs, nq, nkv, d, P, window, seed=6)
+  tpb = ops.attn_prefill_tokens_per_block(nq, nkv, d)
+  work = [(b, i) for b, n in enumerate(c["q_lens"]) for i in range(-(-n // tpb))]
+  out = torch.zeros(c["T"], nq * d, dtype=torch.bfloat16, device=DEV)
+  ops.attn_prefill(c["q"], nq, nkv, d, out, c["kp"], c["vp"], c["table"],
+                   torch.tensor(work, dtype=torch.int32, device=DEV), c["cu"], c["kv"], d ** -0.5, window)
+  torch.testing.assert_close(out.double().cpu(), c["want"], rtol=1.6e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("splits", [1, 3, 16])
+@pytest.mark.parametrize("nq,nkv,d,P,window", MFMA_SHAPES)
+def test_mfma_decode_attention_any_number_of_splits(nq, nkv, d, P, window, splits):
+  from miniinfer_amd.kernels import ops
+  # two multi-token entries first (skipped by the decode kernel), then single-token entries
+  reqs = [(5, 3), (0, 2), (129, 1), (0, 1), (15, 1), (16, 1), (700, 1), (63, 1)]
+  c = _paged_case(reqs, nq, nkv, d, P, window, seed=7)
+  first, n = 2, 6
+  out = torch.zeros(c["T"], nq * d, dtype=torch.bfloat16, device=DEV)
+  part_o = torch.empty(n * nq * splits * d, dtype=torch.float32, device=DEV)
+  part_ml = torch.empty(n * nq * splits * 2, dtype=torch.float32, device=DEV)
+  ops.attn_decode(c["q"], nq, nkv, d, out, c["kp"], c["vp"], c["table"], c["cu"], c["kv"], first, n, splits, part_o,
+                  part_ml, d ** -0.5, window)
+  torch.testing.assert_close(out.double().cpu()[5:], c["want"][5:], rtol=1.6e-2, atol=1e-2)
+  assert float(out[:5].abs().sum()) == 0.0       # rows of the multi-token entries are not touched
+
+
+def test_mfma_attention_finds_a_far_key_and_respects_the_window_edge():
+  """One key among hundreds is made to stand out (its score is far above the rest): the output must be its value.
+  With a window that just excludes it, it must vanish; with one that just includes it, it is back."""
+  from miniinfer_amd.kernels import ops
+  nq, nkv, d, P = 4, 2, 64, 16
+  kv, far = 600, 37
+  c = _paged_case([(kv - 1, 1)], nq, nkv, d, P, 0, seed=8)
+  q = c["q"].clone()
+  kp, vp, table = c["kp"].clone(), c["vp"].clone(), c["table"]
+  page, off = int(table[0, far // P]), far % P
+  qh = q[0, :nq * d].float().view(nq, d)
+  for g in range(nkv):
+    kp[page, g, off] = (qh[g * 2] * 4).bfloat16()        # aligned with the first head of each group
+  out = torch.empty(1, nq * d, dtype=torch.bfloat16, device=DEV)
+  po = torch.empty(nq * 8 * d, dtype=torch.float32, device=DEV)
+  pm = torch.empty(nq * 8 * 2, dtype=torch.float32, device=DEV)
+  run = lambda w: ops.attn_decode(q, nq, nkv, d, out, kp, vp, table, c["cu"], c["kv"], 0, 1, 8, po, pm, d ** -0.5, w)
+  run(0)
+  for g in range(nkv):
+    torch.testing.assert_close(out[0, g * 2 * d:(g * 2 + 1) * d].float(), vp[page, g, :, off].float(), rtol=2e-2, atol=2e-2)
+  run(kv - 1 - far)          # sees keys far+1 .. kv-1: the far key is just outside
+  assert (out[0, :d].float() - vp[page, 0, :, off].float()).abs().max() > 0.5
+  run(kv - far)              # just inside
+  torch.testing.assert_close(out[0, :d].float(), vp[page, 0, :, off].float(), rtol=2e-2, atol=2e-2)
