@@ -29,13 +29,39 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int D = HEAD_DIM;
 constexpr int KSTEPS = D / 32;          // 16x16x32 products over the head dim
-constexpr bool KREM = (D % 32) != 0;    // plus one 16x16x16 product
+constexpr bool KREM = (D % 32) != 0;    // plus one more, half of it zeros
 constexpr int DBLK = D / 16;            // 16-row blocks of O^T
 
+// The last 16 dims of a head size that is no multiple of 32 go through the same 16x16x32 product with the
+// upper half of the contraction zeroed: lanes 0..31 hold 8 dims each, lanes 32..63 hold zeros.  (Finishing
+// the score with a 16x16x16 product on the accumulator of the 16x16x32 ones gave wrong sums on gfx950 with
+// hipcc 7.2 whenever a wave ran more than one tile; one opcode per accumulator chain does not.)
 struct QRegs {
-  bf16x8 full[KSTEPS > 0 ? KSTEPS : 1];
-  s16x4 rem;
+  bf16x8 full[KSTEPS + (KREM ? 1 : 0)];
 };
+constexpr int QSTEPS = KSTEPS + (KREM ? 1 : 0);
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+// operand registers of one row (a key's or a query's `D` elements) in the lane's MFMA slots
+__device__ __forceinline__ void load_row(bf16x8 (&r)[QSTEPS], const uint16_t* row, bool ok) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    r[s] = *reinterpret_cast<const bf16x8*>(row + 32 * s + 8 * (lane >> 4));
+    if (!ok) r[s] = zero8();
+  }
+  if (KREM) {
+    const bool low = (lane >> 4) < 2;
+    r[KSTEPS] = *reinterpret_cast<const bf16x8*>(row + 32 * KSTEPS + 8 * ((lane >> 4) & 1));
+    if (!ok || !low) r[KSTEPS] = zero8();
+  }
+}
 
 struct Geometry {
   const uint16_t* k_pages;   // [pages, nkv, P, D]
@@ -66,17 +92,7 @@ __device__ __forceinline__ void load_queries(QRegs (&q)[NB], const uint16_t* q_b
     const int tok = col / gpad, hh = col % gpad;
     const bool ok = hh < G && tok < q_tokens;
     const uint16_t* row = q_base + (int64_t)(ok ? tok : 0) * q_row_stride + (int64_t)(head0 + (ok ? hh : 0)) * D;
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      bf16x8 v = *reinterpret_cast<const bf16x8*>(row + 32 * s + 8 * (lane >> 4));
-      if (!ok) v = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      q[nb].full[s] = v;
-    }
-    if (KREM) {
-      s16x4 v = *reinterpret_cast<const s16x4*>(row + 32 * KSTEPS + 4 * (lane >> 4));
-      if (!ok) v = s16x4{0, 0, 0, 0};
-      q[nb].rem = v;
-    }
+    load_row(q[nb].full, row, ok);
   }
 }
 
@@ -102,11 +118,8 @@ __device__ __forceinline__ void attend(State<NB>& st, const QRegs (&q)[NB], cons
     kk = kk > last ? last : kk;
     const int64_t kpage = geo.bt[kk >> geo.page_shift];
     const uint16_t* krow = geo.k_pages + ((kpage * geo.nkv + geo.g) * P + (kk & (P - 1))) * D;
-    bf16x8 ka[KSTEPS > 0 ? KSTEPS : 1];
-    s16x4 ka_rem;
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) ka[s] = *reinterpret_cast<const bf16x8*>(krow + 32 * s + 8 * (lane >> 4));
-    if (KREM) ka_rem = *reinterpret_cast<const s16x4*>(krow + 32 * KSTEPS + 4 * (lane >> 4));
+    bf16x8 ka[QSTEPS];
+    load_row(ka, krow, true);
     int vk = j0 + 4 * (lane >> 4);
     vk = vk > last ? (last & ~3) : vk;
     const int64_t vpage = geo.bt[vk >> geo.page_shift];
@@ -119,8 +132,7 @@ __device__ __forceinline__ void attend(State<NB>& st, const QRegs (&q)[NB], cons
     for (int nb = 0; nb < NB; ++nb) {
       f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int k = 0; k < KSTEPS; ++k) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[k], q[nb].full[k], s, 0, 0, 0);
-      if (KREM) s = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka_rem, q[nb].rem, s, 0, 0, 0);
+      for (int k = 0; k < QSTEPS; ++k) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[k], q[nb].full[k], s, 0, 0, 0);
       // lane holds S^T[key j0 + 4 (lane / 16) + i][column lane % 16]
       const int kbase = j0 + 4 * (lane >> 4);
       float sv[4];
