@@ -63,7 +63,7 @@ class LLMEngine:
     self.num_pages = cfg.num_pages if cfg.num_pages is not None else self._pages_from_memory(needs)
     self.cache = CacheManager(needs, page_size=cfg.page_size, num_pages=self.num_pages, max_requests=cfg.max_num_seqs,
                               max_model_len=self.max_model_len, dtype=self.dtype, device=self.device)
-    self.runner = ModelRunner(self.model, self.cache)
+    self.runner = ModelRunner(self.model, self.cache, use_graphs=not cfg.enforce_eager)
     eos = cfg.eos if cfg.eos is not None else getattr(self.model_config, "eos_token_id", None)
     self.eos_token_id = eos
     self.scheduler = Scheduler(self.cache, max_num_seqs=cfg.max_num_seqs,

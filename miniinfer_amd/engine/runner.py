@@ -82,13 +82,102 @@ class StepContext:
     return t
 
 
+class _Layout:
+  """Host-side arrays of one step (numpy int32), in the order the device buffer holds them."""
+  FIELDS = ("token_ids", "positions", "token_req", "cu_q", "kv_len", "req_slots", "logit_rows", "slots", "tables")
+
+  def __init__(self, T, B, R, G, W):
+    self.T, self.B, self.R, self.G, self.W = T, B, R, G, W
+    self.sizes = dict(token_ids=T, positions=T, token_req=T, cu_q=B + 1, kv_len=B, req_slots=B, logit_rows=R,
+                      slots=G * T, tables=G * B * W)
+    self.offsets = {}
+    o = 0
+    for f in self.FIELDS:
+      self.offsets[f] = o
+      o += self.sizes[f]
+    self.total = o
+
+  def views(self, buf):
+    """Slices of a flat int32 buffer (numpy array or torch tensor), one per field."""
+    return {f: buf[self.offsets[f]:self.offsets[f] + self.sizes[f]] for f in self.FIELDS}
+
+  def context(self, dev: torch.Tensor, cache: CacheManager, device) -> StepContext:
+    v = self.views(dev)
+    ctx = StepContext()
+    ctx._cache, ctx._device = cache, device
+    ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = self.T, self.B, self.R
+    ctx.token_ids, ctx.positions, ctx.token_req = v["token_ids"], v["positions"], v["token_req"]
+    ctx.cu_q, ctx.kv_len, ctx.req_slots, ctx.logit_rows = v["cu_q"], v["kv_len"], v["req_slots"], v["logit_rows"]
+    ctx.slots = [v["slots"][g * self.T:(g + 1) * self.T] for g in range(self.G)]
+    ctx.block_tables = [v["tables"][g * self.B * self.W:(g + 1) * self.B * self.W].view(self.B, self.W)
+                        for g in range(self.G)]
+    return ctx
+
+
+class _DecodeGraph:
+  """One captured decode step for `B` single-token entries and block tables `W` pages wide.
+  Its integer inputs live in one static device buffer that a step refreshes with one copy."""
+
+  def __init__(self, runner: "ModelRunner", B: int, W: int):
+    self.B, self.W = B, W
+    cache = runner.cache
+    G = len(cache.paged)
+    self.layout = _Layout(T=B, B=B, R=B, G=G, W=W)
+    self.stage = torch.zeros(self.layout.total, dtype=torch.int32, pin_memory=True)
+    self.host = self.layout.views(self.stage.numpy())
+    # what never changes: one token per entry, every row's logits
+    self.host["token_req"][:] = np.arange(B, dtype=np.int32)
+    self.host["cu_q"][:] = np.arange(B + 1, dtype=np.int32)
+    self.host["logit_rows"][:] = np.arange(B, dtype=np.int32)
+    self.fill_padding(0)
+    self.dev = torch.zeros(self.layout.total, dtype=torch.int32, device=runner.device)
+    self.dev.copy_(self.stage)
+    ctx = self.layout.context(self.dev, cache, runner.device)
+    ctx.q_lens, ctx.kv_lens = [1] * B, [W * cache.page_size] * B   # host-side sizes the kernels are tuned for
+    ctx.num_multi, ctx.max_q_len, ctx.max_kv_len = 0, 1, W * cache.page_size
+    self.ctx = ctx
+    # every entry is padding while warming up and capturing: it reads and writes the scratch page only
+    side = torch.cuda.Stream(device=runner.device)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      runner.model.forward(ctx)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    self.graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(self.graph):
+      self.logits = runner.model.forward(ctx)
+
+  def fill_padding(self, first: int) -> None:
+    """Entries first.. are padding: token 0 at position 0 of a request of one key in the scratch page."""
+    h = self.host
+    h["token_ids"][first:] = 0
+    h["positions"][first:] = 0
+    h["kv_len"][first:] = 1
+    h["req_slots"][first:] = 0
+    G, B, W = self.layout.G, self.B, self.W
+    h["slots"].reshape(G, B)[:, first:] = 0
+    h["tables"].reshape(G, B, W)[:, first:, :] = 0
+
+  def run(self) -> torch.Tensor:
+    self.dev.copy_(self.stage, non_blocking=True)
+    self.graph.replay()
+    return self.logits
+
+
+_GRAPH_BATCHES = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64)
+
+
 class ModelRunner:
-  def __init__(self, model: DecoderModel, cache: CacheManager):
+  def __init__(self, model: DecoderModel, cache: CacheManager, use_graphs: bool = False):
+    """use_graphs: replay steps that hold only single decoded tokens (at most 64 of them) from HIP graphs,
+    captured on demand per (batch bucket, block-table width bucket)."""
     self.model = model
     self.cache = cache
     self.device = model.ctx.device
     self.vocab_size = model.spec.vocab_size
+    self.use_graphs = use_graphs and self.device.type == "cuda"
     self._staging: Optional[torch.Tensor] = None
+    self._graphs: Dict[tuple, _DecodeGraph] = {}
 
   # ------------------------------------------------------------------ host side of a step
   def _stage(self, n: int) -> torch.Tensor:
@@ -97,10 +186,11 @@ class ModelRunner:
       self._staging = torch.empty(cap, dtype=torch.int32, pin_memory=(self.device.type == "cuda"))
     return self._staging
 
-  def build_context(self, entries: Sequence[StepEntry]):
-    """Grows the requests' page tables and lays the step out.  Returns (ctx, order, new lengths)."""
+  def _plan(self, entries: Sequence[StepEntry]):
+    """Checks the entries, grows the requests' page tables (all or nothing), and orders the entries: those
+    with several tokens first, single tokens last (stable), so kernels that treat the two kinds differently
+    get contiguous ranges.  Returns (order, q_lens, starts, kv_lens)."""
     cache = self.cache
-    P = cache.page_size
     if not entries:
       raise ValueError("a step needs at least one entry")
     seen = set()
@@ -115,79 +205,66 @@ class ModelRunner:
       for w in e.want:
         if not 0 <= w < len(e.tokens):
           raise IndexError(f"request {e.req!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
-    # multi-token entries first, single tokens last (stable), so kernels that treat the two
-    # kinds differently get contiguous ranges
+      for t in e.tokens:
+        if not 0 <= t < self.vocab_size:
+          raise ValueError(f"request {e.req!r}: token id {t} is outside [0, {self.vocab_size})")
     order = sorted(range(len(entries)), key=lambda i: 0 if len(entries[i].tokens) > 1 else 1)
-    B = len(entries)
     q_lens = [len(entries[i].tokens) for i in order]
     starts = [cache.length(entries[i].req) for i in order]
     kv_lens = [s + n for s, n in zip(starts, q_lens)]
-    T = sum(q_lens)
-    # all or nothing: check the whole step's need before any table grows
     need = sum(cache.pages_needed(entries[i].req, kv) for i, kv in zip(order, kv_lens))
     if need > cache.num_free_pages():
       from ..cache.manager import OutOfPages
       raise OutOfPages(f"step needs {need} new pages, {cache.num_free_pages()} are free")
     for i, kv in zip(order, kv_lens):
       cache.grow(entries[i].req, kv)
+    return order, q_lens, starts, kv_lens
 
-    cu_q = np.zeros(B + 1, dtype=np.int32)
-    np.cumsum(q_lens, out=cu_q[1:])
-    token_ids = np.empty(T, dtype=np.int32)
-    positions = np.empty(T, dtype=np.int32)
-    token_req = np.empty(T, dtype=np.int32)
+  def _fill(self, host, lay: _Layout, entries, order, q_lens, starts, kv_lens) -> None:
+    """Writes the step's integer arrays into `host` (views of a flat buffer laid out by `lay`).  Only the first
+    len(order) entries are written; a wider layout's tail belongs to the caller."""
+    cache = self.cache
+    P = cache.page_size
+    B, T, G, W = len(order), sum(q_lens), lay.G, lay.W
+    cu = np.zeros(B + 1, dtype=np.int64)
+    np.cumsum(q_lens, out=cu[1:])
+    host["cu_q"][:B + 1] = cu
+    host["kv_len"][:B] = kv_lens
+    tables = host["tables"].reshape(G, lay.B, W)
+    slots = host["slots"].reshape(G, lay.T)
     for b, i in enumerate(order):
-      lo, hi = cu_q[b], cu_q[b + 1]
-      token_ids[lo:hi] = np.asarray(entries[i].tokens, dtype=np.int64)
-      positions[lo:hi] = np.arange(starts[b], kv_lens[b], dtype=np.int32)
-      token_req[lo:hi] = b
-    if T and (token_ids.min() < 0 or token_ids.max() >= self.vocab_size):
-      raise ValueError(f"token id outside [0, {self.vocab_size})")
-    # logit rows in the order of the entries as given, then of `want`
-    first_row = {i: int(cu_q[b]) for b, i in enumerate(order)}
-    rows = [first_row[i] + w for i, e in enumerate(entries) for w in e.want]
-    R = len(rows)
-    req_slots = np.asarray([cache.slot(entries[i].req) for i in order], dtype=np.int32)
-
-    G = len(cache.paged)
-    W = max(1, max(-(-kv // P) for kv in kv_lens))
-    tables = np.zeros((G, B, W), dtype=np.int32)
-    slots = np.empty((G, T), dtype=np.int32)
-    for g in range(G):
-      for b, i in enumerate(order):
+      lo, hi = int(cu[b]), int(cu[b + 1])
+      host["token_ids"][lo:hi] = entries[i].tokens
+      pos = np.arange(starts[b], kv_lens[b], dtype=np.int32)
+      host["positions"][lo:hi] = pos
+      host["token_req"][lo:hi] = b
+      host["req_slots"][b] = cache.slot(entries[i].req)
+      for g in range(G):
         tab = cache.table(g, entries[i].req)
         n = min(len(tab), W)
         tables[g, b, :n] = tab[:n]
-        pos = positions[cu_q[b]:cu_q[b + 1]]
-        slots[g, cu_q[b]:cu_q[b + 1]] = tables[g, b, pos // P] * P + pos % P
+        tables[g, b, n:] = 0
+        slots[g, lo:hi] = tables[g, b, pos // P] * P + pos % P
 
-    parts = [token_ids, positions, token_req, cu_q, np.asarray(kv_lens, dtype=np.int32), req_slots,
-             np.asarray(rows, dtype=np.int32), slots.reshape(-1), tables.reshape(-1)]
-    total = sum(p.size for p in parts)
-    stage = self._stage(total)
-    host = stage.numpy()
-    offs = []
-    o = 0
-    for p in parts:
-      host[o:o + p.size] = p
-      offs.append(o)
-      o += p.size
-    dev = torch.empty(total, dtype=torch.int32, device=self.device)
-    dev.copy_(stage[:total], non_blocking=False)
-
-    ctx = StepContext()
-    ctx._cache = cache
-    ctx._device = self.device
-    ctx.num_tokens, ctx.num_requests, ctx.num_logit_rows = T, B, R
-    ctx.token_ids = dev[offs[0]:offs[0] + T]
-    ctx.positions = dev[offs[1]:offs[1] + T]
-    ctx.token_req = dev[offs[2]:offs[2] + T]
-    ctx.cu_q = dev[offs[3]:offs[3] + B + 1]
-    ctx.kv_len = dev[offs[4]:offs[4] + B]
-    ctx.req_slots = dev[offs[5]:offs[5] + B]
-    ctx.logit_rows = dev[offs[6]:offs[6] + R]
-    ctx.slots = [dev[offs[7] + g * T:offs[7] + (g + 1) * T] for g in range(G)]
-    ctx.block_tables = [dev[offs[8] + g * B * W:offs[8] + (g + 1) * B * W].view(B, W) for g in range(G)]
+  def build_context(self, entries: Sequence[StepEntry]):
+    """Grows the requests' page tables and lays the step out on the device.  Returns (ctx, order, new lengths)."""
+    cache = self.cache
+    order, q_lens, starts, kv_lens = self._plan(entries)
+    B, T = len(order), sum(q_lens)
+    # logit rows in the order of the entries as given, then of `want`
+    first = np.zeros(B, dtype=np.int64)
+    first[1:] = np.cumsum(q_lens)[:-1]
+    first_row = {i: int(first[b]) for b, i in enumerate(order)}
+    rows = [first_row[i] + w for i, e in enumerate(entries) for w in e.want]
+    W = max(1, max(-(-kv // cache.page_size) for kv in kv_lens))
+    lay = _Layout(T=T, B=B, R=len(rows), G=len(cache.paged), W=W)
+    stage = self._stage(lay.total)
+    host = lay.views(stage.numpy())
+    self._fill(host, lay, entries, order, q_lens, starts, kv_lens)
+    host["logit_rows"][:] = rows
+    dev = torch.empty(lay.total, dtype=torch.int32, device=self.device)
+    dev.copy_(stage[:lay.total], non_blocking=False)
+    ctx = lay.context(dev, cache, self.device)
     ctx.q_lens, ctx.kv_lens = q_lens, kv_lens
     ctx.num_multi = sum(1 for n in q_lens if n > 1)
     ctx.max_q_len, ctx.max_kv_len = max(q_lens), max(kv_lens)
@@ -198,8 +275,35 @@ class ModelRunner:
   def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
     """Runs the entries as one batch.  Returns float32 logits [number of wanted places, vocab] on the
     device, in the order of the entries and of each entry's `want`."""
+    if self.use_graphs and len(entries) <= _GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries):
+      return self._step_from_graph(entries)
     ctx, order, kv_lens = self.build_context(entries)
     logits = self.model.forward(ctx)
     for i, kv in zip(order, kv_lens):
       self.cache.commit(entries[i].req, kv)
     return logits
+
+  def _step_from_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    """A step of single tokens only, replayed from the graph of its batch and table-width buckets."""
+    cache = self.cache
+    order, q_lens, starts, kv_lens = self._plan(entries)     # all single tokens: order is the given order
+    B = len(entries)
+    Bb = next(b for b in _GRAPH_BATCHES if b >= B)
+    W = max(1, max(-(-kv // cache.page_size) for kv in kv_lens))
+    Wb = max(16, 1 << (W - 1).bit_length())
+    Wb = min(Wb, max(cache.max_pages_per_request, W))
+    g = self._graphs.get((Bb, Wb))
+    if g is None:
+      g = _DecodeGraph(self, Bb, Wb)
+      self._graphs[(Bb, Wb)] = g
+    self._fill(g.host, g.layout, entries, order, q_lens, starts, kv_lens)
+    g.fill_padding(B)
+    logits = g.run()
+    for i, kv in zip(order, kv_lens):
+      cache.commit(entries[i].req, kv)
+    rows = [b for b, e in enumerate(entries) for w in e.want]
+    if rows == list(range(B)):
+      return logits[:B]
+    if not rows:
+      return logits[:0]
+    return logits.index_select(0, torch.tensor(rows, dtype=torch.int64, device=self.device))

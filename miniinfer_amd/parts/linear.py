@@ -21,7 +21,21 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
   M, N = x.shape[0], weight.shape[0]
   if not x.is_cuda:
     raise ops.KernelError("miniinfer_amd runs on the GPU only")
+  if ops.gemm_skinny_supported(x, weight):
+    # few rows (decode): the time is the time to stream the weights; this library's MFMA kernel
+    return ops.gemm_skinny(x, weight, torch.empty((M, N), dtype=out_dtype, device=x.device))
   if x.dtype == torch.float32 or out_dtype != x.dtype:
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     return ops.gemm_nt(x, weight, out)
   return torch.matmul(x, weight.t())
+
+
+def silu_mul_linear(gate_up: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+  """(silu(gate) * up) @ W^T for a gate|up buffer [M, 2K]: one fused kernel for few rows, two otherwise."""
+  M, K = gate_up.shape[0], weight.shape[1]
+  if ops.gemm_skinny_supported(gate_up, weight, silu=True):
+    return ops.gemm_skinny(gate_up, weight, torch.empty((M, weight.shape[0]), dtype=gate_up.dtype,
+                                                        device=gate_up.device), silu=True)
+  act = torch.empty((M, K), dtype=gate_up.dtype, device=gate_up.device)
+  ops.silu_mul(gate_up, act)
+  return linear(act, weight)

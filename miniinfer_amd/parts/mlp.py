@@ -7,9 +7,8 @@ from typing import List, Optional
 
 import torch
 
-from ..kernels import ops
 from .base import BuildContext, ParamSpec, Part, Source, register_feed_forward
-from .linear import linear
+from .linear import linear, silu_mul_linear
 
 
 class GatedMLP(Part):
@@ -31,10 +30,7 @@ class GatedMLP(Part):
     ]
 
   def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-    gu = linear(x, self.gate_up_weight)
-    act = torch.empty((x.shape[0], self.inter), dtype=x.dtype, device=x.device)
-    ops.silu_mul(gu, act)
-    return linear(act, self.down_weight)
+    return silu_mul_linear(linear(x, self.gate_up_weight), self.down_weight)
 
 
 register_feed_forward("gated_mlp", GatedMLP)

@@ -1,0 +1,76 @@
+"""Decode steps replayed from HIP graphs give the logits of the same steps run eagerly: several replays of each
+graph, with eager prompt steps and synchronisations between them, batches that change size (so padding entries
+come and go), and block tables that grow past a width bucket."""
+
+import numpy as np
+import pytest
+import torch
+
+import tiny_models as tm
+
+pytestmark = pytest.mark.gpu
+
+
+def _runner(folder, dtype, graphs, pages=96):
+  from miniinfer_amd.cache.manager import CacheManager
+  from miniinfer_amd.engine.runner import ModelRunner
+  from miniinfer_amd.weights import load_model
+  dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
+  model, _ = load_model(str(folder), dt, "cuda:0")
+  cache = CacheManager(model.cache_needs(), page_size=16, num_pages=pages, max_requests=8,
+                       max_model_len=model.spec.max_positions, dtype=dt, device="cuda:0")
+  return ModelRunner(model, cache, use_graphs=graphs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(tmp_path, dtype):
+  from miniinfer_amd.engine.runner import StepEntry
+  cfg, _ = tm.make_model(str(tmp_path / "m"), "C", seed=4, dtype=torch.bfloat16 if dtype == "bfloat16" else torch.float32,
+                         std=0.05)
+  runners = [_runner(tmp_path / "m", dtype, graphs=False), _runner(tmp_path / "m", dtype, graphs=True)]
+  prompts = {r: tm.random_tokens(cfg, n, seed=n) for r, n in (("a", 250), ("b", 3), ("c", 40), ("d", 17), ("e", 9))}
+  stream = {r: tm.random_tokens(cfg, 40, seed=100 + len(p)) for r, p in prompts.items()}
+  outs = [[], []]
+  for k, rn in enumerate(runners):
+    live = []
+
+    def start(r):
+      rn.cache.admit(r)
+      outs[k].append(rn.step([StepEntry(r, prompts[r], [len(prompts[r]) - 1])]).float().cpu())   # eager prompt step
+      live.append(r)
+
+    start("a"); start("b")
+    for t in range(30):
+      if t == 3: start("c")
+      if t == 5: start("d"); start("e")
+      if t == 12:
+        rn.cache.release("b"); live.remove("b")
+      if t == 20:
+        rn.cache.release("d"); live.remove("d")
+      lg = rn.step([StepEntry(r, [stream[r][t]], [0]) for r in live])       # single tokens only: graph path
+      torch.cuda.synchronize()
+      outs[k].append(lg.float().cpu())
+    # request "a" crossed from 250 to 280 tokens: its table grew from 16 to 18 pages, past the 16-page bucket
+    assert rn.cache.length("a") == 280
+  assert len(runners[1]._graphs) >= 3 and not runners[0]._graphs
+  tol = 1e-5 if dtype == "float32" else 2e-2
+  for e, g in zip(*outs):
+    assert e.shape == g.shape
+    scale = float(e.abs().max())
+    assert float((e - g).abs().max()) <= tol * max(scale, 1.0)
+
+
+def test_engine_generates_the_same_with_and_without_graphs(tmp_path):
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, _ = tm.make_model(str(tmp_path / "m"), "B", seed=6, dtype=torch.float32, std=0.05)
+  prompts = [tm.random_tokens(cfg, n, seed=n) for n in (4, 31, 18)]
+  sps = [SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True),
+         SamplingParams(temperature=0.9, max_tokens=25, ignore_eos=True, seed=3),
+         SamplingParams(temperature=0.7, top_k=20, top_p=0.9, max_tokens=14, ignore_eos=True, seed=5)]
+  res = []
+  for eager in (True, False):
+    with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, num_pages=64, max_num_seqs=4,
+                   enforce_eager=eager) as eng:
+      res.append([o["token_ids"] for o in eng.generate(prompts, sps, use_tqdm=False)])
+      assert bool(eng.runner._graphs) == (not eager)
+  assert res[0] == res[1]

@@ -306,3 +306,33 @@ def test_mfma_attention_finds_a_far_key_and_respects_the_window_edge():
   assert (out[0, :d].float() - vp[page, 0, :, off].float()).abs().max() > 0.5
   run(kv - far)              # just inside
   torch.testing.assert_close(out[0, :d].float(), vp[page, 0, :, off].float(), rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (8, 4096, 1024), (16, 1024, 3072), (17, 500, 80), (64, 6144, 1024),
+                                   (3, 151936, 256), (33, 48, 2048), (5, 130, 88), (64, 1000, 40)])
+def test_gemm_skinny(M, N, K, out_dtype):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(9)
+  a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+  w = (torch.randn(N, K, generator=g) * 0.1).bfloat16().to(DEV)
+  out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+  ops.gemm_skinny(a, w, out)
+  want = a.double() @ w.double().T
+  if out_dtype == torch.float32:
+    torch.testing.assert_close(out.double(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)
+  else:
+    torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 1024, 3072), (1, 80, 112), (40, 96, 160)])
+def test_gemm_skinny_with_fused_silu_mul(M, N, K):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(10)
+  gu = torch.randn(M, 2 * K, generator=g).bfloat16().to(DEV)
+  w = (torch.randn(N, K, generator=g) * 0.1).bfloat16().to(DEV)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+  ops.gemm_skinny(gu, w, out, silu=True)
+  act = (torch.nn.functional.silu(gu.float()[:, :K]) * gu.float()[:, K:]).bfloat16()
+  want = act.double() @ w.double().T
+  torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
