@@ -292,27 +292,62 @@ __global__ __launch_bounds__(64) void decode_split_kernel(
 }
 
 // out[token of entry e][head] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s
-__global__ void decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                    uint16_t* __restrict__ out, int64_t out_row_stride, const int* __restrict__ cu_q,
-                                    int first_entry, int nq, int num_splits) {
+// One wave per (entry, head).  The lanes first share out the splits (maximum, weights, sum), then the dims;
+// the loads of a phase do not depend on one another, so they are all in flight together.
+__global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part_o,
+                                                          const float* __restrict__ part_ml,
+                                                          uint16_t* __restrict__ out, int64_t out_row_stride,
+                                                          const int* __restrict__ cu_q, int first_entry, int nq,
+                                                          int num_splits) {
+  const int lane = threadIdx.x;
   const int e = blockIdx.x / nq, head = blockIdx.x % nq;
   const int64_t base = ((int64_t)e * nq + head) * num_splits;
+  constexpr int MAXR = 16;                       // 64 * 16 = 1024 splits at most
+  float mv[MAXR], lv[MAXR];
   float M = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
-  float L = 0.f;
-  for (int s = 0; s < num_splits; ++s) {
-    const float m = part_ml[(base + s) * 2];
-    if (m != -INFINITY) L += expf(m - M) * part_ml[(base + s) * 2 + 1];
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    const int s = lane + 64 * r;
+    const bool ok = s < num_splits;
+    const float2 ml = ok ? *reinterpret_cast<const float2*>(part_ml + (base + s) * 2) : float2{-INFINITY, 0.f};
+    mv[r] = ml.x;
+    lv[r] = ml.y;
+    M = fmaxf(M, ml.x);
+    if (64 * (r + 1) >= num_splits) break;
   }
+  M = wave_max(M);
+  float L = 0.f;
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    mv[r] = (mv[r] == -INFINITY) ? 0.f : expf(mv[r] - M);   // now the split's weight
+    L += mv[r] * lv[r];
+    if (64 * (r + 1) >= num_splits) break;
+  }
+  L = wave_sum(L);
   const float inv = 1.f / L;
   uint16_t* o = out + (int64_t)cu_q[first_entry + e] * out_row_stride + (int64_t)head * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < num_splits; ++s) {
-      const float m = part_ml[(base + s) * 2];
-      if (m != -INFINITY) acc += expf(m - M) * part_o[(base + s) * D + d];
+  // dims: 4 per lane and round; every lane runs every round (the shuffles below need all lanes)
+#pragma unroll
+  for (int round = 0; round < (D + 255) / 256; ++round) {
+    const int dd = 256 * round + 4 * lane;
+    const bool live = dd < D;
+    const int d0 = live ? dd : 0;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      const int n = min(64, num_splits - 64 * r);
+#pragma unroll 8
+      for (int j = 0; j < n; ++j) {
+        const float w = __shfl(mv[r], j, 64);
+        const f32x4 v = *reinterpret_cast<const f32x4*>(part_o + (base + 64 * r + j) * D + d0);
+        acc[0] += w * v[0];
+        acc[1] += w * v[1];
+        acc[2] += w * v[2];
+        acc[3] += w * v[3];
+      }
+      if (64 * (r + 1) >= num_splits) break;
     }
-    o[d] = float_to_bf16_bits(acc * inv);
+    if (live) *reinterpret_cast<s16x4*>(o + d0) = pack_bf16x4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
   }
 }
 

@@ -34,8 +34,9 @@ __device__ __forceinline__ bf16x8 silu_mul8(const uint16_t* gate, const uint16_t
   for (int i = 0; i < 4; ++i) {
     const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
     const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
-    r.h[2 * i] = float_to_bf16_bits(g0 / (1.f + expf(-g0)) * u0);
-    r.h[2 * i + 1] = float_to_bf16_bits(g1 / (1.f + expf(-g1)) * u1);
+    // hardware exp and reciprocal (about 1 ulp each): the result is rounded to bfloat16 anyway
+    r.h[2 * i] = float_to_bf16_bits(g0 * __builtin_amdgcn_rcpf(1.f + __expf(-g0)) * u0);
+    r.h[2 * i + 1] = float_to_bf16_bits(g1 * __builtin_amdgcn_rcpf(1.f + __expf(-g1)) * u1);
   }
   return r.v;
 }

@@ -171,6 +171,85 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   if (threadIdx.x == 0) out[r] = a.i < V ? a.i : 0;
 }
 
+// ---------------------------------------------------------------- rows without top_k / top_p: the vocabulary in parts
+// Stage 1: block (part, row) finds the best (value, index) of its part of the vocabulary, value = logit for a greedy
+// row and logit / T + Gumbel noise for a sampled one.  Stage 2: one wave per row picks the best part.
+#define PART_THREADS 256
+#define PART_ELEMS 4096
+
+__global__ __launch_bounds__(PART_THREADS) void sample_parts_kernel(
+    const float* __restrict__ logits, int64_t row_stride, int V, const float* __restrict__ temperature,
+    const uint64_t* __restrict__ seeds, const int64_t* __restrict__ steps, float* __restrict__ part_val,
+    int* __restrict__ part_idx) {
+  __shared__ ArgMax scratch[PART_THREADS / MI_WAVE];
+  const int r = blockIdx.y, part = blockIdx.x, nparts = gridDim.x;
+  const float* row = logits + (int64_t)r * row_stride;
+  const float temp = temperature ? temperature[r] : 0.f;
+  const bool greedy = !(temp > 0.f);
+  const float inv_t = greedy ? 1.f : 1.f / temp;
+  const uint64_t seed = seeds ? seeds[r] : 0;
+  const uint64_t step = steps ? (uint64_t)steps[r] : 0;
+  const int begin = part * PART_ELEMS;
+  const int end = min(V, begin + PART_ELEMS);
+  ArgMax a = {-INFINITY, V};
+  for (int i = begin + threadIdx.x; i < end; i += PART_THREADS) {
+    float x = row[i];
+    if (!greedy) x = x * inv_t - logf(-logf(uniform01(seed, step, (uint64_t)i)));
+    a = better(a, ArgMax{x, i});
+  }
+  const int lane = threadIdx.x & (MI_WAVE - 1), wave = threadIdx.x / MI_WAVE;
+#pragma unroll
+  for (int o = MI_WAVE / 2; o > 0; o >>= 1) {
+    ArgMax b;
+    b.v = __shfl_xor(a.v, o, MI_WAVE);
+    b.i = __shfl_xor(a.i, o, MI_WAVE);
+    a = better(a, b);
+  }
+  if (lane == 0) scratch[wave] = a;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < PART_THREADS / MI_WAVE; ++w) a = better(a, scratch[w]);
+    part_val[(int64_t)r * nparts + part] = a.v;
+    part_idx[(int64_t)r * nparts + part] = a.i;
+  }
+}
+
+__global__ __launch_bounds__(MI_WAVE) void sample_pick_kernel(const float* __restrict__ part_val,
+                                                              const int* __restrict__ part_idx, int nparts, int V,
+                                                              int* __restrict__ out) {
+  const int r = blockIdx.x;
+  ArgMax a = {-INFINITY, V};
+  for (int p = threadIdx.x; p < nparts; p += MI_WAVE)
+    a = better(a, ArgMax{part_val[(int64_t)r * nparts + p], part_idx[(int64_t)r * nparts + p]});
+#pragma unroll
+  for (int o = MI_WAVE / 2; o > 0; o >>= 1) {
+    ArgMax b;
+    b.v = __shfl_xor(a.v, o, MI_WAVE);
+    b.i = __shfl_xor(a.i, o, MI_WAVE);
+    a = better(a, b);
+  }
+  if (threadIdx.x == 0) out[r] = a.i < V ? a.i : 0;
+}
+
+MI_EXPORT int mi_sample_parts_count(int V) { return (V + PART_ELEMS - 1) / PART_ELEMS; }
+
+// Greedy and plain temperature rows (no top_k, no top_p).  part_val / part_idx: scratch of R * mi_sample_parts_count(V).
+MI_EXPORT int mi_sample_simple(const float* logits, int64_t row_stride, int R, int V, const float* temperature,
+                               const uint64_t* seeds, const int64_t* steps, float* part_val, int* part_idx, int* out,
+                               hipStream_t stream) {
+  MI_REQUIRE(R >= 0 && V > 0 && row_stride >= V, "sample: bad sizes R=%d V=%d stride=%lld", R, V, (long long)row_stride);
+  MI_REQUIRE(R <= 65535, "sample: %d rows are too many for one launch", R);
+  MI_REQUIRE(part_val && part_idx, "sample: no scratch");
+  if (R == 0) return 0;
+  const int nparts = (V + PART_ELEMS - 1) / PART_ELEMS;
+  sample_parts_kernel<<<dim3(nparts, R), PART_THREADS, 0, stream>>>(logits, row_stride, V, temperature, seeds, steps,
+                                                                    part_val, part_idx);
+  MI_CHECK_LAUNCH("sample parts");
+  sample_pick_kernel<<<R, MI_WAVE, 0, stream>>>(part_val, part_idx, nparts, V, out);
+  MI_CHECK_LAUNCH("sample pick");
+  return 0;
+}
+
 MI_EXPORT int mi_sample(const float* logits, int64_t row_stride, int R, int V, const float* temperature,
                         const int* top_k, const float* top_p, const uint64_t* seeds, const int64_t* steps, int* out,
                         hipStream_t stream) {

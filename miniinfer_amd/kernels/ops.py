@@ -104,6 +104,9 @@ _SIGS["gemm_skinny"] = {
 
 _SIGS["sampling"] = {
   "mi_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+  "mi_sample_simple": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                       c_void_p],
+  "mi_sample_parts_count": [c_int],
 }
 
 _libs = {}
@@ -348,6 +351,14 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_k: Opt
       raise KernelError(f"sample: {name} must be int64 [R]")
   _i32("out", out, R)
   lib = _lib("sampling")
+  if top_k is None and top_p is None:
+    # greedy and plain temperature rows: the vocabulary is searched in parts by many workgroups
+    nparts = lib.mi_sample_parts_count(V)
+    part_val = torch.empty(R * nparts, dtype=torch.float32, device=logits.device)
+    part_idx = torch.empty(R * nparts, dtype=torch.int32, device=logits.device)
+    _check(lib, lib.mi_sample_simple(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature),
+                                     _ptr(seeds), _ptr(steps), _ptr(part_val), _ptr(part_idx), _ptr(out), _stream()))
+    return out
   _check(lib, lib.mi_sample(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, _ptr(temperature), _ptr(top_k),
                             _ptr(top_p), _ptr(seeds), _ptr(steps), _ptr(out), _stream()))
   return out
