@@ -104,71 +104,97 @@ struct State {
   f32x4 o[NB][DBLK];  // O^T accumulators: dims 16 blk + 4 (lane / 16) + i of column lane % 16
 };
 
-// One pass over the keys [key_begin, key_end) in tiles of 16 (key_begin a multiple of 16).
-// pos_hi[nb] / pos_lo[nb]: the last and first key the lane's column of block nb may see (pos_hi < 0: none).
-template <int NB>
-__device__ __forceinline__ void attend(State<NB>& st, const QRegs (&q)[NB], const Geometry& geo, int key_begin,
-                                       int key_end, const int (&pos_lo)[NB], const int (&pos_hi)[NB]) {
+// The cache operands of one tile of 16 keys in the lane's MFMA slots.
+struct TileRegs {
+  bf16x8 ka[QSTEPS];
+  s16x4 va[DBLK];
+};
+
+// Page ids of the tile that starts at key j0 (addresses clamped to the request's last key: masked keys read
+// valid memory of the request).
+__device__ __forceinline__ void tile_pages(const Geometry& geo, int j0, int& kk, int& vk, int& kpage, int& vpage) {
+  const int lane = threadIdx.x & 63;
+  const int last = geo.kv_len - 1;
+  kk = j0 + (lane & 15);
+  kk = kk > last ? last : kk;
+  vk = j0 + 4 * (lane >> 4);
+  vk = vk > last ? (last & ~3) : vk;
+  kpage = geo.bt[kk >> geo.page_shift];
+  vpage = geo.bt[vk >> geo.page_shift];
+}
+
+__device__ __forceinline__ void tile_load(TileRegs& t, const Geometry& geo, int kk, int vk, int kpage, int vpage) {
   const int lane = threadIdx.x & 63;
   const int P = 1 << geo.page_shift;
-  const int last = geo.kv_len - 1;
-  for (int j0 = key_begin; j0 < key_end; j0 += 16) {
-    // ---- operands from the cache (addresses clamped to the request's last key: masked keys read valid memory)
-    int kk = j0 + (lane & 15);
-    kk = kk > last ? last : kk;
-    const int64_t kpage = geo.bt[kk >> geo.page_shift];
-    const uint16_t* krow = geo.k_pages + ((kpage * geo.nkv + geo.g) * P + (kk & (P - 1))) * D;
-    bf16x8 ka[QSTEPS];
-    load_row(ka, krow, true);
-    int vk = j0 + 4 * (lane >> 4);
-    vk = vk > last ? (last & ~3) : vk;
-    const int64_t vpage = geo.bt[vk >> geo.page_shift];
-    const uint16_t* vbase = geo.v_pages + ((vpage * geo.nkv + geo.g) * D + (lane & 15)) * P + (vk & (P - 1));
-    s16x4 va[DBLK];
+  const uint16_t* krow = geo.k_pages + (((int64_t)kpage * geo.nkv + geo.g) * P + (kk & (P - 1))) * D;
+  load_row(t.ka, krow, true);
+  const uint16_t* vbase = geo.v_pages + (((int64_t)vpage * geo.nkv + geo.g) * D + (lane & 15)) * P + (vk & (P - 1));
 #pragma unroll
-    for (int blk = 0; blk < DBLK; ++blk) va[blk] = *reinterpret_cast<const s16x4*>(vbase + (int64_t)16 * blk * P);
+  for (int blk = 0; blk < DBLK; ++blk) t.va[blk] = *reinterpret_cast<const s16x4*>(vbase + (int64_t)16 * blk * P);
+}
 
+// Scores, running softmax and the value product of one tile whose operands are in `t`.
+template <int NB>
+__device__ __forceinline__ void tile_compute(State<NB>& st, const QRegs (&q)[NB], const TileRegs& t, float scale, int j0,
+                                             const int (&pos_lo)[NB], const int (&pos_hi)[NB]) {
+  const int lane = threadIdx.x & 63;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int nb = 0; nb < NB; ++nb) {
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int k = 0; k < QSTEPS; ++k) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[k], q[nb].full[k], s, 0, 0, 0);
-      // lane holds S^T[key j0 + 4 (lane / 16) + i][column lane % 16]
-      const int kbase = j0 + 4 * (lane >> 4);
-      float sv[4];
-      float tmax = -INFINITY;
+    for (int k = 0; k < QSTEPS; ++k) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.ka[k], q[nb].full[k], s, 0, 0, 0);
+    // lane holds S^T[key j0 + 4 (lane / 16) + i][column lane % 16]
+    const int kbase = j0 + 4 * (lane >> 4);
+    float sv[4];
+    float tmax = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = kbase + i;
-        const bool ok = key <= pos_hi[nb] && key >= pos_lo[nb];
-        sv[i] = ok ? s[i] * geo.scale : -INFINITY;
-        tmax = fmaxf(tmax, sv[i]);
-      }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(st.m[nb], tmax);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a column that has seen no key yet
-      const float alpha = expf(st.m[nb] - m_use);               // exp(-inf) = 0 on the first visible tile
-      float p[4];
-      float psum = 0.f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[i] = expf(sv[i] - m_use);                             // exp(-inf) = 0 for masked keys
-        psum += p[i];
-      }
-      st.l[nb] = st.l[nb] * alpha + psum;
-      st.m[nb] = m_new;
-      const s16x4 pb = pack_bf16x4(p[0], p[1], p[2], p[3]);
-#pragma unroll
-      for (int blk = 0; blk < DBLK; ++blk) {
-        f32x4 o = st.o[nb][blk];
-        o[0] *= alpha;
-        o[1] *= alpha;
-        o[2] *= alpha;
-        o[3] *= alpha;
-        st.o[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[blk], pb, o, 0, 0, 0);
-      }
+    for (int i = 0; i < 4; ++i) {
+      const int key = kbase + i;
+      const bool ok = key <= pos_hi[nb] && key >= pos_lo[nb];
+      sv[i] = ok ? s[i] * scale : -INFINITY;
+      tmax = fmaxf(tmax, sv[i]);
     }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(st.m[nb], tmax);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a column that has seen no key yet
+    const float alpha = expf(st.m[nb] - m_use);               // exp(-inf) = 0 on the first visible tile
+    float p[4];
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = expf(sv[i] - m_use);                             // exp(-inf) = 0 for masked keys
+      psum += p[i];
+    }
+    st.l[nb] = st.l[nb] * alpha + psum;
+    st.m[nb] = m_new;
+    const s16x4 pb = pack_bf16x4(p[0], p[1], p[2], p[3]);
+#pragma unroll
+    for (int blk = 0; blk < DBLK; ++blk) {
+      f32x4 o = st.o[nb][blk];
+      o[0] *= alpha;
+      o[1] *= alpha;
+      o[2] *= alpha;
+      o[3] *= alpha;
+      st.o[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.va[blk], pb, o, 0, 0, 0);
+    }
+  }
+}
+
+// One pass over the tiles of 16 keys that start at key_begin, key_begin + stride, ... below key_end
+// (key_begin a multiple of 16, stride a multiple of 16).
+// pos_hi[nb] / pos_lo[nb]: the last and first key the lane's column of block nb may see (pos_hi < 0: none).
+// (Running the loads a tile ahead of the arithmetic by hand was measured and gained nothing: the waves of a
+// compute unit already overlap one another's loads.)
+template <int NB>
+__device__ __forceinline__ void attend(State<NB>& st, const QRegs (&q)[NB], const Geometry& geo, int key_begin,
+                                       int key_end, int stride, const int (&pos_lo)[NB], const int (&pos_hi)[NB]) {
+  for (int j0 = key_begin; j0 < key_end; j0 += stride) {
+    TileRegs t;
+    int kk, vk, kpage, vpage;
+    tile_pages(geo, j0, kk, vk, kpage, vpage);
+    tile_load(t, geo, kk, vk, kpage, vpage);
+    tile_compute<NB>(st, q, t, geo.scale, j0, pos_lo, pos_hi);
   }
 }
 
@@ -223,7 +249,7 @@ __global__ __launch_bounds__(256) void prefill_kernel(
 
   State<NB> st;
   init_state<NB>(st);
-  attend<NB>(st, qr, geo, lo & ~15, last_pos + 1, pos_lo, pos_hi);
+  attend<NB>(st, qr, geo, lo & ~15, last_pos + 1, 16, pos_lo, pos_hi);
 
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
@@ -244,13 +270,25 @@ __global__ __launch_bounds__(256) void prefill_kernel(
 }
 
 // ---------------------------------------------------------------- decode: one new token per entry, keys split
-// Grid (num_splits, nkv, entries).  Partials: part_o [entries, nq, num_splits, D], part_ml [entries, nq, num_splits, 2].
-__global__ __launch_bounds__(64) void decode_split_kernel(
-    const uint16_t* __restrict__ q, int64_t q_row_stride, const uint16_t* __restrict__ k_pages,
-    const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
-    const int* __restrict__ cu_q, const int* __restrict__ kv_len, int first_entry, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int nq, int nkv, int page_shift, float scale, int window) {
+// Grid (num_splits, nkv, entries), 4 waves per workgroup.  The tiles of a split go round-robin to the waves, which
+// combine their running softmax states through LDS.  With one split the workgroup writes the output itself;
+// with several it writes a partial (max, sum, unnormalised output) per head, and the merge kernel below
+// combines the partials with the log-sum-exp rule.  (Merging inside this kernel, by the workgroup that
+// finishes last, was measured: the device-wide fences it needs cost many times the second launch.)
+// Partials: part_o [entries, nq, num_splits, D], part_ml [entries, nq, num_splits, 2].
+// (2 waves for the largest head sizes, whose states would not fit 64 KB of LDS fourfold)
+constexpr int DECODE_WAVES = D > 128 ? 2 : 4;
+
+__global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
+    const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
+    const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
+    int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int first_entry,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv, int page_shift, float scale, int window) {
+  __shared__ float lds_o[DECODE_WAVES][DBLK][64][4];
+  __shared__ float lds_m[DECODE_WAVES][16];
+  __shared__ float lds_l[DECODE_WAVES][16];
   const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   const int split = blockIdx.x, num_splits = gridDim.x;
   const int g = blockIdx.y;
   const int e = blockIdx.z;             // entry index among the decode entries
@@ -268,26 +306,60 @@ __global__ __launch_bounds__(64) void decode_split_kernel(
   State<1> st;
   init_state<1>(st);
   const bool col_ok = (lane & 15) < G;
-  if (t0 < t1) {
+  {
     Geometry geo{k_pages, v_pages, block_table + (int64_t)b * table_width, nkv, g, page_shift, kv, scale};
     QRegs qr[1];
     load_queries<1>(qr, q + (int64_t)cu_q[b] * q_row_stride, q_row_stride, 0, 16, G, 1, g * G);
     const int pos_lo[1] = {lo};
     const int pos_hi[1] = {col_ok ? pos : -1};
-    attend<1>(st, qr, geo, t0 << 4, t1 << 4, pos_lo, pos_hi);
+    attend<1>(st, qr, geo, (t0 + wave) << 4, t1 << 4, 16 * DECODE_WAVES, pos_lo, pos_hi);
   }
+  // ---- combine the waves: every wave leaves its state in LDS
   float l = st.l[0];
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
-  if (!col_ok) return;
-  const int head = g * G + (lane & 15);
-  const int64_t slot = ((int64_t)e * nq + head) * num_splits + split;
-  float* po = part_o + slot * D + 4 * (lane >> 4);
 #pragma unroll
-  for (int blk = 0; blk < DBLK; ++blk) *reinterpret_cast<f32x4*>(po + 16 * blk) = st.o[0][blk];
-  if ((lane >> 4) == 0) {
-    part_ml[slot * 2] = st.m[0];
-    part_ml[slot * 2 + 1] = l;
+  for (int blk = 0; blk < DBLK; ++blk) *reinterpret_cast<f32x4*>(&lds_o[wave][blk][lane][0]) = st.o[0][blk];
+  if (lane < 16) {
+    lds_m[wave][lane] = st.m[0];
+    lds_l[wave][lane] = l;
+  }
+  __syncthreads();
+  // thread -> (block of dims, lane slot): column c = slot % 16, dims 16 blk + 4 (slot / 16) + i
+  for (int idx = threadIdx.x; idx < DBLK * 64; idx += blockDim.x) {
+    const int blk = idx >> 6, slot = idx & 63;
+    const int c = slot & 15;
+    if (c >= G) continue;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DECODE_WAVES; ++w) M = fmaxf(M, lds_m[w][c]);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < DECODE_WAVES; ++w) {
+      const float mw = lds_m[w][c];
+      const float wt = (mw == -INFINITY) ? 0.f : expf(mw - M);
+      const f32x4 v = *reinterpret_cast<const f32x4*>(&lds_o[w][blk][slot][0]);
+      acc[0] += wt * v[0];
+      acc[1] += wt * v[1];
+      acc[2] += wt * v[2];
+      acc[3] += wt * v[3];
+      L += wt * lds_l[w][c];
+    }
+    const int head = g * G + c;
+    const int dim = 16 * blk + 4 * (slot >> 4);
+    if (num_splits == 1) {
+      const float inv = 1.f / L;
+      uint16_t* o = out + (int64_t)cu_q[b] * out_row_stride + (int64_t)head * D + dim;
+      *reinterpret_cast<s16x4*>(o) = pack_bf16x4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
+    } else {
+      const int64_t ps = ((int64_t)e * nq + head) * num_splits + split;
+      *reinterpret_cast<f32x4*>(part_o + ps * D + dim) = acc;
+      if (blk == 0 && (slot >> 4) == 0) {
+        part_ml[ps * 2] = M;
+        part_ml[ps * 2 + 1] = L;
+      }
+    }
   }
 }
 
@@ -302,7 +374,7 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   const int lane = threadIdx.x;
   const int e = blockIdx.x / nq, head = blockIdx.x % nq;
   const int64_t base = ((int64_t)e * nq + head) * num_splits;
-  constexpr int MAXR = 16;                       // 64 * 16 = 1024 splits at most
+  constexpr int MAXR = 16;
   float mv[MAXR], lv[MAXR];
   float M = -INFINITY;
 #pragma unroll
@@ -319,14 +391,13 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   float L = 0.f;
 #pragma unroll
   for (int r = 0; r < MAXR; ++r) {
-    mv[r] = (mv[r] == -INFINITY) ? 0.f : expf(mv[r] - M);   // now the split's weight
+    mv[r] = (mv[r] == -INFINITY) ? 0.f : expf(mv[r] - M);
     L += mv[r] * lv[r];
     if (64 * (r + 1) >= num_splits) break;
   }
   L = wave_sum(L);
   const float inv = 1.f / L;
   uint16_t* o = out + (int64_t)cu_q[first_entry + e] * out_row_stride + (int64_t)head * D;
-  // dims: 4 per lane and round; every lane runs every round (the shuffles below need all lanes)
 #pragma unroll
   for (int round = 0; round < (D + 255) / 256; ++round) {
     const int dd = 256 * round + 4 * lane;
@@ -412,15 +483,18 @@ MI_EXPORT int mi_attn_decode(const void* q, int64_t q_row_stride, void* out, int
   MI_REQUIRE(num_entries >= 0 && first_entry >= 0 && window >= 0, "attn_decode: bad entry range or window");
   MI_REQUIRE(num_splits >= 1 && num_splits <= 1024, "attn_decode: %d splits", num_splits);
   MI_REQUIRE(num_entries <= 65535 && nkv <= 65535, "attn_decode: grid too large");
-  MI_REQUIRE(part_o && part_ml, "attn_decode: no partial buffers");
+  MI_REQUIRE(num_splits == 1 || (part_o && part_ml), "attn_decode: no partial buffers");
   if (num_entries == 0) return 0;
   dim3 grid(num_splits, nkv, num_entries);
-  decode_split_kernel<<<grid, 64, 0, stream>>>((const uint16_t*)q, q_row_stride, (const uint16_t*)k_pages,
-                                               (const uint16_t*)v_pages, block_table, table_width, cu_q, kv_len,
-                                               first_entry, part_o, part_ml, nq, nkv, log2_of(page_size), scale, window);
-  MI_CHECK_LAUNCH("attn_decode split");
-  decode_merge_kernel<<<num_entries * nq, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q,
-                                                           first_entry, nq, num_splits);
-  MI_CHECK_LAUNCH("attn_decode merge");
+  decode_kernel<<<grid, 64 * DECODE_WAVES, 0, stream>>>(
+      (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
+      (const uint16_t*)v_pages, block_table, table_width, cu_q, kv_len, first_entry, part_o, part_ml, nq, nkv,
+      log2_of(page_size), scale, window);
+  MI_CHECK_LAUNCH("attn_decode");
+  if (num_splits > 1) {
+    decode_merge_kernel<<<num_entries * nq, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q,
+                                                             first_entry, nq, num_splits);
+    MI_CHECK_LAUNCH("attn_decode merge");
+  }
   return 0;
 }

@@ -74,6 +74,76 @@ __global__ void add_rmsnorm_kernel(const TX* __restrict__ x, float* __restrict__
   }
 }
 
+// The same with every value held in registers: one read of x, residual and w (all loads issued together), one
+// reduction, one write.  Each thread takes CH chunks of 4 consecutive elements; N must be a multiple of 4.
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load4(const bf16* p, float (&v)[4]) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
+  *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+}
+__device__ __forceinline__ void store4(bf16* p, const float (&v)[4]) {
+  uint2 t;
+  t.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+  t.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = t;
+}
+
+template <typename TX, typename TY, int CH>
+__global__ void add_rmsnorm_reg_kernel(const TX* __restrict__ x, float* __restrict__ residual,
+                                       const float* __restrict__ w, TY* __restrict__ y, const int* __restrict__ rows,
+                                       int N, float eps, int write_back) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const int64_t s = rows ? rows[i] : i;
+  const TX* xr = x ? x + s * N : nullptr;
+  float* rr = residual ? residual + s * N : nullptr;
+  TY* yr = y + (int64_t)i * N;
+  float v[CH][4], wv[CH][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = 4 * (threadIdx.x + c * blockDim.x);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[c][j] = 0.f, wv[c][j] = 0.f;
+    if (e < N) {
+      if (rr) load4(rr + e, v[c]);
+      if (xr) {
+        float t[4];
+        load4(xr + e, t);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[c][j] += t[j];
+      }
+      load4(w + e, wv[c]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = 4 * (threadIdx.x + c * blockDim.x);
+    if (write_back && e < N) store4(rr + e, v[c]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ss += v[c][j] * v[c][j];
+  }
+  ss = block_sum(ss, scratch);
+  const float rstd = rsqrtf(ss / (float)N + eps);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = 4 * (threadIdx.x + c * blockDim.x);
+    if (e < N) {
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = v[c][j] * rstd * wv[c][j];
+      store4(yr + e, o);
+    }
+  }
+}
+
 // x_dtype: dtype of x (ignored when x is null); y_dtype: dtype of y.
 MI_EXPORT int mi_add_rmsnorm(int x_dtype, int y_dtype, const void* x, float* residual, const float* w, void* y,
                              const int* rows, int M, int N, float eps, int write_back, hipStream_t stream) {
@@ -82,11 +152,24 @@ MI_EXPORT int mi_add_rmsnorm(int x_dtype, int y_dtype, const void* x, float* res
   MI_REQUIRE(!(write_back && rows), "add_rmsnorm: write_back with a row selection is not defined");
   MI_REQUIRE(!(write_back && !residual), "add_rmsnorm: write_back without a residual");
   if (M == 0) return 0;
-  const int threads = N >= 2048 ? 512 : (N >= 512 ? 256 : (N >= 128 ? 128 : 64));
-#define LAUNCH(TX, TY)                                                                                       \
-  add_rmsnorm_kernel<TX, TY><<<M, threads, 0, stream>>>((const TX*)x, residual, w, (TY*)y, rows, N, eps, \
-                                                        write_back)
   if (!x) x_dtype = MI_DTYPE_F32;
+  // rows of up to 16384 elements, a multiple of 4: everything in registers; otherwise two passes over the row
+  const int chunks = N / 4;
+  const bool regs = (N % 4 == 0) && chunks <= 4 * 1024;
+  const int ch = chunks <= 1024 ? (chunks <= 256 ? 1 : (chunks <= 512 ? 2 : 4)) : 4;
+  const int rthreads = regs ? (((chunks + ch - 1) / ch + 63) / 64) * 64 : 0;
+  const int threads = N >= 2048 ? 512 : (N >= 512 ? 256 : (N >= 128 ? 128 : 64));
+#define LAUNCH(TX, TY)                                                                                         \
+  do {                                                                                                         \
+    if (regs && ch == 1)                                                                                       \
+      add_rmsnorm_reg_kernel<TX, TY, 1><<<M, rthreads, 0, stream>>>((const TX*)x, residual, w, (TY*)y, rows, N, eps, write_back); \
+    else if (regs && ch == 2)                                                                                  \
+      add_rmsnorm_reg_kernel<TX, TY, 2><<<M, rthreads, 0, stream>>>((const TX*)x, residual, w, (TY*)y, rows, N, eps, write_back); \
+    else if (regs)                                                                                             \
+      add_rmsnorm_reg_kernel<TX, TY, 4><<<M, rthreads, 0, stream>>>((const TX*)x, residual, w, (TY*)y, rows, N, eps, write_back); \
+    else                                                                                                       \
+      add_rmsnorm_kernel<TX, TY><<<M, threads, 0, stream>>>((const TX*)x, residual, w, (TY*)y, rows, N, eps, write_back); \
+  } while (0)
   if (x_dtype == MI_DTYPE_F32 && y_dtype == MI_DTYPE_F32) LAUNCH(float, float);
   else if (x_dtype == MI_DTYPE_BF16 && y_dtype == MI_DTYPE_BF16) LAUNCH(bf16, bf16);
   else if (x_dtype == MI_DTYPE_F32 && y_dtype == MI_DTYPE_BF16) LAUNCH(float, bf16);
@@ -170,45 +253,58 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_strid
   }
   if (h >= nq + nkv) return;
 
+  // every load that does not depend on another is issued first: the head's elements as rotation pairs
+  // (j, j + half) and the pass-through tail, the norm weights, the position
   const float* w = (h < nq) ? qw : kw;
-  float rstd = 1.f;
-  if (w) {
-    float ss = 0.f;
-    for (int e = lane; e < d; e += MI_WAVE) {
-      const float v = to_float(src[e]);
-      ss += v * v;
-    }
-    ss = wave_sum(ss);
-    rstd = rsqrtf(ss / (float)d + eps);
-  }
-  const int half = cos_sin ? rotary_dim / 2 : 0;
   const int rd = cos_sin ? rotary_dim : 0;
+  const int half = rd / 2;
   int pos = positions ? positions[t] : 0;
   pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+  float x1[2], x2[2], w1[2], w2[2];      // pairs lane, lane + 64 (half <= 128)
+  float xt[4], wt[4];                    // tail elements rd + lane + 64 c (d <= 256)
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int j = lane + 64 * c;
+    const bool ok = j < half;
+    x1[c] = ok ? to_float(src[j]) : 0.f;
+    x2[c] = ok ? to_float(src[j + half]) : 0.f;
+    w1[c] = (ok && w) ? w[j] : 1.f;
+    w2[c] = (ok && w) ? w[j + half] : 1.f;
+    ss += x1[c] * x1[c] + x2[c] * x2[c];
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int e = rd + lane + 64 * c;
+    const bool ok = e < d;
+    xt[c] = ok ? to_float(src[e]) : 0.f;
+    wt[c] = (ok && w) ? w[e] : 1.f;
+    ss += xt[c] * xt[c];
+  }
+  float rstd = 1.f;
+  if (w) rstd = rsqrtf(wave_sum(ss) / (float)d + eps);
   const float* cs = cos_sin ? cos_sin + (int64_t)pos * rotary_dim : nullptr;
-
-  for (int e = lane; e < d; e += MI_WAVE) {
-    if (e < half) {
-      const int e2 = e + half;
-      float x1 = to_float(src[e]) * rstd;
-      float x2 = to_float(src[e2]) * rstd;
-      if (w) {
-        x1 *= w[e];
-        x2 *= w[e2];
-      }
-      const float c = cs[e], s = cs[half + e];
-      const T o1 = from_float<T>(x1 * c - x2 * s);
-      const T o2 = from_float<T>(x2 * c + x1 * s);
-      src[e] = o1;
-      src[e2] = o2;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int j = lane + 64 * c;
+    if (j < half) {
+      const float cv = cs[j], sv = cs[half + j];
+      const float a = x1[c] * rstd * w1[c], b = x2[c] * rstd * w2[c];
+      const T o1 = from_float<T>(a * cv - b * sv);
+      const T o2 = from_float<T>(b * cv + a * sv);
+      src[j] = o1;
+      src[j + half] = o2;
       if (dst) {
-        dst[e] = o1;
-        dst[e2] = o2;
+        dst[j] = o1;
+        dst[j + half] = o2;
       }
-    } else if (e >= rd) {
-      float x1 = to_float(src[e]) * rstd;
-      if (w) x1 *= w[e];
-      const T o = from_float<T>(x1);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int e = rd + lane + 64 * c;
+    if (e < d) {
+      const T o = from_float<T>(xt[c] * rstd * wt[c]);
       src[e] = o;
       if (dst) dst[e] = o;
     }
@@ -220,6 +316,7 @@ MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, in
                                     int rotary_dim, int max_pos, const int* positions, void* k_pages, void* v_pages,
                                     const int* slots, int page_size, hipStream_t stream) {
   MI_REQUIRE(num_tokens >= 0 && nq > 0 && nkv > 0 && d > 0, "qk_norm_rope_cache: bad sizes");
+  MI_REQUIRE(d <= 256, "qk_norm_rope_cache: head size %d; this kernel takes at most 256", d);
   MI_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qk_norm_rope_cache: row stride %lld too small",
              (long long)row_stride);
   MI_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0, "qk_norm_rope_cache: page size %d is no power of two",

@@ -7,9 +7,9 @@
 // fill the other operand.  A workgroup owns 16 * RB weight rows; its waves split K and add their partial
 // blocks through LDS.  32-bit accumulation; the result is stored as bfloat16 or float32.
 //
-// With SILU the left operand is made on the fly from a gate|up buffer [M, 2K]:
-// a[m, k] = bf16( silu(gate[m, k]) * up[m, k] ), the feed-forward's activation
-// (kernels/triton/silu_mul.py:33-37 of the reference) fused into the down projection.
+// With GATE_UP, W is a fused gate|up matrix [2 N, K] (gate rows first) and the result is the feed-forward's
+// activation C[m, n] = silu(A W_gate^T)[m, n] * (A W_up^T)[m, n] (kernels/triton/silu_mul.py:33-37 of the
+// reference), made from the 32-bit sums of gate row n and up row n, which the same workgroup owns.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -22,26 +22,9 @@ __device__ __forceinline__ bf16x8 zero_bf16x8() {
   return z;
 }
 
-__device__ __forceinline__ bf16x8 silu_mul8(const uint16_t* gate, const uint16_t* up) {
-  const uint4 g = *reinterpret_cast<const uint4*>(gate);
-  const uint4 u = *reinterpret_cast<const uint4*>(up);
-  const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
-  union {
-    bf16x8 v;
-    uint16_t h[8];
-  } r;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
-    const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
-    // hardware exp and reciprocal (about 1 ulp each): the result is rounded to bfloat16 anyway
-    r.h[2 * i] = float_to_bf16_bits(g0 * __builtin_amdgcn_rcpf(1.f + __expf(-g0)) * u0);
-    r.h[2 * i + 1] = float_to_bf16_bits(g1 * __builtin_amdgcn_rcpf(1.f + __expf(-g1)) * u1);
-  }
-  return r.v;
-}
+__device__ __forceinline__ float silu_f(float g) { return g / (1.f + expf(-g)); }
 
-template <int MB, int RB, bool OUT_F32, bool SILU>
+template <int MB, int RB, bool OUT_F32, bool GATE_UP>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __restrict__ A, int64_t lda,
                                                            const uint16_t* __restrict__ W, int64_t ldw,
                                                            void* __restrict__ C, int64_t ldc, int M, int N, int K) {
@@ -49,7 +32,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
-  const int n0 = blockIdx.x * 16 * RB;
+  // GATE_UP: RB == 2, row block 0 = gate rows n0.., row block 1 = up rows N + n0..; N counts output columns
+  const int n0 = GATE_UP ? blockIdx.x * 16 : blockIdx.x * 16 * RB;
   const int steps = (K + 31) / 32;
   const int spw = (steps + nw - 1) / nw;
   const int s_begin = wave * spw;
@@ -64,8 +48,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   const uint16_t* wrow[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    int row = n0 + 16 * rb + (lane & 15);
+    int row = GATE_UP ? n0 + (lane & 15) : n0 + 16 * rb + (lane & 15);
     row = row < N ? row : N - 1;            // rows past the end read the last row; they are never stored
+    if (GATE_UP && rb == 1) row += N;
     wrow[rb] = W + (int64_t)row * ldw;
   }
   const uint16_t* arow[MB];
@@ -77,30 +62,43 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     arow[mb] = A + (int64_t)(mok[mb] ? m : 0) * lda;
   }
 
-#pragma unroll 4
-  for (int s = s_begin; s < s_end; ++s) {
-    const int k = 32 * s + 8 * (lane >> 4);
-    const bool kok = k < K;                 // K is a multiple of 8: a lane's 8 elements are all in or all out
-    bf16x8 w[RB], a[MB];
+  // Steps are taken CH at a time: first every load of the chunk is issued (weights, and the raw left operand),
+  // then the operands are converted and multiplied, so one memory round trip covers CH steps.
+  constexpr int CH = MB == 1 ? 8 : (MB == 2 ? 4 : 2);   // what fits the 128 registers of a 16-wave workgroup
+  for (int s0 = s_begin; s0 < s_end; s0 += CH) {
+    bf16x8 w[CH][RB];
+    uint4 ar[CH][MB];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) w[rb] = kok ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
+    for (int c = 0; c < CH; ++c) {
+      const int k = 32 * (s0 + c) + 8 * (lane >> 4);
+      const bool kok = (s0 + c < s_end) && k < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      if (kok && mok[mb]) {
-        if (SILU) a[mb] = silu_mul8(arow[mb] + k, arow[mb] + K + k);
-        else a[mb] = *reinterpret_cast<const bf16x8*>(arow[mb] + k);
-      } else {
-        a[mb] = zero_bf16x8();
+      for (int rb = 0; rb < RB; ++rb) w[c][rb] = kok ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const bool ok = kok && mok[mb];
+        ar[c][mb] = ok ? *reinterpret_cast<const uint4*>(arow[mb] + k) : uint4{0, 0, 0, 0};
       }
     }
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+    for (int c = 0; c < CH; ++c) {
+      if (s0 + c >= s_end) break;
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[rb], a[mb], acc[rb][mb], 0, 0, 0);
+      for (int mb = 0; mb < MB; ++mb) {
+        union {
+          uint4 u;
+          bf16x8 v;
+        } a;
+        a.u = ar[c][mb];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+          acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[c][rb], a.v, acc[rb][mb], 0, 0, 0);
+      }
+    }
   }
 
   // lane holds C^T[n0 + 16 rb + 4 (lane / 16) + i][16 mb + lane % 16]
+  constexpr int OB = GATE_UP ? MB : RB * MB;          // output blocks of the workgroup
   if (nw > 1) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
@@ -109,12 +107,16 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         *reinterpret_cast<f32x4*>(red + ((wave * RB * MB + rb * MB + mb) * 64 + lane) * 4) = acc[rb][mb];
     __syncthreads();
     // element e of the workgroup's result: block e / 256, lane (e % 256) / 4, register e % 4
-    for (int e = threadIdx.x; e < RB * MB * 256; e += blockDim.x) {
+    for (int e = threadIdx.x; e < OB * 256; e += blockDim.x) {
       const int blk = e >> 8, r = e & 255;
-      float v = 0.f;
-      for (int w = 0; w < nw; ++w) v += red[(w * RB * MB + blk) * 256 + r];
+      float v = 0.f, u = 0.f;
+      for (int w = 0; w < nw; ++w) {
+        v += red[(w * RB * MB + blk) * 256 + r];
+        if (GATE_UP) u += red[(w * RB * MB + MB + blk) * 256 + r];
+      }
+      if (GATE_UP) v = silu_f(v) * u;
       const int ln = r >> 2, i = r & 3;
-      const int n = n0 + 16 * (blk / MB) + 4 * (ln >> 4) + i;
+      const int n = n0 + 16 * (GATE_UP ? 0 : blk / MB) + 4 * (ln >> 4) + i;
       const int m = 16 * (blk % MB) + (ln & 15);
       if (n < N && m < M) {
         if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n] = v;
@@ -123,57 +125,68 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     }
   } else {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+    for (int ob = 0; ob < OB; ++ob) {
+      const int rb = GATE_UP ? 0 : ob / MB, mb = ob % MB;
+      const int m = 16 * mb + (lane & 15);
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const int m = 16 * mb + (lane & 15);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int n = n0 + 16 * rb + 4 * (lane >> 4) + i;
-          if (n < N && m < M) {
-            if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n] = acc[rb][mb][i];
-            else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n] = float_to_bf16_bits(acc[rb][mb][i]);
-          }
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 16 * rb + 4 * (lane >> 4) + i;
+        float v = acc[rb][mb][i];
+        if (GATE_UP) v = silu_f(v) * acc[GATE_UP ? 1 : 0][mb][i];
+        if (n < N && m < M) {
+          if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n] = v;
+          else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n] = float_to_bf16_bits(v);
         }
       }
+    }
   }
 }
 
 template <int MB, int RB>
-static int launch(bool out_f32, bool silu, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
-                  int M, int N, int K, int waves, hipStream_t stream) {
-  const dim3 grid((N + 16 * RB - 1) / (16 * RB));
+static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                  int64_t ldc, int M, int N, int K, int waves, hipStream_t stream) {
+  const dim3 grid(gate_up ? (N + 15) / 16 : (N + 16 * RB - 1) / (16 * RB));
   const dim3 block(64 * waves);
   const size_t lds = waves > 1 ? (size_t)waves * RB * MB * 256 * sizeof(float) : 0;
-#define GO(F32, SILU)                                                                                              \
-  gemm_skinny_kernel<MB, RB, F32, SILU><<<grid, block, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, \
-                                                                      ldw, C, ldc, M, N, K)
-  if (out_f32 && silu) GO(true, true);
-  else if (out_f32) GO(true, false);
-  else if (silu) GO(false, true);
-  else GO(false, false);
+#define GO(F32, GU)                                                                                              \
+  gemm_skinny_kernel<MB, RB, F32, GU><<<grid, block, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, \
+                                                                    ldw, C, ldc, M, N, K)
+  if (gate_up) {
+    if constexpr (RB == 2) {
+      if (out_f32) GO(true, true);
+      else GO(false, true);
+    }
+  } else {
+    if (out_f32) GO(true, false);
+    else GO(false, false);
+  }
 #undef GO
   return 0;
 }
 
-// A [M, K] (or, with silu, the gate|up buffer [M, 2K]), W [N, K], C [M, N] bfloat16 or float32.
-MI_EXPORT int mi_gemm_skinny(int out_f32, int silu, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+// Tuning knob for experiments: waves per workgroup (0 = chosen from the shape).
+static int g_waves_override = 0;
+MI_EXPORT void mi_gemm_skinny_set_waves(int waves) { g_waves_override = waves; }
+
+// A [M, K], C [M, N] bfloat16 or float32; W [N, K], or with gate_up the fused matrix [2 N, K].
+MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                              int64_t ldc, int M, int N, int K, hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);
   MI_REQUIRE(lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: row strides (%lld, %lld) must be multiples of 8", (long long)lda,
              (long long)ldw);
-  MI_REQUIRE(lda >= (silu ? 2 * (int64_t)K : K) && ldw >= K && ldc >= N, "gemm_skinny: leading dimensions too small");
+  MI_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_skinny: leading dimensions too small");
   if (M == 0) return 0;
   const int row_blocks = (N + 15) / 16;
-  const int RB = row_blocks >= 1024 ? 2 : 1;
-  const int groups = (row_blocks + RB - 1) / RB;
+  const int RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
+  const int groups = gate_up ? row_blocks : (row_blocks + RB - 1) / RB;
   const int steps = (K + 31) / 32;
   // enough waves to fill the chip, at least 2 steps of K per wave, at most 16 waves per workgroup
   int waves = (4096 + groups - 1) / groups;
   if (waves > 16) waves = 16;
   if (waves > steps / 2) waves = steps / 2;
   if (waves < 1) waves = 1;
+  if (g_waves_override > 0) waves = g_waves_override;
   const int MB = (M + 15) / 16;
   size_t lds = waves > 1 ? (size_t)waves * RB * MB * 1024 : 0;
   while (lds > 64 * 1024 && waves > 1) {     // the default LDS allotment of a workgroup
@@ -182,7 +195,7 @@ MI_EXPORT int mi_gemm_skinny(int out_f32, int silu, const void* A, int64_t lda, 
   }
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \
-    launch<mb, rb>(out_f32 != 0, silu != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, stream);                \
+    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, stream);              \
     MI_CHECK_LAUNCH("gemm_skinny");                                                                           \
     return 0;                                                                                                 \
   }

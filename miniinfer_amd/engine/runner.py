@@ -73,11 +73,12 @@ class StepContext:
       self._work[tokens_per_block] = w
     return w
 
-  def scratch(self, name: str, numel: int, dtype: torch.dtype) -> torch.Tensor:
-    """A device buffer that lives for this step (reused by every layer that asks under the same name)."""
+  def scratch(self, name: str, numel: int, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
+    """A device buffer that lives for this step (reused by every layer that asks under the same name).
+    zero: the buffer is all zero when it is made, and every user leaves it all zero."""
     t = self._scratch.get(name)
     if t is None or t.numel() < numel or t.dtype != dtype:
-      t = torch.empty(numel, dtype=dtype, device=self._device)
+      t = (torch.zeros if zero else torch.empty)(numel, dtype=dtype, device=self._device)
       self._scratch[name] = t
     return t
 

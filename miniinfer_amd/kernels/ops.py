@@ -273,28 +273,33 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor
 SKINNY_MAX_ROWS = 64
 
 
-def gemm_skinny_supported(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> bool:
+def gemm_skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
   K = w.shape[1]
   return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_MAX_ROWS and K % 8 == 0
           and a.stride(1) == 1 and w.stride(1) == 1 and (a.shape[0] <= 1 or a.stride(0) % 8 == 0)
-          and (w.shape[0] <= 1 or w.stride(0) % 8 == 0) and a.shape[1] == (2 * K if silu else K)
+          and (w.shape[0] <= 1 or w.stride(0) % 8 == 0) and a.shape[1] == K
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, silu: bool = False) -> torch.Tensor:
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bool = False) -> torch.Tensor:
   """out[M, N] = a[M, K] @ w[N, K]^T on the matrix cores for M <= 64 rows, bfloat16 operands, bfloat16 or float32
-  result.  With `silu`, a is a gate|up buffer [M, 2K] and the left operand is bf16(silu(gate) * up)."""
+  result.  With `gate_up`, w is a fused gate|up matrix [2 N, K] (gate rows first) and
+  out = silu(a @ w_gate^T) * (a @ w_up^T), made from the 32-bit sums."""
   _dev(a, w, out)
-  if not gemm_skinny_supported(a, w, silu):
+  if not gemm_skinny_supported(a, w):
     raise KernelError(f"gemm_skinny does not take a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}")
   M = a.shape[0]
   N, K = w.shape
+  if gate_up:
+    if N % 2:
+      raise KernelError("gemm_skinny: a gate|up matrix has an even number of rows")
+    N //= 2
   if tuple(out.shape) != (M, N) or out.stride(1) != 1 or out.dtype not in (torch.bfloat16, torch.float32):
     raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit [{M}, {N}]")
   lib = _lib("gemm_skinny")
-  _check(lib, lib.mi_gemm_skinny(1 if out.dtype == torch.float32 else 0, 1 if silu else 0, _ptr(a),
-                                 a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0) if N > 1 else K,
-                                 _ptr(out), out.stride(0) if M > 1 else N, M, N, K, _stream()))
+  _check(lib, lib.mi_gemm_skinny(1 if out.dtype == torch.float32 else 0, 1 if gate_up else 0, _ptr(a),
+                                 a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), _ptr(out),
+                                 out.stride(0) if M > 1 else N, M, N, K, _stream()))
   return out
 
 

@@ -90,10 +90,10 @@ class PagedAttention(Part):
 
 
 def decode_splits(num_head_entries: int, max_keys: int, target_waves: int = 2048) -> int:
-  """Into how many key ranges a decoding request is cut: enough waves to fill the chip, at least 4 tiles of 16
-  keys each."""
+  """Into how many key ranges (workgroups of 4 waves) a decoding request is cut: enough waves to fill the chip,
+  at least 4 tiles of 16 keys per range."""
   tiles = -(-max_keys // 16)
-  want = -(-target_waves // max(1, num_head_entries))
+  want = -(-target_waves // max(1, 4 * num_head_entries))     # up to 4 waves per workgroup
   return int(max(1, min(want, max(1, tiles // 4), 256)))
 
 

@@ -30,12 +30,13 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
   return torch.matmul(x, weight.t())
 
 
-def silu_mul_linear(gate_up: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-  """(silu(gate) * up) @ W^T for a gate|up buffer [M, 2K]: one fused kernel for few rows, two otherwise."""
-  M, K = gate_up.shape[0], weight.shape[1]
-  if ops.gemm_skinny_supported(gate_up, weight, silu=True):
-    return ops.gemm_skinny(gate_up, weight, torch.empty((M, weight.shape[0]), dtype=gate_up.dtype,
-                                                        device=gate_up.device), silu=True)
-  act = torch.empty((M, K), dtype=gate_up.dtype, device=gate_up.device)
-  ops.silu_mul(gate_up, act)
-  return linear(act, weight)
+def gate_up_activation(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+  """silu(x Wg^T) * (x Wu^T) for a fused gate|up matrix [2 I, K]: one kernel for few rows (the activation is made
+  from the 32-bit sums in the product's epilogue), product and activation kernels otherwise."""
+  M, inter = x.shape[0], gate_up_weight.shape[0] // 2
+  if ops.gemm_skinny_supported(x, gate_up_weight):
+    return ops.gemm_skinny(x, gate_up_weight, torch.empty((M, inter), dtype=x.dtype, device=x.device), gate_up=True)
+  gu = linear(x, gate_up_weight)
+  act = torch.empty((M, inter), dtype=x.dtype, device=x.device)
+  ops.silu_mul(gu, act)
+  return act

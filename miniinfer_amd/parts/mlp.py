@@ -8,7 +8,7 @@ from typing import List, Optional
 import torch
 
 from .base import BuildContext, ParamSpec, Part, Source, register_feed_forward
-from .linear import linear, silu_mul_linear
+from .linear import gate_up_activation, linear
 
 
 class GatedMLP(Part):
@@ -30,7 +30,7 @@ class GatedMLP(Part):
     ]
 
   def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-    return silu_mul_linear(linear(x, self.gate_up_weight), self.down_weight)
+    return linear(gate_up_activation(x, self.gate_up_weight), self.down_weight)
 
 
 register_feed_forward("gated_mlp", GatedMLP)

@@ -325,14 +325,14 @@ def test_gemm_skinny(M, N, K, out_dtype):
     torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 1024, 3072), (1, 80, 112), (40, 96, 160)])
-def test_gemm_skinny_with_fused_silu_mul(M, N, K):
+@pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 112, 80), (40, 160, 96), (64, 100, 256)])
+def test_gemm_skinny_gate_up_activation(M, I, K):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(10)
-  gu = torch.randn(M, 2 * K, generator=g).bfloat16().to(DEV)
-  w = (torch.randn(N, K, generator=g) * 0.1).bfloat16().to(DEV)
-  out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-  ops.gemm_skinny(gu, w, out, silu=True)
-  act = (torch.nn.functional.silu(gu.float()[:, :K]) * gu.float()[:, K:]).bfloat16()
-  want = act.double() @ w.double().T
+  x = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+  w = (torch.randn(2 * I, K, generator=g) * 0.1).bfloat16().to(DEV)
+  out = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+  ops.gemm_skinny(x, w, out, gate_up=True)
+  gu = x.double() @ w.double().T
+  want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
   torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
