@@ -142,6 +142,154 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   }
 }
 
+// ---------------------------------------------------------------- residual add + RMS norm + product, fused
+// For up to 16 rows:  r' = r + x   (x optional; r' is written to a second buffer, each workgroup a share of it)
+//                     C  = ( rmsnorm(r') * w ) W^T
+// The norm needs no pass of its own: the left operand is bf16(r' * w), the sum of squares of each row is
+// gathered beside the products (every workgroup sees whole rows, its waves split K), and the row's
+// rsqrt(mean + eps) scales the 32-bit result.  `rows` (optional) picks the rows of r and x.
+template <int RB, bool GATE_UP>
+__global__ __launch_bounds__(512) void norm_gemm_kernel(const float* __restrict__ R, const uint16_t* __restrict__ X,
+                                                        float* __restrict__ R_out, const float* __restrict__ NW,
+                                                        const int* __restrict__ rows, float eps,
+                                                        const uint16_t* __restrict__ W, int64_t ldw,
+                                                        uint16_t* __restrict__ C, int64_t ldc, int M, int N, int K) {
+  extern __shared__ float red[];   // [waves][RB][256] sums, then [waves][16] squares
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int n0 = GATE_UP ? blockIdx.x * 16 : blockIdx.x * 16 * RB;
+  const int steps = (K + 31) / 32;
+  const int spw = (steps + nw - 1) / nw;
+  const int s_begin = wave * spw;
+  const int s_end = min(steps, s_begin + spw);
+  float* red_ss = red + nw * RB * 256;
+
+  f32x4 acc[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) acc[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const uint16_t* wrow[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    int row = GATE_UP ? n0 + (lane & 15) : n0 + 16 * rb + (lane & 15);
+    row = row < N ? row : N - 1;
+    if (GATE_UP && rb == 1) row += N;
+    wrow[rb] = W + (int64_t)row * ldw;
+  }
+  const int m = lane & 15;
+  const bool mok = m < M;
+  const int64_t src = mok ? (rows ? rows[m] : m) : 0;
+  const float* rrow = R + src * K;
+  const uint16_t* xrow = X ? X + src * K : nullptr;
+  float* orow = R_out ? R_out + (int64_t)(mok ? m : 0) * K : nullptr;
+  float ss = 0.f;
+
+  constexpr int CH = 4;
+  for (int s0 = s_begin; s0 < s_end; s0 += CH) {
+    bf16x8 w[CH][RB];
+    float4 r0[CH], r1[CH], g0[CH], g1[CH];
+    uint4 xr[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int k = 32 * (s0 + c) + 8 * (lane >> 4);
+      const bool kok = (s0 + c < s_end) && k < K;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) w[c][rb] = kok ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
+      const bool ok = kok && mok;
+      r0[c] = ok ? *reinterpret_cast<const float4*>(rrow + k) : float4{0.f, 0.f, 0.f, 0.f};
+      r1[c] = ok ? *reinterpret_cast<const float4*>(rrow + k + 4) : float4{0.f, 0.f, 0.f, 0.f};
+      xr[c] = (ok && xrow) ? *reinterpret_cast<const uint4*>(xrow + k) : uint4{0, 0, 0, 0};
+      g0[c] = kok ? *reinterpret_cast<const float4*>(NW + k) : float4{0.f, 0.f, 0.f, 0.f};
+      g1[c] = kok ? *reinterpret_cast<const float4*>(NW + k + 4) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      if (s0 + c >= s_end) break;
+      const int k = 32 * (s0 + c) + 8 * (lane >> 4);
+      float v[8] = {r0[c].x, r0[c].y, r0[c].z, r0[c].w, r1[c].x, r1[c].y, r1[c].z, r1[c].w};
+      const uint32_t xw[4] = {xr[c].x, xr[c].y, xr[c].z, xr[c].w};
+      const float gw[8] = {g0[c].x, g0[c].y, g0[c].z, g0[c].w, g1[c].x, g1[c].y, g1[c].z, g1[c].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] += __uint_as_float(xw[i] << 16);
+        v[2 * i + 1] += __uint_as_float(xw[i] & 0xffff0000u);
+      }
+      union {
+        bf16x8 v8;
+        uint16_t h[8];
+      } a;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        ss += v[i] * v[i];
+        a.h[i] = float_to_bf16_bits(v[i] * gw[i]);
+      }
+      // this workgroup's share of the new residual: the steps s with s % gridDim.x == blockIdx.x
+      if (orow && mok && k < K && ((s0 + c) % gridDim.x) == blockIdx.x) {
+        *reinterpret_cast<float4*>(orow + k) = float4{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<float4*>(orow + k + 4) = float4{v[4], v[5], v[6], v[7]};
+      }
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[c][rb], a.v8, acc[rb], 0, 0, 0);
+    }
+  }
+  // squares: the 4 lanes that share a row, then the waves
+  ss += __shfl_xor(ss, 16, 64);
+  ss += __shfl_xor(ss, 32, 64);
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) *reinterpret_cast<f32x4*>(red + ((wave * RB + rb) * 64 + lane) * 4) = acc[rb];
+  if (lane < 16) red_ss[wave * 16 + lane] = ss;
+  __syncthreads();
+  constexpr int OB = GATE_UP ? 1 : RB;
+  for (int e = threadIdx.x; e < OB * 256; e += blockDim.x) {
+    const int blk = e >> 8, r = e & 255;
+    const int ln = r >> 2, i = r & 3;
+    const int mm = ln & 15;
+    float v = 0.f, u = 0.f, sq = 0.f;
+    for (int w = 0; w < nw; ++w) {
+      v += red[(w * RB + blk) * 256 + r];
+      if (GATE_UP) u += red[(w * RB + 1) * 256 + r];
+      sq += red_ss[w * 16 + mm];
+    }
+    const float rstd = rsqrtf(sq / (float)K + eps);
+    v *= rstd;
+    if (GATE_UP) v = silu_f(v) * (u * rstd);
+    const int n = n0 + 16 * blk + 4 * (ln >> 4) + i;
+    if (n < N && mm < M) C[(int64_t)mm * ldc + n] = float_to_bf16_bits(v);
+  }
+}
+
+// R [*, K] float32 residual, X [*, K] bfloat16 or null, R_out [M, K] float32 or null (written when given),
+// NW [K] float32 norm weight, rows [M] or null, W [N, K] (gate_up: [2 N, K]) bfloat16, C [M, N] bfloat16.
+MI_EXPORT int mi_norm_gemm_skinny(int gate_up, const float* R, const void* X, float* R_out, const float* NW,
+                                  const int* rows, float eps, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
+                                  int N, int K, hipStream_t stream) {
+  MI_REQUIRE(M >= 0 && M <= 16, "norm_gemm_skinny: M=%d; this kernel takes at most 16 rows", M);
+  MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && ldw % 8 == 0 && ldw >= K && ldc >= N, "norm_gemm_skinny: N=%d K=%d ldw=%lld",
+             N, K, (long long)ldw);
+  MI_REQUIRE(R && NW && W && C, "norm_gemm_skinny: missing operand");
+  MI_REQUIRE(!(rows && R_out), "norm_gemm_skinny: a row selection cannot update the residual");
+  if (M == 0) return 0;
+  const int row_blocks = (N + 15) / 16;
+  const int RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
+  const int groups = gate_up ? row_blocks : (row_blocks + RB - 1) / RB;
+  const int steps = (K + 31) / 32;
+  int waves = (4096 + groups - 1) / groups;
+  if (waves > 8) waves = 8;
+  if (waves > steps / 2) waves = steps / 2;
+  if (waves < 1) waves = 1;
+  const size_t lds = ((size_t)waves * RB * 256 + waves * 16) * sizeof(float);
+  const dim3 grid(groups), block(64 * waves);
+#define GO(rb, GU)                                                                                                  \
+  norm_gemm_kernel<rb, GU><<<grid, block, lds, stream>>>(R, (const uint16_t*)X, R_out, NW, rows, eps,               \
+                                                         (const uint16_t*)W, ldw, (uint16_t*)C, ldc, M, N, K)
+  if (gate_up) GO(2, true);
+  else if (RB == 2) GO(2, false);
+  else GO(1, false);
+#undef GO
+  MI_CHECK_LAUNCH("norm_gemm_skinny");
+  return 0;
+}
+
 template <int MB, int RB>
 static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                   int64_t ldc, int M, int N, int K, int waves, hipStream_t stream) {

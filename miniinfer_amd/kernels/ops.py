@@ -102,6 +102,9 @@ _SIGS["gemm_skinny"] = {
                      c_void_p],
 }
 
+_SIGS["gemm_skinny"]["mi_norm_gemm_skinny"] = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                               c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]
+
 _SIGS["sampling"] = {
   "mi_sample": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
   "mi_sample_simple": [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -300,6 +303,46 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bo
   _check(lib, lib.mi_gemm_skinny(1 if out.dtype == torch.float32 else 0, 1 if gate_up else 0, _ptr(a),
                                  a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), _ptr(out),
                                  out.stride(0) if M > 1 else N, M, N, K, _stream()))
+  return out
+
+
+NORM_GEMM_MAX_ROWS = 16
+
+
+def norm_gemm_supported(num_rows: int, residual: torch.Tensor, x: Optional[torch.Tensor], w: torch.Tensor) -> bool:
+  K = w.shape[1]
+  return (w.dtype == torch.bfloat16 and num_rows <= NORM_GEMM_MAX_ROWS and K % 8 == 0 and residual.shape[-1] == K
+          and residual.dtype == torch.float32 and residual.is_contiguous() and w.stride(1) == 1
+          and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0 and residual.data_ptr() % 16 == 0
+          and (x is None or (x.dtype == torch.bfloat16 and x.is_contiguous() and x.shape == residual.shape
+                             and x.data_ptr() % 16 == 0)))
+
+
+def norm_gemm_skinny(residual: torch.Tensor, x: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float,
+                     w: torch.Tensor, out: torch.Tensor, residual_out: Optional[torch.Tensor] = None,
+                     rows: Optional[torch.Tensor] = None, gate_up: bool = False) -> torch.Tensor:
+  """For up to 16 rows, in one kernel: r' = residual + x (x may be None); out = (rmsnorm(r') * norm_weight) @ w^T,
+  or with `gate_up` silu(.. @ w_gate^T) * (.. @ w_up^T) for a fused gate|up matrix.  r' is written to
+  `residual_out` (another buffer than `residual`) when given.  `rows` picks rows of residual and x instead."""
+  _dev(residual, x, norm_weight, w, out, residual_out, rows)
+  M = rows.numel() if rows is not None else residual.shape[0]
+  if not norm_gemm_supported(M, residual, x, w):
+    raise KernelError("norm_gemm_skinny does not take these operands")
+  N, K = w.shape
+  if gate_up:
+    N //= 2
+  _f32("norm_weight", norm_weight, K)
+  _i32("rows", rows)
+  if tuple(out.shape) != (M, N) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+    raise KernelError(f"norm_gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit [{M}, {N}] bfloat16")
+  if residual_out is not None:
+    if rows is not None or residual_out.shape != residual.shape or residual_out.dtype != torch.float32 \
+        or not residual_out.is_contiguous() or residual_out.data_ptr() == residual.data_ptr():
+      raise KernelError("norm_gemm_skinny: residual_out must be another float32 buffer of the residual's shape")
+  lib = _lib("gemm_skinny")
+  _check(lib, lib.mi_norm_gemm_skinny(1 if gate_up else 0, _ptr(residual), _ptr(x), _ptr(residual_out),
+                                      _ptr(norm_weight), _ptr(rows), float(eps), _ptr(w), w.stride(0), _ptr(out), N,
+                                      M, N, K, _stream()))
   return out
 
 

@@ -3,3 +3,4 @@ from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, BuildContext
                    register_position)
 from . import norm, position, attention, mlp, block   # registers the built-in kinds
 from .model import DecoderModel
+from .norm import DeferredNorm

@@ -18,6 +18,8 @@ from .linear import linear
 
 
 class PagedAttention(Part):
+  takes_deferred_norm = True    # the input goes straight into `linear`, which can fuse the norm
+
   def __init__(self, spec, ctx: BuildContext):
     if spec.num_heads % spec.num_kv_heads:
       raise ValueError(f"{spec.num_heads} query heads are no multiple of {spec.num_kv_heads} kv heads")
@@ -54,7 +56,7 @@ class PagedAttention(Part):
     return PagedKV(num_kv_heads=self.nkv, head_dim=self.d, window=self.window)
 
   # ------------------------------------------------------------------ one step
-  def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+  def forward(self, x, ctx, cache) -> torch.Tensor:
     T = x.shape[0]
     qkv = linear(x, self.qkv_weight)
     table = self.position.rotary_table()
@@ -64,7 +66,7 @@ class PagedAttention(Part):
       self.q_norm.weight if self.q_norm is not None else None,
       self.k_norm.weight if self.k_norm is not None else None,
       eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
-    out = torch.empty((T, self.nq * self.d), dtype=x.dtype, device=x.device)
+    out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
     self._attend(qkv, out, ctx, cache)
     return linear(out, self.o_weight)
 

@@ -30,13 +30,26 @@ class PreNormBlock(Part):
     fn = getattr(self.mixer, "cache_requirement", None)
     return fn() if fn else None
 
-  def forward(self, h: Optional[torch.Tensor], residual: torch.Tensor, ctx, cache) -> torch.Tensor:
-    """h: the previous block's pending output (None for the first block); residual [T, hidden] float32,
-    updated in place.  Returns this block's pending output."""
-    x = self.mixer_norm.forward_residual(h, residual)
-    a = self.mixer.forward(x, ctx, cache)
-    x = self.ff_norm.forward_residual(a, residual)
-    return self.feed_forward.forward(x, ctx)
+  def forward(self, h: Optional[torch.Tensor], residual: torch.Tensor, ctx, cache):
+    """h: the previous block's pending output (None for the first block); residual [T, hidden] float32.
+    Returns (this block's pending output, the residual stream), which may be a new buffer.
+
+    A part that sets `takes_deferred_norm` gets its input as a DeferredNorm and may fuse the add and the norm into
+    its own first kernel; any other part gets the normed tensor."""
+    x = self.mixer_norm.defer(h, residual)
+    if not getattr(self.mixer, "takes_deferred_norm", False):
+      x.materialize()
+    a = self.mixer.forward(x if getattr(self.mixer, "takes_deferred_norm", False) else x.value, ctx, cache)
+    if not x.consumed:
+      x.materialize()       # a mixer that ignored its input still leaves the residual updated
+    residual = x.residual
+    y = self.ff_norm.defer(a, residual)
+    if not getattr(self.feed_forward, "takes_deferred_norm", False):
+      y.materialize()
+    m = self.feed_forward.forward(y if getattr(self.feed_forward, "takes_deferred_norm", False) else y.value, ctx)
+    if not y.consumed:
+      y.materialize()
+    return m, y.residual
 
 
 register_block("prenorm", PreNormBlock)

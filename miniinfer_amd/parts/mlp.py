@@ -12,6 +12,8 @@ from .linear import gate_up_activation, linear
 
 
 class GatedMLP(Part):
+  takes_deferred_norm = True
+
   def __init__(self, spec, ctx: BuildContext):
     if spec.activation != "silu":
       raise ValueError(f"activation {spec.activation!r} is not supported, only 'silu'")
@@ -29,7 +31,7 @@ class GatedMLP(Part):
       ParamSpec("down_weight", (self.hidden, self.inter), (Source(d + ".weight", self.hidden),)),
     ]
 
-  def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+  def forward(self, x, ctx) -> torch.Tensor:
     return linear(gate_up_activation(x, self.gate_up_weight), self.down_weight)
 
 

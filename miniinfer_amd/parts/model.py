@@ -66,7 +66,7 @@ class DecoderModel(Part):
     ops.embed(self.embedding, ctx.token_ids, residual)
     h = None
     for li in self.spec.run_order:
-      h = self.blocks[li].forward(h, residual, ctx, ctx.layer_cache(self.cache_layer_of(li)))
+      h, residual = self.blocks[li].forward(h, residual, ctx, ctx.layer_cache(self.cache_layer_of(li)))
     R = ctx.num_logit_rows
     if R == 0:
       return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.ctx.device)

@@ -10,6 +10,44 @@ from ..kernels import ops
 from .base import BuildContext, ParamSpec, Part, register_norm
 
 
+class DeferredNorm:
+  """norm(residual + x) that has not been computed yet.  A consumer that can fuse the add and the norm into its
+  own first kernel takes the pieces (`linear` and `gate_up_activation` do, for few rows); any other calls
+  `materialize()`.  After either, `residual` is the updated residual stream (it may be a new buffer)."""
+
+  def __init__(self, norm: "RMSNorm", x: Optional[torch.Tensor], residual: torch.Tensor):
+    self.norm = norm
+    self.x = x
+    self.residual = residual
+    self.value: Optional[torch.Tensor] = None
+    self.consumed = False
+
+  @property
+  def shape(self):
+    return self.residual.shape
+
+  @property
+  def dtype(self):
+    return self.norm.ctx.dtype
+
+  @property
+  def device(self):
+    return self.residual.device
+
+  def materialize(self) -> torch.Tensor:
+    if self.value is None:
+      if self.consumed:
+        raise RuntimeError("a deferred norm was fused into one product and then asked for again")
+      self.value = self.norm.forward_residual(self.x, self.residual)
+      self.consumed = True
+    return self.value
+
+  def fused(self, new_residual: torch.Tensor) -> None:
+    """A consumer has done the add and the norm inside its own kernel."""
+    self.residual = new_residual
+    self.consumed = True
+
+
 class RMSNorm(Part):
   def __init__(self, spec, ctx: BuildContext):
     self.size = spec.size
@@ -24,6 +62,9 @@ class RMSNorm(Part):
     """norm(x); x [M, size] in the activation dtype or float32; result in the activation dtype."""
     out = torch.empty(x.shape, dtype=self.ctx.dtype, device=x.device)
     return ops.add_rmsnorm(x, None, self.weight, self.eps, out)
+
+  def defer(self, x: Optional[torch.Tensor], residual: torch.Tensor) -> DeferredNorm:
+    return DeferredNorm(self, x, residual)
 
   def forward_residual(self, x: Optional[torch.Tensor], residual: torch.Tensor,
                        rows: Optional[torch.Tensor] = None) -> torch.Tensor:

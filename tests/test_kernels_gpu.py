@@ -336,3 +336,33 @@ def test_gemm_skinny_gate_up_activation(M, I, K):
   gu = x.double() @ w.double().T
   want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
   torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("M,N,K,with_x,gate_up", [(8, 4096, 1024, True, False), (1, 500, 80, False, False),
+                                                   (16, 3072, 1024, True, True), (5, 112, 88, True, True),
+                                                   (3, 151936, 256, False, False)])
+def test_norm_gemm_skinny(M, N, K, with_x, gate_up):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(11)
+  r = (torch.randn(M, K, generator=g) * 2).to(DEV)
+  x = torch.randn(M, K, generator=g).bfloat16().to(DEV) if with_x else None
+  nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+  w = (torch.randn(2 * N if gate_up else N, K, generator=g) * 0.1).bfloat16().to(DEV)
+  out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+  r_out = torch.empty_like(r) if with_x else None
+  ops.norm_gemm_skinny(r, x, nw, 1e-5, w, out, residual_out=r_out, gate_up=gate_up)
+  v = r.double() + (x.double() if with_x else 0)
+  if with_x:
+    torch.testing.assert_close(r_out.double(), v, rtol=1e-6, atol=1e-6)
+  # the kernel's own rounding points: the left operand is bfloat16(r' * w); the row's rstd scales the 32-bit sums
+  rstd = torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)
+  y = ((v * nw.double()).bfloat16().double() @ w.double().T) * rstd
+  torch.testing.assert_close(y, torch.nn.functional.rms_norm(v, (K,), nw.double(), 1e-5) @ w.double().T, rtol=3e-2,
+                             atol=3e-2 * float(y.abs().max()))
+  want = torch.nn.functional.silu(y[:, :N]) * y[:, N:] if gate_up else y
+  torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
+  # rows picked by index, residual untouched
+  rows = torch.tensor([M - 1, 0], dtype=torch.int32, device=DEV)
+  out2 = torch.empty(2, N, dtype=torch.bfloat16, device=DEV)
+  ops.norm_gemm_skinny(r, x, nw, 1e-5, w, out2, rows=rows, gate_up=gate_up)
+  torch.testing.assert_close(out2.double(), want[rows.long()], rtol=1e-2, atol=1e-2)
