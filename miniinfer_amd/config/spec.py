@@ -48,6 +48,8 @@ class AttentionSpec:
   position: Any                      # RotarySpec | NoPositionSpec | another registered kind
   qk_norm: Optional[NormSpec] = None  # per-head norm of q and k before the rotation
   window: Optional[int] = None       # a query at p sees keys p-window < j <= p; None = all
+  shares_kv: bool = False            # no k/v projections of its own: reads the keys and values of the layer
+                                     # named by LayerSpec.cache_of
   # checkpoint names of the q, k, v and output projections and of the q and k norms
   tensor_names: Tuple[str, ...] = ("q_proj", "k_proj", "v_proj", "o_proj", "q_norm", "k_norm")
   kind: str = "paged_attention"
@@ -67,9 +69,9 @@ class GatedMLPSpec:
 class LayerSpec:
   """One block: a mixer and a feed-forward, each behind its own norm, on a residual stream.
 
-  `prefix` is the checkpoint-name prefix of the block's tensors.  `cache_of` lets a layer
-  read and write the cache of another layer (by index into `ModelSpec.layers`) instead of
-  owning one."""
+  `prefix` is the checkpoint-name prefix of the block's tensors.  `cache_of` lets a layer read the
+  cache of another layer (by index into `ModelSpec.layers`; the cache of that layer's first run)
+  instead of owning one."""
   prefix: str
   mixer: Any
   feed_forward: Any
@@ -87,7 +89,8 @@ class ModelSpec:
   vocab_size: int
   hidden_size: int
   layers: Tuple[LayerSpec, ...]
-  run_order: Tuple[int, ...]          # indices into `layers`; a layer may be named twice
+  run_order: Tuple[int, ...]          # indices into `layers`; a layer may be named twice (each run has a
+                                      # cache of its own unless the layer borrows one)
   final_norm: Any
   embedding_name: str = "model.embed_tokens.weight"
   final_norm_prefix: str = "model.norm."

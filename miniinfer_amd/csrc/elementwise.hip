@@ -315,7 +315,7 @@ MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, in
                                     const float* qw, const float* kw, float eps, const float* cos_sin,
                                     int rotary_dim, int max_pos, const int* positions, void* k_pages, void* v_pages,
                                     const int* slots, int page_size, hipStream_t stream) {
-  MI_REQUIRE(num_tokens >= 0 && nq > 0 && nkv > 0 && d > 0, "qk_norm_rope_cache: bad sizes");
+  MI_REQUIRE(num_tokens >= 0 && nq > 0 && nkv >= 0 && d > 0, "qk_norm_rope_cache: bad sizes");
   MI_REQUIRE(d <= 256, "qk_norm_rope_cache: head size %d; this kernel takes at most 256", d);
   MI_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qk_norm_rope_cache: row stride %lld too small",
              (long long)row_stride);

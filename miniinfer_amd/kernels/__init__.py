@@ -12,5 +12,18 @@ ALL_MODULES = [("elementwise", ()), ("gemm", ()), ("gemm_skinny", ()), ("attenti
 
 
 def build_all(force: bool = False) -> List[str]:
-  """Compile every shared object for gfx950 (all of them again when `force`)."""
-  return jit.compile_many(ALL_MODULES, force=force)
+  """Compile every shared object for gfx950 (all of them again when `force`) and drop built objects of older
+  sources from the in-tree build folder."""
+  import os
+  paths = jit.compile_many(ALL_MODULES, force=force)
+  keep = {os.path.abspath(p) for p in paths}
+  d = jit.build_dirs()[-2] if len(jit.build_dirs()) > 1 else jit.build_dirs()[0]
+  if os.path.isdir(d):
+    for fn in os.listdir(d):
+      full = os.path.abspath(os.path.join(d, fn))
+      if fn.endswith(".so") and full not in keep:
+        try:
+          os.unlink(full)
+        except OSError:
+          pass
+  return paths

@@ -34,23 +34,28 @@ class PagedAttention(Part):
     self.position = POSITIONS.build(spec.position, ctx)
     self.q_norm = NORMS.build(spec.qk_norm, ctx) if spec.qk_norm is not None else None
     self.k_norm = NORMS.build(spec.qk_norm, ctx) if spec.qk_norm is not None else None
-    self.qkv_weight: Optional[torch.Tensor] = None
+    self.shares_kv = bool(getattr(spec, "shares_kv", False))
+    self.qkv_weight: Optional[torch.Tensor] = None   # q rows only when the keys and values are borrowed
     self.o_weight: Optional[torch.Tensor] = None
 
   # ------------------------------------------------------------------ tensors
   def param_specs(self) -> List[ParamSpec]:
     qn, kn, vn, on = self.spec.tensor_names[:4]
     nq, nkv, d, H = self.nq, self.nkv, self.d, self.hidden
-    return [
-      ParamSpec("qkv_weight", ((nq + 2 * nkv) * d, H),
-                (Source(qn + ".weight", nq * d), Source(kn + ".weight", nkv * d), Source(vn + ".weight", nkv * d))),
-      ParamSpec("o_weight", (H, nq * d), (Source(on + ".weight", H),)),
-    ]
+    if self.shares_kv:
+      qkv = ParamSpec("qkv_weight", (nq * d, H), (Source(qn + ".weight", nq * d),))
+    else:
+      qkv = ParamSpec("qkv_weight", ((nq + 2 * nkv) * d, H),
+                      (Source(qn + ".weight", nq * d), Source(kn + ".weight", nkv * d), Source(vn + ".weight", nkv * d)))
+    return [qkv, ParamSpec("o_weight", (H, nq * d), (Source(on + ".weight", H),))]
 
   def children(self) -> List[Tuple[str, Part]]:
     if self.q_norm is None:
       return []
-    return [(self.spec.tensor_names[4] + ".", self.q_norm), (self.spec.tensor_names[5] + ".", self.k_norm)]
+    out = [(self.spec.tensor_names[4] + ".", self.q_norm)]
+    if not self.shares_kv:
+      out.append((self.spec.tensor_names[5] + ".", self.k_norm))
+    return out
 
   def cache_requirement(self):
     return PagedKV(num_kv_heads=self.nkv, head_dim=self.d, window=self.window)
@@ -61,11 +66,16 @@ class PagedAttention(Part):
     qkv = linear(x, self.qkv_weight)
     table = self.position.rotary_table()
     eps = self.q_norm.eps if self.q_norm is not None else 0.0
-    ops.qk_norm_rope_cache(
-      qkv, self.nq, self.nkv, self.d,
-      self.q_norm.weight if self.q_norm is not None else None,
-      self.k_norm.weight if self.k_norm is not None else None,
-      eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
+    if self.shares_kv:
+      # only queries of its own: they are normed and rotated; the borrowed pages are read, never written
+      ops.qk_norm_rope_cache(qkv, self.nq, 0, self.d, self.q_norm.weight if self.q_norm is not None else None, None,
+                             eps, table, ctx.positions, None, None, None, cache.page_size)
+    else:
+      ops.qk_norm_rope_cache(
+        qkv, self.nq, self.nkv, self.d,
+        self.q_norm.weight if self.q_norm is not None else None,
+        self.k_norm.weight if self.k_norm is not None else None,
+        eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
     out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
     self._attend(qkv, out, ctx, cache)
     return linear(out, self.o_weight)

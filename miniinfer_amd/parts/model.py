@@ -42,21 +42,28 @@ class DecoderModel(Part):
     return out
 
   def cache_needs(self) -> List[object]:
-    """Per layer: what its mixer keeps between steps; a layer that borrows another's cache keeps nothing."""
+    """Per run of `run_order`: what that run's mixer keeps between steps.  A layer that is run twice keeps a cache
+    per run; a layer that borrows another layer's cache keeps nothing."""
     needs = []
-    for ls, b in zip(self.spec.layers, self.blocks):
+    for li in self.spec.run_order:
+      ls, b = self.spec.layers[li], self.blocks[li]
       needs.append(None if ls.cache_of is not None else b.cache_requirement())
-    for i, ls in enumerate(self.spec.layers):
-      if ls.cache_of is not None:
-        if not 0 <= ls.cache_of < len(self.blocks) or self.spec.layers[ls.cache_of].cache_of is not None:
-          raise ValueError(f"layer {i} borrows the cache of layer {ls.cache_of}, which has none of its own")
-        if self.blocks[ls.cache_of].cache_requirement() != self.blocks[i].cache_requirement():
-          raise ValueError(f"layer {i} borrows the cache of layer {ls.cache_of}, whose geometry differs")
+    for li in self.spec.run_order:
+      ls = self.spec.layers[li]
+      if ls.cache_of is None:
+        continue
+      if not 0 <= ls.cache_of < len(self.blocks) or self.spec.layers[ls.cache_of].cache_of is not None:
+        raise ValueError(f"layer {li} borrows the cache of layer {ls.cache_of}, which has none of its own")
+      if ls.cache_of not in self.spec.run_order[:self.spec.run_order.index(li)]:
+        raise ValueError(f"layer {li} borrows the cache of layer {ls.cache_of}, which has not run before it")
+      if self.blocks[ls.cache_of].cache_requirement() != self.blocks[li].cache_requirement():
+        raise ValueError(f"layer {li} borrows the cache of layer {ls.cache_of}, whose geometry differs")
     return needs
 
-  def cache_layer_of(self, layer: int) -> int:
-    co = self.spec.layers[layer].cache_of
-    return layer if co is None else co
+  def cache_index(self, run: int) -> int:
+    """Which run's cache the run at position `run` of `run_order` uses."""
+    co = self.spec.layers[self.spec.run_order[run]].cache_of
+    return run if co is None else self.spec.run_order.index(co)
 
   # ------------------------------------------------------------------ one step
   def forward(self, ctx) -> torch.Tensor:
@@ -65,8 +72,8 @@ class DecoderModel(Part):
     residual = torch.empty((T, H), dtype=torch.float32, device=self.ctx.device)
     ops.embed(self.embedding, ctx.token_ids, residual)
     h = None
-    for li in self.spec.run_order:
-      h, residual = self.blocks[li].forward(h, residual, ctx, ctx.layer_cache(self.cache_layer_of(li)))
+    for run, li in enumerate(self.spec.run_order):
+      h, residual = self.blocks[li].forward(h, residual, ctx, ctx.layer_cache(self.cache_index(run)))
     R = ctx.num_logit_rows
     if R == 0:
       return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.ctx.device)
