@@ -102,6 +102,7 @@ def main() -> int:
   ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
   ap.add_argument("--eager", action="store_true")
   ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+  ap.add_argument("--only-prefill", action="store_true", help="run only the 2,048-token prefill (for profiling)")
   args = ap.parse_args()
   if args.gpus != 1:
     print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -123,6 +124,11 @@ def main() -> int:
                      num_pages=pages, max_num_seqs=max_batch, max_model_len=max_len, max_num_batched_tokens=8192,
                      enforce_eager=args.eager)
   esize = 2 if args.dtype == "bfloat16" else 4
+  if args.only_prefill:
+    psec = time_prefill(engine, 2048, reps=max(1, args.steps), seed=2)
+    print(json.dumps({"prefill": {"value": round(2048 / psec, 1), "tokens": 2048, "ms": round(psec * 1e3, 3),
+                                  "frac": round(prefill_flops(cfg, layers, 2048) / psec / PEAK_FLOPS[args.dtype], 4)}}))
+    return 0
 
   sec = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
   value = args.batch / sec
