@@ -3,19 +3,24 @@
 //
 // Same function as attention.hip (bottom-right aligned causal mask, optional window, grouped heads:
 // miniinfer/layers/attention.py:112-191), in two launches:
-//   prefill: entries with several new tokens; one wave per (kv head, block of query columns);
-//   decode:  entries with one new token; the keys of a request are split over several waves
-//            (flash-decoding), which write (max, sum, unnormalised output) partials that a merge kernel
-//            combines with the log-sum-exp rule.
+//   prefill: entries with several new tokens; a workgroup of 4 waves takes 4 blocks of query columns of one
+//            entry and kv head and shares each tile of keys and values through LDS;
+//   decode:  entries with one new token; the keys of a request are split over workgroups (flash-decoding),
+//            which write (max, sum, unnormalised output) partials that a merge kernel combines with the
+//            log-sum-exp rule.
 //
-// Layout of the products, chosen so that every operand comes straight from global memory or from the
-// previous product's accumulators, with no trip through LDS:
+// Layout of the products, chosen so that every operand comes straight from memory or from the previous
+// product's accumulators:
 //   S^T[key, col] = K[key, :] . Q[col, :]      A = K rows (16 B per lane from a key's row), B = Q rows
 //   O^T[dim, col] = V^T[dim, :] . P^T[:, col]  A = V^T rows (value pages are stored [dim][key in page]),
 //                                              B = P, which is exactly where S^T's accumulators sit
 // A "column" is a (query token, query head of the kv group) pair; 16 columns form an MFMA block.  All
 // softmax statistics of a column live in the lanes with lane % 16 == column.  Scores, softmax and
 // accumulation are 32-bit; P is rounded to bfloat16 for the second product.
+//
+// The running softmax is updated once per macro tile of MT * 16 keys (one maximum, one rescale of the output
+// accumulators, and that only when some column's maximum moved), in base 2: scores are scaled by
+// scale * log2(e), so a probability is one v_exp_f32.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -24,22 +29,27 @@
 static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256, "head size must be a multiple of 16 up to 256");
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // (arrays of HIP's uint4 class end up in scratch memory)
 
 constexpr int D = HEAD_DIM;
 constexpr int KSTEPS = D / 32;          // 16x16x32 products over the head dim
 constexpr bool KREM = (D % 32) != 0;    // plus one more, half of it zeros
+constexpr int QSTEPS = KSTEPS + (KREM ? 1 : 0);
 constexpr int DBLK = D / 16;            // 16-row blocks of O^T
+constexpr int MT = D > 128 ? 2 : 4;     // tiles of 16 keys per macro tile
+constexpr int MKEYS = 16 * MT;          // keys per macro tile
 
 // The last 16 dims of a head size that is no multiple of 32 go through the same 16x16x32 product with the
 // upper half of the contraction zeroed: lanes 0..31 hold 8 dims each, lanes 32..63 hold zeros.  (Finishing
 // the score with a 16x16x16 product on the accumulator of the 16x16x32 ones gave wrong sums on gfx950 with
 // hipcc 7.2 whenever a wave ran more than one tile; one opcode per accumulator chain does not.)
 struct QRegs {
-  bf16x8 full[KSTEPS + (KREM ? 1 : 0)];
+  bf16x8 full[QSTEPS];
 };
-constexpr int QSTEPS = KSTEPS + (KREM ? 1 : 0);
 
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
@@ -48,7 +58,7 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-// operand registers of one row (a key's or a query's `D` elements) in the lane's MFMA slots
+// operand registers of one row (a key's or a query's D elements) in the lane's MFMA slots
 __device__ __forceinline__ void load_row(bf16x8 (&r)[QSTEPS], const uint16_t* row, bool ok) {
   const int lane = threadIdx.x & 63;
 #pragma unroll
@@ -63,32 +73,32 @@ __device__ __forceinline__ void load_row(bf16x8 (&r)[QSTEPS], const uint16_t* ro
   }
 }
 
-struct Geometry {
-  const uint16_t* k_pages;   // [pages, nkv, P, D]
-  const uint16_t* v_pages;   // [pages, nkv, D, P]
-  const int* bt;             // this request's block table row
-  int nkv, g, page_shift, kv_len;
-  float scale;
-};
-
-__device__ __forceinline__ s16x4 pack_bf16x4(float a, float b, float c, float d) {
-  s16x4 r;
-  r[0] = (short)float_to_bf16_bits(a);
-  r[1] = (short)float_to_bf16_bits(b);
-  r[2] = (short)float_to_bf16_bits(c);
-  r[3] = (short)float_to_bf16_bits(d);
-  return r;
+// two floats -> two bfloat16 in one register (v_cvt_pk_bf16_f32, round to nearest even)
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const f32x2 v = {a, b};
+  const bf16x2 r = __builtin_convertvector(v, bf16x2);
+  return *reinterpret_cast<const uint32_t*>(&r);
 }
 
-// Loads the query rows of NB blocks of 16 columns.  Column c of block nb is token (first_col + 16 nb + c) / gpad
-// of the entry, head (...) % gpad of the group; columns without a query hold zeros.
+__device__ __forceinline__ s16x4 pack_bf16x4(float a, float b, float c, float d) {
+  union {
+    uint32_t u[2];
+    s16x4 v;
+  } r;
+  r.u[0] = pack_bf16x2(a, b);
+  r.u[1] = pack_bf16x2(c, d);
+  return r.v;
+}
+
+// Loads the query rows of NB blocks of 16 columns.  Column c of block nb is token (16 nb + c) / gpad of the
+// `q_tokens` tokens that start at q_base, head (16 nb + c) % gpad of the group; columns without a query hold zeros.
 template <int NB>
-__device__ __forceinline__ void load_queries(QRegs (&q)[NB], const uint16_t* q_base, int64_t q_row_stride, int first_col,
-                                             int gpad, int G, int q_tokens, int head0) {
+__device__ __forceinline__ void load_queries(QRegs (&q)[NB], const uint16_t* q_base, int64_t q_row_stride, int gpad,
+                                             int G, int q_tokens, int head0) {
   const int lane = threadIdx.x & 63;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
-    const int col = first_col + 16 * nb + (lane & 15);
+    const int col = 16 * nb + (lane & 15);
     const int tok = col / gpad, hh = col % gpad;
     const bool ok = hh < G && tok < q_tokens;
     const uint16_t* row = q_base + (int64_t)(ok ? tok : 0) * q_row_stride + (int64_t)(head0 + (ok ? hh : 0)) * D;
@@ -96,107 +106,13 @@ __device__ __forceinline__ void load_queries(QRegs (&q)[NB], const uint16_t* q_b
   }
 }
 
-// Running softmax state of NB column blocks.
+// Running softmax state of NB column blocks (maxima in base-2 units of the scaled scores).
 template <int NB>
 struct State {
   float m[NB];        // running maximum of the column (same in the 4 lanes that share it)
   float l[NB];        // this lane's share of the running sum
   f32x4 o[NB][DBLK];  // O^T accumulators: dims 16 blk + 4 (lane / 16) + i of column lane % 16
 };
-
-// The cache operands of one tile of 16 keys in the lane's MFMA slots.
-struct TileRegs {
-  bf16x8 ka[QSTEPS];
-  s16x4 va[DBLK];
-};
-
-// Page ids of the tile that starts at key j0 (addresses clamped to the request's last key: masked keys read
-// valid memory of the request).
-__device__ __forceinline__ void tile_pages(const Geometry& geo, int j0, int& kk, int& vk, int& kpage, int& vpage) {
-  const int lane = threadIdx.x & 63;
-  const int last = geo.kv_len - 1;
-  kk = j0 + (lane & 15);
-  kk = kk > last ? last : kk;
-  vk = j0 + 4 * (lane >> 4);
-  vk = vk > last ? (last & ~3) : vk;
-  kpage = geo.bt[kk >> geo.page_shift];
-  vpage = geo.bt[vk >> geo.page_shift];
-}
-
-__device__ __forceinline__ void tile_load(TileRegs& t, const Geometry& geo, int kk, int vk, int kpage, int vpage) {
-  const int lane = threadIdx.x & 63;
-  const int P = 1 << geo.page_shift;
-  const uint16_t* krow = geo.k_pages + (((int64_t)kpage * geo.nkv + geo.g) * P + (kk & (P - 1))) * D;
-  load_row(t.ka, krow, true);
-  const uint16_t* vbase = geo.v_pages + (((int64_t)vpage * geo.nkv + geo.g) * D + (lane & 15)) * P + (vk & (P - 1));
-#pragma unroll
-  for (int blk = 0; blk < DBLK; ++blk) t.va[blk] = *reinterpret_cast<const s16x4*>(vbase + (int64_t)16 * blk * P);
-}
-
-// Scores, running softmax and the value product of one tile whose operands are in `t`.
-template <int NB>
-__device__ __forceinline__ void tile_compute(State<NB>& st, const QRegs (&q)[NB], const TileRegs& t, float scale, int j0,
-                                             const int (&pos_lo)[NB], const int (&pos_hi)[NB]) {
-  const int lane = threadIdx.x & 63;
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int k = 0; k < QSTEPS; ++k) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.ka[k], q[nb].full[k], s, 0, 0, 0);
-    // lane holds S^T[key j0 + 4 (lane / 16) + i][column lane % 16]
-    const int kbase = j0 + 4 * (lane >> 4);
-    float sv[4];
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int key = kbase + i;
-      const bool ok = key <= pos_hi[nb] && key >= pos_lo[nb];
-      sv[i] = ok ? s[i] * scale : -INFINITY;
-      tmax = fmaxf(tmax, sv[i]);
-    }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(st.m[nb], tmax);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a column that has seen no key yet
-    const float alpha = expf(st.m[nb] - m_use);               // exp(-inf) = 0 on the first visible tile
-    float p[4];
-    float psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      p[i] = expf(sv[i] - m_use);                             // exp(-inf) = 0 for masked keys
-      psum += p[i];
-    }
-    st.l[nb] = st.l[nb] * alpha + psum;
-    st.m[nb] = m_new;
-    const s16x4 pb = pack_bf16x4(p[0], p[1], p[2], p[3]);
-#pragma unroll
-    for (int blk = 0; blk < DBLK; ++blk) {
-      f32x4 o = st.o[nb][blk];
-      o[0] *= alpha;
-      o[1] *= alpha;
-      o[2] *= alpha;
-      o[3] *= alpha;
-      st.o[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(t.va[blk], pb, o, 0, 0, 0);
-    }
-  }
-}
-
-// One pass over the tiles of 16 keys that start at key_begin, key_begin + stride, ... below key_end
-// (key_begin a multiple of 16, stride a multiple of 16).
-// pos_hi[nb] / pos_lo[nb]: the last and first key the lane's column of block nb may see (pos_hi < 0: none).
-// (Running the loads a tile ahead of the arithmetic by hand was measured and gained nothing: the waves of a
-// compute unit already overlap one another's loads.)
-template <int NB>
-__device__ __forceinline__ void attend(State<NB>& st, const QRegs (&q)[NB], const Geometry& geo, int key_begin,
-                                       int key_end, int stride, const int (&pos_lo)[NB], const int (&pos_hi)[NB]) {
-  for (int j0 = key_begin; j0 < key_end; j0 += stride) {
-    TileRegs t;
-    int kk, vk, kpage, vpage;
-    tile_pages(geo, j0, kk, vk, kpage, vpage);
-    tile_load(t, geo, kk, vk, kpage, vpage);
-    tile_compute<NB>(st, q, t, geo.scale, j0, pos_lo, pos_hi);
-  }
-}
 
 template <int NB>
 __device__ __forceinline__ void init_state(State<NB>& st) {
@@ -209,48 +125,90 @@ __device__ __forceinline__ void init_state(State<NB>& st) {
   }
 }
 
-// ---------------------------------------------------------------- prefill: several new tokens per entry
-// work[w] = {entry b, block index within the entry}; a block is 16 * NB columns = 16 * NB / gpad query tokens.
+// S^T of one tile of 16 keys (operands `ka`) against the NB query blocks.
 template <int NB>
-__global__ __launch_bounds__(256) void prefill_kernel(
-    const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
-    const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
-    int table_width, const int* __restrict__ work, int num_work, const int* __restrict__ cu_q,
-    const int* __restrict__ kv_len, int nq, int nkv, int gpad, int page_shift, float scale, int window) {
-  const int lane = threadIdx.x & 63;
-  const int w = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (w >= num_work) return;
-  const int b = work[2 * w], blk_idx = work[2 * w + 1];
-  const int g = blockIdx.y;
-  const int G = nq / nkv;
-  const int q_begin = cu_q[b];
-  const int q_len = cu_q[b + 1] - q_begin;
-  const int kv = kv_len[b];
-  const int tokens_per_block = 16 * NB / gpad;
-  const int tok0 = blk_idx * tokens_per_block;          // first query token of this block within the entry
-  const int q_tokens = min(tokens_per_block, q_len - tok0);
-  const int pos0 = kv - q_len + tok0;                   // its position
-
-  Geometry geo{k_pages, v_pages, block_table + (int64_t)b * table_width, nkv, g, page_shift, kv, scale};
-  QRegs qr[NB];
-  load_queries<NB>(qr, q + (int64_t)(q_begin + tok0) * q_row_stride, q_row_stride, 0, gpad, G, q_tokens, g * G);
-
-  int pos_lo[NB], pos_hi[NB];
+__device__ __forceinline__ void tile_scores(f32x4 (&s)[NB], const bf16x8 (&ka)[QSTEPS], const QRegs (&q)[NB]) {
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
-    const int col = 16 * nb + (lane & 15);
-    const int tok = col / gpad, hh = col % gpad;
-    const bool ok = hh < G && tok < q_tokens;
-    pos_hi[nb] = ok ? pos0 + tok : -1;
-    pos_lo[nb] = (ok && window > 0 && pos0 + tok - window + 1 > 0) ? pos0 + tok - window + 1 : 0;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < QSTEPS; ++k) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[k], q[nb].full[k], acc, 0, 0, 0);
+    s[nb] = acc;
   }
-  const int first_pos = pos0, last_pos = pos0 + q_tokens - 1;
-  const int lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+}
 
-  State<NB> st;
-  init_state<NB>(st);
-  attend<NB>(st, qr, geo, lo & ~15, last_pos + 1, 16, pos_lo, pos_hi);
+// The running softmax over the macro tile that starts at key j0: masks and scales the scores in s[t][nb]
+// (lane: key j0 + 16 t + 4 (lane / 16) + i, column lane % 16), moves the maxima, rescales sums and accumulators,
+// and leaves the probabilities, rounded to bfloat16, in p[t][nb].  c = scale * log2(e).
+// pos_hi[nb] / pos_lo[nb]: the last and first key the lane's column of block nb may see (pos_hi < 0: none).
+template <int NB>
+__device__ __forceinline__ void softmax_update(State<NB>& st, f32x4 (&s)[MT][NB], s16x4 (&p)[MT][NB], float c, int j0,
+                                               const int (&pos_lo)[NB], const int (&pos_hi)[NB]) {
+  const int lane = threadIdx.x & 63;
+  const int kbase = j0 + 4 * (lane >> 4);
+  float alpha[NB];
+  bool moved = false;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kbase + 16 * t + i;
+        const bool ok = key <= pos_hi[nb] && key >= pos_lo[nb];
+        const float v = ok ? s[t][nb][i] * c : -INFINITY;
+        s[t][nb][i] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(st.m[nb], tmax);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;    // a column that has seen no key yet
+    alpha[nb] = __builtin_amdgcn_exp2f(st.m[nb] - m_use);      // 2^-inf = 0 on the first visible tile
+    moved = moved || (m_new != st.m[nb]);
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      float e[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        e[i] = __builtin_amdgcn_exp2f(s[t][nb][i] - m_use);    // 0 for masked keys
+        psum += e[i];
+      }
+      p[t][nb] = pack_bf16x4(e[0], e[1], e[2], e[3]);
+    }
+    st.l[nb] = st.l[nb] * alpha[nb] + psum;
+    st.m[nb] = m_new;
+  }
+  if (__any(moved)) {     // the same for every lane of the wave
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int blk = 0; blk < DBLK; ++blk) {
+        st.o[nb][blk][0] *= alpha[nb];
+        st.o[nb][blk][1] *= alpha[nb];
+        st.o[nb][blk][2] *= alpha[nb];
+        st.o[nb][blk][3] *= alpha[nb];
+      }
+  }
+}
 
+// O^T += V^T P^T for one tile of 16 keys (operands `va`).
+template <int NB>
+__device__ __forceinline__ void tile_values(State<NB>& st, const s16x4 (&va)[DBLK], const s16x4 (&p)[NB]) {
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int blk = 0; blk < DBLK; ++blk)
+      st.o[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[blk], p[nb], st.o[nb][blk], 0, 0, 0);
+}
+
+// Normalises and stores the columns of a wave: token col / gpad of the rows that start at out_base.
+template <int NB>
+__device__ __forceinline__ void store_output(const State<NB>& st, uint16_t* out_base, int64_t out_row_stride, int gpad,
+                                             int head0, const int (&pos_hi)[NB]) {
+  const int lane = threadIdx.x & 63;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     float l = st.l[nb];
@@ -260,7 +218,7 @@ __global__ __launch_bounds__(256) void prefill_kernel(
     const float inv = 1.f / l;
     const int col = 16 * nb + (lane & 15);
     const int tok = col / gpad, hh = col % gpad;
-    uint16_t* o = out + (int64_t)(q_begin + tok0 + tok) * out_row_stride + (int64_t)(g * G + hh) * D + 4 * (lane >> 4);
+    uint16_t* o = out_base + (int64_t)tok * out_row_stride + (int64_t)(head0 + hh) * D + 4 * (lane >> 4);
 #pragma unroll
     for (int blk = 0; blk < DBLK; ++blk) {
       const f32x4 v = st.o[nb][blk];
@@ -269,21 +227,156 @@ __global__ __launch_bounds__(256) void prefill_kernel(
   }
 }
 
+// ---------------------------------------------------------------- prefill: several new tokens per entry
+// A workgroup of 4 waves takes 4 consecutive query blocks of one entry and one kv head.  All four need the same
+// keys and values, so each macro tile is read from global memory once per workgroup, by all 256 threads
+// together, into LDS (the next tile's loads are in flight in registers while the current one is multiplied), and
+// every wave takes its MFMA operands from there.  Rows are padded so that the 16 lanes of an operand read hit
+// different banks.  work[w] = {entry, block of 4 * (16 NB / gpad) query tokens}.  Pages hold 8 tokens or more.
+#ifndef PREFILL_NB
+#define PREFILL_NB 1
+#endif
+constexpr int LDS_KSTR = D + 8;                  // elements per key row in LDS
+constexpr int LDS_VSTR = MKEYS + 8;              // elements per dim row of the transposed values in LDS
+constexpr int LDS_KCHUNKS = MKEYS * (D / 8);     // 16-byte chunks of a key tile
+constexpr int LDS_VCHUNKS = D * (MKEYS / 8);     // 16-byte chunks of a value tile
+constexpr int LDS_KITER = (LDS_KCHUNKS + 255) / 256;
+constexpr int LDS_VITER = (LDS_VCHUNKS + 255) / 256;
+
+template <int NB>
+__global__ __launch_bounds__(256) void prefill_kernel(
+    const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
+    const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
+    int table_width, const int* __restrict__ work, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int nq,
+    int nkv, int gpad, int page_shift, float scale, int window) {
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[MKEYS * LDS_KSTR];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[D * LDS_VSTR];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int b = work[2 * blockIdx.x], sb = work[2 * blockIdx.x + 1];
+  const int g = blockIdx.y;
+  const int G = nq / nkv;
+  const int P = 1 << page_shift;
+  const int q_begin = cu_q[b];
+  const int q_len = cu_q[b + 1] - q_begin;
+  const int kv = kv_len[b];
+  const int last = kv - 1;
+  const int tokens_per_wave = 16 * NB / gpad;
+  const int wg_tok0 = sb * 4 * tokens_per_wave;                    // first query token of the workgroup
+  const int wg_tokens = min(4 * tokens_per_wave, q_len - wg_tok0);
+  const int tok0 = wg_tok0 + wave * tokens_per_wave;               // of this wave
+  const int q_tokens = max(0, min(tokens_per_wave, q_len - tok0));
+  const int pos0 = kv - q_len + tok0;
+  const int* bt = block_table + (int64_t)b * table_width;
+
+  QRegs qr[NB];
+  load_queries<NB>(qr, q + (int64_t)(q_begin + (q_tokens > 0 ? tok0 : wg_tok0)) * q_row_stride, q_row_stride, gpad, G,
+                   q_tokens, g * G);
+  int pos_lo[NB], pos_hi[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int col = 16 * nb + (lane & 15);
+    const int tok = col / gpad, hh = col % gpad;
+    const bool ok = hh < G && tok < q_tokens;
+    pos_hi[nb] = ok ? pos0 + tok : -1;
+    pos_lo[nb] = (ok && window > 0 && pos0 + tok - window + 1 > 0) ? pos0 + tok - window + 1 : 0;
+  }
+  // keys the workgroup walks, and the part of them this wave's queries can see
+  const int wg_first = kv - q_len + wg_tok0, wg_last = wg_first + wg_tokens - 1;
+  const int wg_lo = ((window > 0 && wg_first - window + 1 > 0) ? wg_first - window + 1 : 0) / MKEYS * MKEYS;
+  const int wg_hi = wg_last + 1;
+  const int w_lo = (q_tokens > 0 && window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int w_hi = q_tokens > 0 ? pos0 + q_tokens : 0;
+  const float c = scale * 1.44269504088896340736f;
+
+  State<NB> st;
+  init_state<NB>(st);
+
+  // this thread's chunks of a macro tile: global -> registers (PREFILL_FETCH), registers -> LDS (PREFILL_STASH)
+  const int kpp = P < MKEYS ? P : MKEYS;   // keys of a macro tile that lie in one page
+  const int cpp = kpp / 8;                 // 16-byte chunks per (page, dim)
+  u32x4 pk[LDS_KITER], pv[LDS_VITER];
+#define PREFILL_FETCH(J0)                                                                                            \
+  {                                                                                                                  \
+    _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
+      int ch = threadIdx.x + 256 * it;                                                                               \
+      ch = ch < LDS_KCHUNKS ? ch : LDS_KCHUNKS - 1; /* threads past the end load the last chunk again, drop it */   \
+      int key = (J0) + ch / (D / 8);                                                                                 \
+      key = key > last ? last : key; /* masked keys read valid memory of the request */                             \
+      const int64_t page = bt[key >> page_shift];                                                                    \
+      pk[it] = *reinterpret_cast<const u32x4*>(k_pages + ((page * nkv + g) * P + (key & (P - 1))) * D +              \
+                                               8 * (ch % (D / 8)));                                                  \
+    }                                                                                                                \
+    _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
+      int ch = threadIdx.x + 256 * it;                                                                               \
+      ch = ch < LDS_VCHUNKS ? ch : LDS_VCHUNKS - 1;                                                                  \
+      /* chunk -> (page of the tile, dim, run of 8 keys): consecutive threads read consecutive memory of a page */  \
+      const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);                                      \
+      int key = (J0) + page_i * kpp + 8 * part;                                                                      \
+      key = key > last ? (last & ~7) : key; /* a run of 8 keys lies in one page */                                  \
+      const int64_t page = bt[key >> page_shift];                                                                    \
+      pv[it] = *reinterpret_cast<const u32x4*>(v_pages + ((page * nkv + g) * D + dim) * P + (key & (P - 1)));        \
+    }                                                                                                                \
+  }
+#define PREFILL_STASH()                                                                                              \
+  {                                                                                                                  \
+    _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
+      const int ch = threadIdx.x + 256 * it;                                                                         \
+      if (ch < LDS_KCHUNKS) *reinterpret_cast<u32x4*>(Ks + (ch / (D / 8)) * LDS_KSTR + 8 * (ch % (D / 8))) = pk[it]; \
+    }                                                                                                                \
+    _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
+      const int ch = threadIdx.x + 256 * it;                                                                         \
+      const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);                                      \
+      if (ch < LDS_VCHUNKS) *reinterpret_cast<u32x4*>(Vs + dim * LDS_VSTR + page_i * kpp + 8 * part) = pv[it];       \
+    }                                                                                                                \
+  }
+
+  PREFILL_FETCH(wg_lo)
+  for (int j0 = wg_lo; j0 < wg_hi; j0 += MKEYS) {
+    __syncthreads();                    // every wave is done with the tile that is in LDS
+    PREFILL_STASH()
+    __syncthreads();
+    if (j0 + MKEYS < wg_hi) PREFILL_FETCH(j0 + MKEYS)
+    if (j0 >= w_hi || j0 + MKEYS <= w_lo) continue;      // nothing this wave can see (same for all its lanes)
+    f32x4 s[MT][NB];
+    s16x4 p[MT][NB];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      bf16x8 ka[QSTEPS];
+      load_row(ka, Ks + (16 * t + (lane & 15)) * LDS_KSTR, true);
+      tile_scores<NB>(s[t], ka, qr);
+    }
+    softmax_update<NB>(st, s, p, c, j0, pos_lo, pos_hi);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      s16x4 va[DBLK];
+#pragma unroll
+      for (int blk = 0; blk < DBLK; ++blk)
+        va[blk] = *reinterpret_cast<const s16x4*>(Vs + (16 * blk + (lane & 15)) * LDS_VSTR + 16 * t + 4 * (lane >> 4));
+      tile_values<NB>(st, va, p[t]);
+    }
+  }
+#undef PREFILL_FETCH
+#undef PREFILL_STASH
+  store_output<NB>(st, out + (int64_t)(q_begin + tok0) * out_row_stride, out_row_stride, gpad, g * G, pos_hi);
+}
+
 // ---------------------------------------------------------------- decode: one new token per entry, keys split
-// Grid (num_splits, nkv, entries), 4 waves per workgroup.  The tiles of a split go round-robin to the waves, which
+// Grid (num_splits, nkv, entries), DECODE_WAVES waves per workgroup.  The macro tiles of a split go round-robin to
+// the waves (operands straight from global memory: all of a macro tile's loads are in flight together), which
 // combine their running softmax states through LDS.  With one split the workgroup writes the output itself;
 // with several it writes a partial (max, sum, unnormalised output) per head, and the merge kernel below
 // combines the partials with the log-sum-exp rule.  (Merging inside this kernel, by the workgroup that
 // finishes last, was measured: the device-wide fences it needs cost many times the second launch.)
-// Partials: part_o [entries, nq, num_splits, D], part_ml [entries, nq, num_splits, 2].
-// (2 waves for the largest head sizes, whose states would not fit 64 KB of LDS fourfold)
+// Partials: part_o [entries, nq, num_splits, D], part_ml [entries, nq, num_splits, 2] (max in base-2 units).
 constexpr int DECODE_WAVES = D > 128 ? 2 : 4;
 
 __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
     const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int first_entry,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv, int page_shift, float scale, int window) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv, int page_shift, float scale,
+    int window) {
   __shared__ float lds_o[DECODE_WAVES][DBLK][64][4];
   __shared__ float lds_m[DECODE_WAVES][16];
   __shared__ float lds_l[DECODE_WAVES][16];
@@ -294,25 +387,49 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
   const int e = blockIdx.z;             // entry index among the decode entries
   const int b = first_entry + e;
   const int G = nq / nkv;
+  const int P = 1 << page_shift;
   const int kv = kv_len[b];
   const int pos = kv - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  // this split's keys: tiles of 16 from the first visible tile, evenly over the splits
-  const int tile_lo = lo >> 4, tile_hi = (pos >> 4) + 1;
+  // this split's keys: macro tiles from the first visible one, evenly over the splits
+  const int tile_lo = lo / MKEYS, tile_hi = pos / MKEYS + 1;
   const int tiles_per_split = (tile_hi - tile_lo + num_splits - 1) / num_splits;
   const int t0 = tile_lo + split * tiles_per_split;
   const int t1 = min(tile_hi, t0 + tiles_per_split);
+  const int* bt = block_table + (int64_t)b * table_width;
+  const float c = scale * 1.44269504088896340736f;
 
   State<1> st;
   init_state<1>(st);
   const bool col_ok = (lane & 15) < G;
-  {
-    Geometry geo{k_pages, v_pages, block_table + (int64_t)b * table_width, nkv, g, page_shift, kv, scale};
-    QRegs qr[1];
-    load_queries<1>(qr, q + (int64_t)cu_q[b] * q_row_stride, q_row_stride, 0, 16, G, 1, g * G);
-    const int pos_lo[1] = {lo};
-    const int pos_hi[1] = {col_ok ? pos : -1};
-    attend<1>(st, qr, geo, (t0 + wave) << 4, t1 << 4, 16 * DECODE_WAVES, pos_lo, pos_hi);
+  QRegs qr[1];
+  load_queries<1>(qr, q + (int64_t)cu_q[b] * q_row_stride, q_row_stride, 16, G, 1, g * G);
+  const int pos_lo[1] = {lo};
+  const int pos_hi[1] = {col_ok ? pos : -1};
+  for (int mt = t0 + wave; mt < t1; mt += DECODE_WAVES) {
+    const int j0 = mt * MKEYS;
+    bf16x8 ka[MT][QSTEPS];
+    s16x4 va[MT][DBLK];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {      // addresses clamped to the request's last key: masked keys read valid memory
+      int kk = j0 + 16 * t + (lane & 15);
+      kk = kk > pos ? pos : kk;
+      const int64_t kpage = bt[kk >> page_shift];
+      load_row(ka[t], k_pages + ((kpage * nkv + g) * P + (kk & (P - 1))) * D, true);
+      int vk = j0 + 16 * t + 4 * (lane >> 4);
+      vk = vk > pos ? (pos & ~3) : vk;
+      const int64_t vpage = bt[vk >> page_shift];
+      const uint16_t* vbase = v_pages + ((vpage * nkv + g) * D + (lane & 15)) * P + (vk & (P - 1));
+#pragma unroll
+      for (int blk = 0; blk < DBLK; ++blk) va[t][blk] = *reinterpret_cast<const s16x4*>(vbase + (int64_t)16 * blk * P);
+    }
+    f32x4 s[MT][1];
+    s16x4 p[MT][1];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) tile_scores<1>(s[t], ka[t], qr);
+    softmax_update<1>(st, s, p, c, j0, pos_lo, pos_hi);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) tile_values<1>(st, va[t], p[t]);
   }
   // ---- combine the waves: every wave leaves its state in LDS
   float l = st.l[0];
@@ -325,28 +442,28 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
     lds_l[wave][lane] = l;
   }
   __syncthreads();
-  // thread -> (block of dims, lane slot): column c = slot % 16, dims 16 blk + 4 (slot / 16) + i
+  // thread -> (block of dims, lane slot): column col = slot % 16, dims 16 blk + 4 (slot / 16) + i
   for (int idx = threadIdx.x; idx < DBLK * 64; idx += blockDim.x) {
     const int blk = idx >> 6, slot = idx & 63;
-    const int c = slot & 15;
-    if (c >= G) continue;
+    const int col = slot & 15;
+    if (col >= G) continue;
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < DECODE_WAVES; ++w) M = fmaxf(M, lds_m[w][c]);
+    for (int w = 0; w < DECODE_WAVES; ++w) M = fmaxf(M, lds_m[w][col]);
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float L = 0.f;
 #pragma unroll
     for (int w = 0; w < DECODE_WAVES; ++w) {
-      const float mw = lds_m[w][c];
-      const float wt = (mw == -INFINITY) ? 0.f : expf(mw - M);
+      const float mw = lds_m[w][col];
+      const float wt = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - M);
       const f32x4 v = *reinterpret_cast<const f32x4*>(&lds_o[w][blk][slot][0]);
       acc[0] += wt * v[0];
       acc[1] += wt * v[1];
       acc[2] += wt * v[2];
       acc[3] += wt * v[3];
-      L += wt * lds_l[w][c];
+      L += wt * lds_l[w][col];
     }
-    const int head = g * G + c;
+    const int head = g * G + col;
     const int dim = 16 * blk + 4 * (slot >> 4);
     if (num_splits == 1) {
       const float inv = 1.f / L;
@@ -363,7 +480,7 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
   }
 }
 
-// out[token of entry e][head] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s
+// out[token of entry e][head] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s
 // One wave per (entry, head).  The lanes first share out the splits (maximum, weights, sum), then the dims;
 // the loads of a phase do not depend on one another, so they are all in flight together.
 __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part_o,
@@ -374,7 +491,7 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   const int lane = threadIdx.x;
   const int e = blockIdx.x / nq, head = blockIdx.x % nq;
   const int64_t base = ((int64_t)e * nq + head) * num_splits;
-  constexpr int MAXR = 16;
+  constexpr int MAXR = 16;                       // 64 * 16 = 1024 splits at most
   float mv[MAXR], lv[MAXR];
   float M = -INFINITY;
 #pragma unroll
@@ -391,13 +508,14 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   float L = 0.f;
 #pragma unroll
   for (int r = 0; r < MAXR; ++r) {
-    mv[r] = (mv[r] == -INFINITY) ? 0.f : expf(mv[r] - M);
+    mv[r] = (mv[r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mv[r] - M);   // now the split's weight
     L += mv[r] * lv[r];
     if (64 * (r + 1) >= num_splits) break;
   }
   L = wave_sum(L);
   const float inv = 1.f / L;
   uint16_t* o = out + (int64_t)cu_q[first_entry + e] * out_row_stride + (int64_t)head * D;
+  // dims: 4 per lane and round; every lane runs every round (the shuffles below need all lanes)
 #pragma unroll
   for (int round = 0; round < (D + 255) / 256; ++round) {
     const int dd = 256 * round + 4 * lane;
@@ -427,7 +545,7 @@ static int check_common(const char* what, int nq, int nkv, int page_size, int64_
                         int table_width) {
   MI_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "%s: %d query heads are no multiple of %d kv heads", what, nq, nkv);
   MI_REQUIRE(nq / nkv <= 16, "%s: %d query heads per kv head; this kernel takes at most 16", what, nq / nkv);
-  MI_REQUIRE(page_size >= 4 && (page_size & (page_size - 1)) == 0, "%s: page size %d is not a power of two >= 4", what,
+  MI_REQUIRE(page_size >= 8 && (page_size & (page_size - 1)) == 0, "%s: page size %d is not a power of two >= 8", what,
              page_size);
   MI_REQUIRE(q_row_stride >= (int64_t)nq * D && q_row_stride % 8 == 0, "%s: query row stride %lld", what,
              (long long)q_row_stride);
@@ -443,14 +561,24 @@ static int log2_of(int v) {
   return s;
 }
 
+static int group_pad(int nq, int nkv) {
+  int gpad = 1;
+  while (gpad < nq / nkv) gpad <<= 1;
+  return gpad;
+}
+
 MI_EXPORT int mi_attn_head_dim() { return D; }
 
-// Columns per block and query tokens per block for `nq / nkv` heads per group.
+// Keys per macro tile: the granule of the decode kernel's key splits.
+MI_EXPORT int mi_attn_macro_tile_keys() { return MKEYS; }
+
+// Waves per workgroup of the decode kernel.
+MI_EXPORT int mi_attn_decode_waves() { return DECODE_WAVES; }
+
+// Query tokens per work item (a workgroup of 4 waves, 16 * PREFILL_NB columns each) of the prefill launch.
 MI_EXPORT int mi_attn_prefill_tokens_per_block(int nq, int nkv) {
-  const int G = nq / nkv;
-  int gpad = 1;
-  while (gpad < G) gpad <<= 1;
-  return gpad > 16 ? 0 : 32 / gpad;
+  const int gpad = group_pad(nq, nkv);
+  return gpad > 16 ? 0 : 4 * (16 * PREFILL_NB / gpad);
 }
 
 MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, int64_t out_row_stride, const void* k_pages,
@@ -459,15 +587,13 @@ MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, in
                               float scale, int window, hipStream_t stream) {
   if (check_common("attn_prefill", nq, nkv, page_size, q_row_stride, out_row_stride, table_width)) return 1;
   MI_REQUIRE(num_work >= 0 && window >= 0, "attn_prefill: bad work count or window");
+  MI_REQUIRE(nkv <= 65535, "attn_prefill: grid too large");
   if (num_work == 0) return 0;
-  const int G = nq / nkv;
-  int gpad = 1;
-  while (gpad < G) gpad <<= 1;
-  dim3 grid((num_work + 3) / 4, nkv);
-  prefill_kernel<2><<<grid, 256, 0, stream>>>((const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride,
-                                              (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,
-                                              table_width, work, num_work, cu_q, kv_len, nq, nkv, gpad,
-                                              log2_of(page_size), scale, window);
+  dim3 grid(num_work, nkv);
+  prefill_kernel<PREFILL_NB><<<grid, 256, 0, stream>>>(
+      (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
+      (const uint16_t*)v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv, group_pad(nq, nkv),
+      log2_of(page_size), scale, window);
   MI_CHECK_LAUNCH("attn_prefill");
   return 0;
 }

@@ -14,6 +14,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // (arrays of HIP's uint4 / float4 classes end up in scratch memory)
 
 __device__ __forceinline__ bf16x8 zero_bf16x8() {
   bf16x8 z;
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   constexpr int CH = MB == 1 ? 8 : (MB == 2 ? 4 : 2);   // what fits the 128 registers of a 16-wave workgroup
   for (int s0 = s_begin; s0 < s_end; s0 += CH) {
     bf16x8 w[CH][RB];
-    uint4 ar[CH][MB];
+    u32x4 ar[CH][MB];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int k = 32 * (s0 + c) + 8 * (lane >> 4);
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const bool ok = kok && mok[mb];
-        ar[c][mb] = ok ? *reinterpret_cast<const uint4*>(arow[mb] + k) : uint4{0, 0, 0, 0};
+        ar[c][mb] = ok ? *reinterpret_cast<const u32x4*>(arow[mb] + k) : u32x4{0, 0, 0, 0};
       }
     }
 #pragma unroll
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         union {
-          uint4 u;
+          u32x4 u;
           bf16x8 v;
         } a;
         a.u = ar[c][mb];
@@ -187,8 +188,8 @@ __global__ __launch_bounds__(512) void norm_gemm_kernel(const float* __restrict_
   constexpr int CH = 4;
   for (int s0 = s_begin; s0 < s_end; s0 += CH) {
     bf16x8 w[CH][RB];
-    float4 r0[CH], r1[CH], g0[CH], g1[CH];
-    uint4 xr[CH];
+    f32x4 r0[CH], r1[CH], g0[CH], g1[CH];
+    u32x4 xr[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int k = 32 * (s0 + c) + 8 * (lane >> 4);
@@ -196,19 +197,19 @@ __global__ __launch_bounds__(512) void norm_gemm_kernel(const float* __restrict_
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) w[c][rb] = kok ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
       const bool ok = kok && mok;
-      r0[c] = ok ? *reinterpret_cast<const float4*>(rrow + k) : float4{0.f, 0.f, 0.f, 0.f};
-      r1[c] = ok ? *reinterpret_cast<const float4*>(rrow + k + 4) : float4{0.f, 0.f, 0.f, 0.f};
-      xr[c] = (ok && xrow) ? *reinterpret_cast<const uint4*>(xrow + k) : uint4{0, 0, 0, 0};
-      g0[c] = kok ? *reinterpret_cast<const float4*>(NW + k) : float4{0.f, 0.f, 0.f, 0.f};
-      g1[c] = kok ? *reinterpret_cast<const float4*>(NW + k + 4) : float4{0.f, 0.f, 0.f, 0.f};
+      r0[c] = ok ? *reinterpret_cast<const f32x4*>(rrow + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+      r1[c] = ok ? *reinterpret_cast<const f32x4*>(rrow + k + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+      xr[c] = (ok && xrow) ? *reinterpret_cast<const u32x4*>(xrow + k) : u32x4{0, 0, 0, 0};
+      g0[c] = kok ? *reinterpret_cast<const f32x4*>(NW + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+      g1[c] = kok ? *reinterpret_cast<const f32x4*>(NW + k + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       if (s0 + c >= s_end) break;
       const int k = 32 * (s0 + c) + 8 * (lane >> 4);
-      float v[8] = {r0[c].x, r0[c].y, r0[c].z, r0[c].w, r1[c].x, r1[c].y, r1[c].z, r1[c].w};
-      const uint32_t xw[4] = {xr[c].x, xr[c].y, xr[c].z, xr[c].w};
-      const float gw[8] = {g0[c].x, g0[c].y, g0[c].z, g0[c].w, g1[c].x, g1[c].y, g1[c].z, g1[c].w};
+      float v[8] = {r0[c][0], r0[c][1], r0[c][2], r0[c][3], r1[c][0], r1[c][1], r1[c][2], r1[c][3]};
+      const uint32_t xw[4] = {xr[c][0], xr[c][1], xr[c][2], xr[c][3]};
+      const float gw[8] = {g0[c][0], g0[c][1], g0[c][2], g0[c][3], g1[c][0], g1[c][1], g1[c][2], g1[c][3]};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         v[2 * i] += __uint_as_float(xw[i] << 16);

@@ -416,15 +416,21 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_k: Opt
 
 def mfma_attention_supported(dtype: torch.dtype, nq: int, nkv: int, d: int, page_size: int) -> bool:
   """The MFMA attention kernels take bfloat16, head sizes that are multiples of 16 up to 256, up to 16 query
-  heads per kv head, and pages of at least 4 tokens; everything else runs on the plain kernel."""
+  heads per kv head, and pages of at least 8 tokens; everything else runs on the plain kernel."""
   return (dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and nq % nkv == 0 and nq // nkv <= 16
-          and page_size >= 4)
+          and page_size >= 8)
 
 
 def attn_prefill_tokens_per_block(nq: int, nkv: int, d: int) -> int:
-  """Query tokens one wave of the prefill kernel takes (the granule of its work list)."""
+  """Query tokens one work item of the prefill launch takes (the granule of its work list)."""
   lib = _lib("attention_mfma", (("HEAD_DIM", d),))
   return lib.mi_attn_prefill_tokens_per_block(nq, nkv)
+
+
+def attn_decode_geometry(d: int):
+  """(keys per macro tile, waves per workgroup) of the decode kernel for this head size."""
+  lib = _lib("attention_mfma", (("HEAD_DIM", d),))
+  return lib.mi_attn_macro_tile_keys(), lib.mi_attn_decode_waves()
 
 
 def _attn_common(what, q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len):

@@ -93,7 +93,9 @@ class PagedAttention(Part):
       ops.attn_prefill(qkv, nq, nkv, d, out, cache.k, cache.v, table, work, ctx.cu_q, ctx.kv_len, self.scale, window)
     n_single = ctx.num_requests - ctx.num_multi
     if n_single > 0:
-      splits = decode_splits(n_single * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len)
+      tile_keys, waves = ops.attn_decode_geometry(d)
+      splits = decode_splits(n_single * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len, tile_keys,
+                             waves)
       need = n_single * nq * splits
       part_o = ctx.scratch("attn_part_o", need * d, torch.float32)
       part_ml = ctx.scratch("attn_part_ml", need * 2, torch.float32)
@@ -101,12 +103,13 @@ class PagedAttention(Part):
                       splits, part_o, part_ml, self.scale, window)
 
 
-def decode_splits(num_head_entries: int, max_keys: int, target_waves: int = 2048) -> int:
-  """Into how many key ranges (workgroups of 4 waves) a decoding request is cut: enough waves to fill the chip,
-  at least 4 tiles of 16 keys per range."""
-  tiles = -(-max_keys // 16)
-  want = -(-target_waves // max(1, 4 * num_head_entries))     # up to 4 waves per workgroup
-  return int(max(1, min(want, max(1, tiles // 4), 256)))
+def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, waves: int = 4,
+                  target_waves: int = 2048) -> int:
+  """Into how many key ranges (workgroups of `waves` waves, each taking macro tiles of `tile_keys` keys in turn) a
+  decoding request is cut: enough waves to fill the chip, at least one macro tile per wave."""
+  tiles = -(-max_keys // tile_keys)
+  want = -(-target_waves // max(1, waves * num_head_entries))
+  return int(max(1, min(want, max(1, tiles // waves), 256)))
 
 
 register_mixer("paged_attention", PagedAttention)

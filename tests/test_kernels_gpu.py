@@ -248,7 +248,7 @@ def _paged_case(reqs, nq, nkv, d, P, window, seed):
               cu=i32(cu), kv=i32(kv_lens), token_req=i32(token_req), want=torch.cat(want, 0), T=T, B=B, q_lens=[n for _, n in reqs])
 
 
-MFMA_SHAPES = [(16, 8, 128, 16, 0), (6, 3, 48, 16, 0), (8, 2, 32, 8, 0), (4, 4, 16, 4, 0), (5, 1, 80, 32, 0),
+MFMA_SHAPES = [(16, 8, 128, 16, 0), (6, 3, 48, 16, 0), (8, 2, 32, 8, 0), (4, 4, 16, 8, 0), (5, 1, 80, 32, 0),
                (16, 1, 64, 16, 0), (12, 4, 96, 64, 0), (4, 2, 256, 16, 0), (8, 4, 128, 16, 50), (6, 2, 64, 8, 17)]
 
 
