@@ -51,6 +51,29 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
 __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(bf16 x) { return bf16_bits_to_float(x.bits); }
 
+// two values of the activation dtype at once (a 32-bit or 64-bit access)
+typedef __bf16 mi_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float mi_f32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void load2(const float* p, float& a, float& b) {
+  const mi_f32x2 v = *reinterpret_cast<const mi_f32x2*>(p);
+  a = v[0];
+  b = v[1];
+}
+__device__ __forceinline__ void load2(const bf16* p, float& a, float& b) {
+  const uint32_t u = *reinterpret_cast<const uint32_t*>(p);
+  a = __uint_as_float(u << 16);
+  b = __uint_as_float(u & 0xffff0000u);
+}
+__device__ __forceinline__ void store2(float* p, float a, float b) {
+  *reinterpret_cast<mi_f32x2*>(p) = mi_f32x2{a, b};
+}
+__device__ __forceinline__ void store2(bf16* p, float a, float b) {   // v_cvt_pk_bf16_f32: round to nearest even
+  const mi_f32x2 v = {a, b};
+  const mi_bf16x2 r = __builtin_convertvector(v, mi_bf16x2);
+  *reinterpret_cast<uint32_t*>(p) = *reinterpret_cast<const uint32_t*>(&r);
+}
+
 template <typename T>
 __device__ __forceinline__ T from_float(float x);
 template <>

@@ -89,10 +89,8 @@ __device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
   *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
 }
 __device__ __forceinline__ void store4(bf16* p, const float (&v)[4]) {
-  uint2 t;
-  t.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
-  t.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
-  *reinterpret_cast<uint2*>(p) = t;
+  store2(p, v[0], v[1]);
+  store2(p + 2, v[2], v[3]);
 }
 
 template <typename TX, typename TY, int CH>
@@ -196,9 +194,40 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   }
 }
 
+// the same, two pairs of columns per thread (I a multiple of 4: 64-bit and 128-bit accesses)
+template <typename T>
+__global__ void silu_mul4_kernel(const T* __restrict__ gu, T* __restrict__ out, int M, int I) {
+  const int q = I / 4;
+  const int64_t total = (int64_t)M * q;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = idx / q;
+    const int c = 4 * (int)(idx - m * q);
+    float g[4], u[4], r[4];
+    load4(gu + m * 2 * I + c, g);
+    load4(gu + m * 2 * I + I + c, u);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = g[j] / (1.f + expf(-g[j])) * u[j];
+    store4(out + m * I + c, r);
+  }
+}
+
 MI_EXPORT int mi_silu_mul(int dtype, const void* gu, void* out, int M, int I, hipStream_t stream) {
   MI_REQUIRE(M >= 0 && I > 0, "silu_mul: bad sizes M=%d I=%d", M, I);
   if (M == 0) return 0;
+  if (I % 4 == 0) {
+    const int64_t total4 = (int64_t)M * (I / 4);
+    int64_t blocks4 = (total4 + 255) / 256;
+    if (blocks4 > 65536) blocks4 = 65536;
+    if (dtype == MI_DTYPE_F32)
+      silu_mul4_kernel<float><<<(int)blocks4, 256, 0, stream>>>((const float*)gu, (float*)out, M, I);
+    else if (dtype == MI_DTYPE_BF16)
+      silu_mul4_kernel<bf16><<<(int)blocks4, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, M, I);
+    else
+      MI_FAIL("silu_mul: unknown dtype %d", dtype);
+    MI_CHECK_LAUNCH("silu_mul");
+    return 0;
+  }
   const int64_t total = (int64_t)M * I;
   const int threads = 256;
   int64_t blocks = (total + threads - 1) / threads;
@@ -254,25 +283,32 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_strid
   if (h >= nq + nkv) return;
 
   // every load that does not depend on another is issued first: the head's elements as rotation pairs
-  // (j, j + half) and the pass-through tail, the norm weights, the position
+  // (j, j + half), two neighbouring pairs per lane, and the pass-through tail, the norm weights, the position
   const float* w = (h < nq) ? qw : kw;
   const int rd = cos_sin ? rotary_dim : 0;
   const int half = rd / 2;
   int pos = positions ? positions[t] : 0;
   pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
-  float x1[2], x2[2], w1[2], w2[2];      // pairs lane, lane + 64 (half <= 128)
-  float xt[4], wt[4];                    // tail elements rd + lane + 64 c (d <= 256)
-  float ss = 0.f;
-#pragma unroll
-  for (int c = 0; c < 2; ++c) {
-    const int j = lane + 64 * c;
-    const bool ok = j < half;
-    x1[c] = ok ? to_float(src[j]) : 0.f;
-    x2[c] = ok ? to_float(src[j + half]) : 0.f;
-    w1[c] = (ok && w) ? w[j] : 1.f;
-    w2[c] = (ok && w) ? w[j + half] : 1.f;
-    ss += x1[c] * x1[c] + x2[c] * x2[c];
+  const bool two = (half % 2 == 0);      // pairs j, j + 1 share 32-bit (bfloat16) or 64-bit accesses
+  const int j = two ? 2 * lane : lane;   // first pair of this lane (half <= 128: one round)
+  const int j2 = two ? j + 1 : j + 64;   // its second pair
+  const bool ok1 = j < half, ok2 = j2 < half;
+  float xa[2] = {0.f, 0.f}, xb[2] = {0.f, 0.f}, wa[2] = {1.f, 1.f}, wb[2] = {1.f, 1.f};
+  if (two) {
+    if (ok1) {
+      load2(src + j, xa[0], xa[1]);
+      load2(src + j + half, xb[0], xb[1]);
+      if (w) {
+        load2(w + j, wa[0], wa[1]);
+        load2(w + j + half, wb[0], wb[1]);
+      }
+    }
+  } else {
+    if (ok1) { xa[0] = to_float(src[j]); xb[0] = to_float(src[j + half]); if (w) { wa[0] = w[j]; wb[0] = w[j + half]; } }
+    if (ok2) { xa[1] = to_float(src[j2]); xb[1] = to_float(src[j2 + half]); if (w) { wa[1] = w[j2]; wb[1] = w[j2 + half]; } }
   }
+  float xt[4], wt[4];                    // tail elements rd + lane + 64 c (d <= 256)
+  float ss = xa[0] * xa[0] + xa[1] * xa[1] + xb[0] * xb[0] + xb[1] * xb[1];
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int e = rd + lane + 64 * c;
@@ -284,19 +320,44 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_strid
   float rstd = 1.f;
   if (w) rstd = rsqrtf(wave_sum(ss) / (float)d + eps);
   const float* cs = cos_sin ? cos_sin + (int64_t)pos * rotary_dim : nullptr;
+  float cv[2] = {1.f, 1.f}, sv[2] = {0.f, 0.f};
+  if (two) {
+    if (ok1) {
+      load2(cs + j, cv[0], cv[1]);
+      load2(cs + half + j, sv[0], sv[1]);
+    }
+  } else {
+    if (ok1) { cv[0] = cs[j]; sv[0] = cs[half + j]; }
+    if (ok2) { cv[1] = cs[j2]; sv[1] = cs[half + j2]; }
+  }
+  float o1[2], o2[2];
 #pragma unroll
   for (int c = 0; c < 2; ++c) {
-    const int j = lane + 64 * c;
-    if (j < half) {
-      const float cv = cs[j], sv = cs[half + j];
-      const float a = x1[c] * rstd * w1[c], b = x2[c] * rstd * w2[c];
-      const T o1 = from_float<T>(a * cv - b * sv);
-      const T o2 = from_float<T>(b * cv + a * sv);
-      src[j] = o1;
-      src[j + half] = o2;
+    const float a = xa[c] * rstd * wa[c], b2 = xb[c] * rstd * wb[c];
+    o1[c] = a * cv[c] - b2 * sv[c];
+    o2[c] = b2 * cv[c] + a * sv[c];
+  }
+  if (two) {
+    if (ok1) {
+      store2(src + j, o1[0], o1[1]);
+      store2(src + j + half, o2[0], o2[1]);
       if (dst) {
-        dst[j] = o1;
-        dst[j + half] = o2;
+        store2(dst + j, o1[0], o1[1]);
+        store2(dst + j + half, o2[0], o2[1]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int jj = c == 0 ? j : j2;
+      if (jj < half) {
+        const T a = from_float<T>(o1[c]), b2 = from_float<T>(o2[c]);
+        src[jj] = a;
+        src[jj + half] = b2;
+        if (dst) {
+          dst[jj] = a;
+          dst[jj + half] = b2;
+        }
       }
     }
   }
