@@ -371,15 +371,38 @@ __global__ __launch_bounds__(256) void prefill_kernel(
 // Partials: part_o [entries, nq, num_splits, D], part_ml [entries, nq, num_splits, 2] (max in base-2 units).
 constexpr int DECODE_WAVES = D > 128 ? 2 : 4;
 
+// With FRONT, the kernel also does what precedes attention for a decoded token (fused_qwen3.py:98-107 of the
+// reference): `q` is then the raw fused projection [tokens, (nq + 2 nkv) D] with rows q | k | v.  Every workgroup
+// norms and rotates its group's queries into LDS; the new key is normed and rotated there too.  The cached keys
+// are those before the new token; the new key and value enter the softmax from registers, in wave 0 of split 0,
+// which also writes them to their cache slot for later steps.
+struct DecodeFront {
+  const float* q_weight;     // [D] or null: per-head RMS norm weights
+  const float* k_weight;
+  float eps;
+  const float* cos_sin;      // [max_pos, rotary_dim] or null
+  int rotary_dim;
+  int max_pos;
+  const int* positions;      // [tokens]
+  const int* slots;          // [tokens] slot of each token's key and value: page * P + offset
+  uint16_t* k_pages;
+  uint16_t* v_pages;
+};
+
+__device__ __forceinline__ float bf16_at(const uint16_t* p) { return __uint_as_float((uint32_t)(*p) << 16); }
+
+template <bool FRONT>
 __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
     const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int first_entry,
     float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv, int page_shift, float scale,
-    int window) {
+    int window, DecodeFront front) {
   __shared__ float lds_o[DECODE_WAVES][DBLK][64][4];
   __shared__ float lds_m[DECODE_WAVES][16];
   __shared__ float lds_l[DECODE_WAVES][16];
+  __shared__ __attribute__((aligned(16))) uint16_t lds_q[FRONT ? 16 * D : 8];   // normed, rotated queries of the group
+  __shared__ __attribute__((aligned(16))) uint16_t lds_k[FRONT ? D : 8];        // and the new key
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int split = blockIdx.x, num_splits = gridDim.x;
@@ -391,38 +414,130 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
   const int kv = kv_len[b];
   const int pos = kv - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int last = FRONT ? pos - 1 : pos;   // last key that is read from the cache
   // this split's keys: macro tiles from the first visible one, evenly over the splits
-  const int tile_lo = lo / MKEYS, tile_hi = pos / MKEYS + 1;
+  const int tile_lo = lo / MKEYS, tile_hi = last < lo ? tile_lo : last / MKEYS + 1;
   const int tiles_per_split = (tile_hi - tile_lo + num_splits - 1) / num_splits;
   const int t0 = tile_lo + split * tiles_per_split;
   const int t1 = min(tile_hi, t0 + tiles_per_split);
   const int* bt = block_table + (int64_t)b * table_width;
   const float c = scale * 1.44269504088896340736f;
+  const int token = cu_q[b];
 
+  // the first macro tile's loads go out before anything else: nothing below depends on them until the products
+  bf16x8 ka[MT][QSTEPS];
+  s16x4 va[MT][DBLK];
+#define DECODE_FETCH(TILE)                                                                                           \
+  {                                                                                                                  \
+    const int j0_ = (TILE) * MKEYS;                                                                                  \
+    _Pragma("unroll") for (int t = 0; t < MT; ++t) { /* clamped addresses: masked keys read valid memory */         \
+      int kk = j0_ + 16 * t + (lane & 15);                                                                           \
+      kk = kk > pos ? pos : kk;                                                                                      \
+      const int64_t kpage = bt[kk >> page_shift];                                                                    \
+      load_row(ka[t], k_pages + ((kpage * nkv + g) * P + (kk & (P - 1))) * D, true);                                 \
+      int vk = j0_ + 16 * t + 4 * (lane >> 4);                                                                       \
+      vk = vk > pos ? (pos & ~3) : vk;                                                                               \
+      const int64_t vpage = bt[vk >> page_shift];                                                                    \
+      const uint16_t* vbase = v_pages + ((vpage * nkv + g) * D + (lane & 15)) * P + (vk & (P - 1));                  \
+      _Pragma("unroll") for (int blk = 0; blk < DBLK; ++blk)                                                         \
+          va[t][blk] = *reinterpret_cast<const s16x4*>(vbase + (int64_t)16 * blk * P);                               \
+    }                                                                                                                \
+  }
+  int mt = t0 + wave;
   State<1> st;
   init_state<1>(st);
   const bool col_ok = (lane & 15) < G;
   QRegs qr[1];
-  load_queries<1>(qr, q + (int64_t)cu_q[b] * q_row_stride, q_row_stride, 16, G, 1, g * G);
-  const int pos_lo[1] = {lo};
-  const int pos_hi[1] = {col_ok ? pos : -1};
-  for (int mt = t0 + wave; mt < t1; mt += DECODE_WAVES) {
-    const int j0 = mt * MKEYS;
-    bf16x8 ka[MT][QSTEPS];
-    s16x4 va[MT][DBLK];
+  if constexpr (FRONT) {
+    // Vector loads come back in the order they were issued, and the compiler can only wait for some of them in
+    // straight-line code.  So everything the norm and the rotation read is asked for first, without branches
+    // (absent operands read a stand-in address and are replaced afterwards), in two dependent rounds (the
+    // position, then its angles); the first macro tile is asked for after that, and the arithmetic runs while the
+    // tile is on its way.  Wave w takes heads w, w + DECODE_WAVES, ... of the group's query heads followed by
+    // its key head; a lane takes the rotation pairs (j, j + D/2), j = lane + 64 c.  Without a rotation table
+    // the pairs are "rotated" by the angle 0.
+    constexpr int HPW = (17 + DECODE_WAVES - 1) / DECODE_WAVES;
+    constexpr int HALF = D / 2;
+    constexpr int NP = (HALF + 63) / 64;
+    const uint16_t* row = q + (int64_t)token * q_row_stride;
+    const float* stand_in = reinterpret_cast<const float*>(row);      // at least D readable floats
+    const bool has_rope = front.cos_sin != nullptr, has_qw = front.q_weight != nullptr,
+               has_kw = front.k_weight != nullptr;
+    int rp = *(has_rope ? front.positions + token : cu_q + b);
+    float xa[HPW][NP], xb[HPW][NP];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {      // addresses clamped to the request's last key: masked keys read valid memory
-      int kk = j0 + 16 * t + (lane & 15);
-      kk = kk > pos ? pos : kk;
-      const int64_t kpage = bt[kk >> page_shift];
-      load_row(ka[t], k_pages + ((kpage * nkv + g) * P + (kk & (P - 1))) * D, true);
-      int vk = j0 + 16 * t + 4 * (lane >> 4);
-      vk = vk > pos ? (pos & ~3) : vk;
-      const int64_t vpage = bt[vk >> page_shift];
-      const uint16_t* vbase = v_pages + ((vpage * nkv + g) * D + (lane & 15)) * P + (vk & (P - 1));
+    for (int i = 0; i < HPW; ++i) {
+      const int hh = wave + DECODE_WAVES * i;
+      const uint16_t* src = row + (int64_t)(hh < G ? g * G + hh : nq + g) * D;
 #pragma unroll
-      for (int blk = 0; blk < DBLK; ++blk) va[t][blk] = *reinterpret_cast<const s16x4*>(vbase + (int64_t)16 * blk * P);
+      for (int cc = 0; cc < NP; ++cc) {
+        const int j = min(lane + 64 * cc, HALF - 1);
+        xa[i][cc] = bf16_at(src + j);
+        xb[i][cc] = bf16_at(src + j + HALF);
+      }
     }
+    float wqa[NP], wqb[NP], wka[NP], wkb[NP], cva[NP], sva[NP];
+    const float* qwp = has_qw ? front.q_weight : stand_in;
+    const float* kwp = has_kw ? front.k_weight : stand_in;
+#pragma unroll
+    for (int cc = 0; cc < NP; ++cc) {
+      const int j = min(lane + 64 * cc, HALF - 1);
+      wqa[cc] = qwp[j];
+      wqb[cc] = qwp[j + HALF];
+      wka[cc] = kwp[j];
+      wkb[cc] = kwp[j + HALF];
+    }
+    rp = rp < 0 ? 0 : (rp >= front.max_pos ? front.max_pos - 1 : rp);
+    const float* cs = has_rope ? front.cos_sin + (int64_t)rp * D : stand_in;
+#pragma unroll
+    for (int cc = 0; cc < NP; ++cc) {
+      const int j = min(lane + 64 * cc, HALF - 1);
+      cva[cc] = cs[j];
+      sva[cc] = cs[HALF + j];
+    }
+    DECODE_FETCH(min(mt, max(t1 - 1, t0)))      // a wave without a tile asks for one all the same and drops it
+#pragma unroll
+    for (int cc = 0; cc < NP; ++cc) {
+      if (!has_qw) wqa[cc] = wqb[cc] = 1.f;
+      if (!has_kw) wka[cc] = wkb[cc] = 1.f;
+      if (!has_rope) {
+        cva[cc] = 1.f;
+        sva[cc] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int hh = wave + DECODE_WAVES * i;
+      if (hh <= G) {                           // the same for every lane of the wave
+        const bool is_key = hh == G;
+        uint16_t* dst = is_key ? lds_k : lds_q + hh * D;
+        float ss = 0.f;
+#pragma unroll
+        for (int cc = 0; cc < NP; ++cc)
+          if (lane + 64 * cc < HALF) ss += xa[i][cc] * xa[i][cc] + xb[i][cc] * xb[i][cc];
+        const float rstd = (is_key ? has_kw : has_qw) ? rsqrtf(wave_sum(ss) / (float)D + front.eps) : 1.f;
+#pragma unroll
+        for (int cc = 0; cc < NP; ++cc) {
+          const int j = lane + 64 * cc;
+          if (j < HALF) {
+            const float a = xa[i][cc] * rstd * (is_key ? wka[cc] : wqa[cc]);
+            const float b2 = xb[i][cc] * rstd * (is_key ? wkb[cc] : wqb[cc]);
+            dst[j] = float_to_bf16_bits(a * cva[cc] - b2 * sva[cc]);
+            dst[j + HALF] = float_to_bf16_bits(b2 * cva[cc] + a * sva[cc]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    load_queries<1>(qr, lds_q, D, 16, G, 1, 0);
+  } else {
+    load_queries<1>(qr, q + (int64_t)token * q_row_stride, q_row_stride, 16, G, 1, g * G);
+    if (mt < t1) DECODE_FETCH(mt)
+  }
+  const int pos_lo[1] = {lo};
+  const int pos_hi[1] = {col_ok ? last : -1};
+  while (mt < t1) {
+    const int j0 = mt * MKEYS;
     f32x4 s[MT][1];
     s16x4 p[MT][1];
 #pragma unroll
@@ -430,6 +545,49 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
     softmax_update<1>(st, s, p, c, j0, pos_lo, pos_hi);
 #pragma unroll
     for (int t = 0; t < MT; ++t) tile_values<1>(st, va[t], p[t]);
+    mt += DECODE_WAVES;
+    if (mt < t1) DECODE_FETCH(mt)
+  }
+#undef DECODE_FETCH
+  if constexpr (FRONT) {
+    if (split == 0 && wave == 0) {
+      // the new token's own key and value: one more softmax step, from LDS and the projection's row
+      bf16x8 kn[QSTEPS];
+      load_row(kn, lds_k, true);
+      float dot = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < QSTEPS; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dot += (float)qr[0].full[ks][i] * (float)kn[ks][i];
+      dot += __shfl_xor(dot, 16, 64);
+      dot += __shfl_xor(dot, 32, 64);
+      const float v = col_ok ? dot * c : -INFINITY;
+      const float m_new = fmaxf(st.m[0], v);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_use);
+      const float pe = __builtin_amdgcn_exp2f(v - m_use);
+      const float pr = __uint_as_float((uint32_t)float_to_bf16_bits(pe) << 16);   // rounded like the tiles' P
+      st.l[0] = st.l[0] * alpha + ((lane >> 4) == 0 ? pe : 0.f);
+      st.m[0] = m_new;
+      const uint16_t* vrow = q + (int64_t)token * q_row_stride + (int64_t)(nq + nkv + g) * D;
+      const int slot = front.slots[token];
+      const int64_t page = slot >> page_shift;
+      const int off = slot & (P - 1);
+#pragma unroll
+      for (int blk = 0; blk < DBLK; ++blk) {
+        const s16x4 vv = *reinterpret_cast<const s16x4*>(vrow + 16 * blk + 4 * (lane >> 4));
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          st.o[0][blk][i] = st.o[0][blk][i] * alpha + pr * __uint_as_float((uint32_t)(uint16_t)vv[i] << 16);
+      }
+      // the cache copies: the key's row, and the value's elements into the transposed page
+      uint16_t* kdst = front.k_pages + ((page * nkv + g) * P + off) * D;
+      uint16_t* vdst = front.v_pages + (page * nkv + g) * (int64_t)D * P + off;
+      for (int i = lane; i < D; i += 64) {
+        kdst[i] = lds_k[i];
+        vdst[(int64_t)i * P] = vrow[i];
+      }
+    }
   }
   // ---- combine the waves: every wave leaves its state in LDS
   float l = st.l[0];
@@ -612,15 +770,53 @@ MI_EXPORT int mi_attn_decode(const void* q, int64_t q_row_stride, void* out, int
   MI_REQUIRE(num_splits == 1 || (part_o && part_ml), "attn_decode: no partial buffers");
   if (num_entries == 0) return 0;
   dim3 grid(num_splits, nkv, num_entries);
-  decode_kernel<<<grid, 64 * DECODE_WAVES, 0, stream>>>(
+  decode_kernel<false><<<grid, 64 * DECODE_WAVES, 0, stream>>>(
       (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
       (const uint16_t*)v_pages, block_table, table_width, cu_q, kv_len, first_entry, part_o, part_ml, nq, nkv,
-      log2_of(page_size), scale, window);
+      log2_of(page_size), scale, window, DecodeFront{});
   MI_CHECK_LAUNCH("attn_decode");
   if (num_splits > 1) {
     decode_merge_kernel<<<num_entries * nq, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q,
                                                              first_entry, nq, num_splits);
     MI_CHECK_LAUNCH("attn_decode merge");
+  }
+  return 0;
+}
+
+// The same for entries whose projection has not been normed, rotated or cached yet: qkv [tokens, >= (nq + 2 nkv) D]
+// holds rows q | k | v of the fused projection; q_weight / k_weight [D] float32 or null; cos_sin [max_pos, rotary_dim]
+// float32 or null; positions and slots per token.  The new keys and values are written to their slots.
+MI_EXPORT int mi_attn_decode_front(const void* qkv, int64_t qkv_row_stride, void* out, int64_t out_row_stride,
+                                   void* k_pages, void* v_pages, const int* block_table, int table_width,
+                                   const int* cu_q, const int* kv_len, int first_entry, int num_entries, int num_splits,
+                                   float* part_o, float* part_ml, int nq, int nkv, int page_size, float scale,
+                                   int window, const float* q_weight, const float* k_weight, float eps,
+                                   const float* cos_sin, int rotary_dim, int max_pos, const int* positions,
+                                   const int* slots, hipStream_t stream) {
+  if (check_common("attn_decode_front", nq, nkv, page_size, qkv_row_stride, out_row_stride, table_width)) return 1;
+  MI_REQUIRE(qkv_row_stride >= (int64_t)(nq + 2 * nkv) * D, "attn_decode_front: row stride %lld holds no q | k | v",
+             (long long)qkv_row_stride);
+  MI_REQUIRE(num_entries >= 0 && first_entry >= 0 && window >= 0, "attn_decode_front: bad entry range or window");
+  MI_REQUIRE(num_splits >= 1 && num_splits <= 1024, "attn_decode_front: %d splits", num_splits);
+  MI_REQUIRE(num_entries <= 65535 && nkv <= 65535, "attn_decode_front: grid too large");
+  MI_REQUIRE(num_splits == 1 || (part_o && part_ml), "attn_decode_front: no partial buffers");
+  MI_REQUIRE(slots && k_pages && v_pages, "attn_decode_front: no cache slots");
+  if (cos_sin)
+    MI_REQUIRE(rotary_dim == D && positions && max_pos > 0,
+               "attn_decode_front: rotary_dim %d; this kernel rotates whole heads of %d only", rotary_dim, D);
+  if (num_entries == 0) return 0;
+  DecodeFront front{q_weight, k_weight, eps, cos_sin, rotary_dim, max_pos, positions, slots, (uint16_t*)k_pages,
+                    (uint16_t*)v_pages};
+  dim3 grid(num_splits, nkv, num_entries);
+  decode_kernel<true><<<grid, 64 * DECODE_WAVES, 0, stream>>>(
+      (const uint16_t*)qkv, qkv_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
+      (const uint16_t*)v_pages, block_table, table_width, cu_q, kv_len, first_entry, part_o, part_ml, nq, nkv,
+      log2_of(page_size), scale, window, front);
+  MI_CHECK_LAUNCH("attn_decode_front");
+  if (num_splits > 1) {
+    decode_merge_kernel<<<num_entries * nq, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q,
+                                                             first_entry, nq, num_splits);
+    MI_CHECK_LAUNCH("attn_decode_front merge");
   }
   return 0;
 }

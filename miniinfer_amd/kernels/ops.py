@@ -94,6 +94,9 @@ _SIGS["attention_mfma"] = {
                       c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
   "mi_attn_decode": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                      c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
+  "mi_attn_decode_front": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                           c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int,
+                           c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
   "mi_attn_prefill_tokens_per_block": [c_int, c_int],
 }
 
@@ -486,3 +489,43 @@ def attn_decode(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k
                                  _ptr(block_table), block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry,
                                  num_entries, num_splits, _ptr(part_o), _ptr(part_ml), nq, nkv, k_pages.shape[2],
                                  float(scale), int(window), _stream()))
+
+
+def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
+                      v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor, kv_len: torch.Tensor,
+                      first_entry: int, num_entries: int, num_splits: int, part_o: torch.Tensor,
+                      part_ml: torch.Tensor, scale: float, window: int, q_weight: Optional[torch.Tensor],
+                      k_weight: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
+                      positions: torch.Tensor, slots: torch.Tensor) -> None:
+  """`attn_decode` for entries whose fused projection qkv [T, (nq + 2 nkv) d] (rows q | k | v) is still raw: the
+  kernel does the per-head RMS norm of q and k (if weights), their rotation (if a table [max_pos, rotary_dim]) and
+  the write of the new key and value to `slots`, as `qk_norm_rope_cache` would, and attends.  qkv is left as it is.
+  A table must rotate whole heads (rotary_dim == d)."""
+  B = _attn_common("attn_decode_front", qkv, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len)
+  T = qkv.shape[0]
+  if qkv.shape[1] != (nq + 2 * nkv) * d:
+    raise KernelError(f"attn_decode_front: qkv {tuple(qkv.shape)} does not hold {nq}+2*{nkv} heads of {d}")
+  if first_entry < 0 or num_entries < 0 or first_entry + num_entries > B:
+    raise KernelError(f"attn_decode_front: entries {first_entry}..{first_entry + num_entries} of {B}")
+  _dev(part_o, part_ml, q_weight, k_weight, cos_sin, positions, slots)
+  need = num_entries * nq * num_splits
+  if part_o.dtype != torch.float32 or part_o.numel() < need * d or part_ml.dtype != torch.float32 \
+      or part_ml.numel() < need * 2 or not part_o.is_contiguous() or not part_ml.is_contiguous():
+    raise KernelError("attn_decode_front: partial buffers are too small or not float32")
+  _f32("q_weight", q_weight, d)
+  _f32("k_weight", k_weight, d)
+  _i32("slots", slots, T)
+  rotary_dim, max_pos = 0, 0
+  if cos_sin is not None:
+    if cos_sin.dtype != torch.float32 or cos_sin.dim() != 2 or not cos_sin.is_contiguous():
+      raise KernelError("attn_decode_front: the rotation table must be a contiguous float32 [positions, rotary_dim]")
+    max_pos, rotary_dim = cos_sin.shape
+    if rotary_dim != d:
+      raise KernelError(f"attn_decode_front: rotary_dim {rotary_dim}; this kernel rotates whole heads of {d} only")
+    _i32("positions", positions, T)
+  lib = _lib("attention_mfma", (("HEAD_DIM", d),))
+  _check(lib, lib.mi_attn_decode_front(
+    _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+    block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry, num_entries, num_splits, _ptr(part_o), _ptr(part_ml),
+    nq, nkv, k_pages.shape[2], float(scale), int(window), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin),
+    rotary_dim, max_pos, _ptr(positions), _ptr(slots), _stream()))

@@ -66,6 +66,12 @@ class PagedAttention(Part):
     qkv = linear(x, self.qkv_weight)
     table = self.position.rotary_table()
     eps = self.q_norm.eps if self.q_norm is not None else 0.0
+    if ctx.num_multi == 0 and not self.shares_kv and (table is None or table.shape[1] == self.d) and \
+        ops.mfma_attention_supported(qkv.dtype, self.nq, self.nkv, self.d, cache.page_size):
+      # a step of decoded tokens only: the attention kernel norms, rotates and caches by itself
+      out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
+      self._attend_decode(qkv, out, ctx, cache, 0, ctx.num_requests, front=(table, eps))
+      return linear(out, self.o_weight)
     if self.shares_kv:
       # only queries of its own: they are normed and rotated; the borrowed pages are read, never written
       ops.qk_norm_rope_cache(qkv, self.nq, 0, self.d, self.q_norm.weight if self.q_norm is not None else None, None,
@@ -93,14 +99,27 @@ class PagedAttention(Part):
       ops.attn_prefill(qkv, nq, nkv, d, out, cache.k, cache.v, table, work, ctx.cu_q, ctx.kv_len, self.scale, window)
     n_single = ctx.num_requests - ctx.num_multi
     if n_single > 0:
-      tile_keys, waves = ops.attn_decode_geometry(d)
-      splits = decode_splits(n_single * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len, tile_keys,
-                             waves)
-      need = n_single * nq * splits
-      part_o = ctx.scratch("attn_part_o", need * d, torch.float32)
-      part_ml = ctx.scratch("attn_part_ml", need * 2, torch.float32)
-      ops.attn_decode(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, ctx.num_multi, n_single,
-                      splits, part_o, part_ml, self.scale, window)
+      self._attend_decode(qkv, out, ctx, cache, ctx.num_multi, n_single)
+
+  def _attend_decode(self, qkv, out, ctx, cache, first: int, count: int, front=None) -> None:
+    """Entries first .. first + count - 1, one token each.  With `front` = (rotation table, eps) the projection is
+    still raw and the kernel does the head norms, the rotation and the cache write too."""
+    nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0
+    table = ctx.block_tables[cache.group]
+    tile_keys, waves = ops.attn_decode_geometry(d)
+    splits = decode_splits(count * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len, tile_keys, waves)
+    need = count * nq * splits
+    part_o = ctx.scratch("attn_part_o", need * d, torch.float32)
+    part_ml = ctx.scratch("attn_part_ml", need * 2, torch.float32)
+    if front is None:
+      ops.attn_decode(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, first, count, splits,
+                      part_o, part_ml, self.scale, window)
+    else:
+      ops.attn_decode_front(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, first, count, splits,
+                            part_o, part_ml, self.scale, window,
+                            self.q_norm.weight if self.q_norm is not None else None,
+                            self.k_norm.weight if self.k_norm is not None else None,
+                            front[1], front[0], ctx.positions, ctx.slots[cache.group])
 
 
 def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, waves: int = 4,

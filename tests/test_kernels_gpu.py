@@ -366,3 +366,71 @@ def test_norm_gemm_skinny(M, N, K, with_x, gate_up):
   out2 = torch.empty(2, N, dtype=torch.bfloat16, device=DEV)
   ops.norm_gemm_skinny(r, x, nw, 1e-5, w, out2, rows=rows, gate_up=gate_up)
   torch.testing.assert_close(out2.double(), want[rows.long()], rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("splits", [1, 4])
+@pytest.mark.parametrize("with_norm,rd_of", [(True, 1.0), (False, 1.0), (True, 0.5), (True, 0.0)])
+@pytest.mark.parametrize("nq,nkv,d,P,window", MFMA_SHAPES)
+def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, window, with_norm, rd_of, splits):
+  """The decode kernel that takes the raw projection: against head norm, rotation and attention done one after the
+  other in 32-bit on the host, with the new key rounded to bfloat16 as the cache holds it.  The slot of the new
+  token holds stale numbers before the call and the new key and value after it."""
+  from miniinfer_amd.kernels import ops
+  reqs = [(129, 1), (0, 1), (15, 1), (16, 1), (700, 1), (63, 1), (1, 1)]
+  c = _paged_case(reqs, nq, nkv, d, P, window, seed=9)
+  g = torch.Generator().manual_seed(10)
+  B, max_pos, theta, eps = len(reqs), 800, 5000.0, 2e-6
+  rd = int(d * rd_of) // 2 * 2
+  qw = (1 + 0.1 * torch.randn(d, generator=g)) if with_norm else None
+  kw = (1 + 0.1 * torch.randn(d, generator=g)) if with_norm else None
+  pos = torch.tensor([past for past, _ in reqs])
+  table_host = c["table"].cpu()
+  slots = torch.tensor([int(table_host[b, past // P]) * P + past % P for b, (past, _) in enumerate(reqs)])
+  cos_sin = None
+  if rd:
+    j = torch.arange(0, rd, 2, dtype=torch.float32)
+    ang = torch.outer(torch.arange(max_pos, dtype=torch.float32), 1.0 / theta ** (j / rd))
+    cos_sin = torch.cat((ang.cos(), ang.sin()), -1).to(DEV)
+
+  raw = c["q"].float().cpu().view(B, nq + 2 * nkv, d)
+  q, k, v = raw[:, :nq], raw[:, nq:nq + nkv], raw[:, nq + nkv:]
+  if with_norm:
+    q = torch.nn.functional.rms_norm(q, (d,), qw, eps)
+    k = torch.nn.functional.rms_norm(k, (d,), kw, eps)
+  if rd:
+    q, k = _rope_ref(q, pos, theta, rd), _rope_ref(k, pos, theta, rd)
+  q, k = q.bfloat16().float(), k.bfloat16().float()
+  kp, vp = c["kp"].clone(), c["vp"].clone()
+  kc, vc = kp.float().cpu(), vp.float().cpu().transpose(2, 3)      # [pages, nkv, P, d]
+  want = []
+  for b, (past, _) in enumerate(reqs):
+    pages = table_host[b, :past // P + 1].tolist()
+    kk = torch.cat([kc[p].transpose(0, 1) for p in pages], 0)[:past]
+    vv = torch.cat([vc[p].transpose(0, 1) for p in pages], 0)[:past]
+    kk, vv = torch.cat((kk, k[b][None]), 0), torch.cat((vv, v[b][None]), 0)
+    want.append(_attention_ref(q[b][None], kk, vv, d ** -0.5, window).reshape(1, nq * d))
+  want = torch.cat(want, 0)
+
+  out = torch.zeros(B, nq * d, dtype=torch.bfloat16, device=DEV)
+  part_o = torch.empty(B * nq * splits * d, dtype=torch.float32, device=DEV)
+  part_ml = torch.empty(B * nq * splits * 2, dtype=torch.float32, device=DEV)
+  before = c["q"].clone()
+  if 0 < rd < d:                                         # a partly rotated head is refused, not miscomputed
+    with pytest.raises(ops.KernelError, match="whole heads"):
+      ops.attn_decode_front(c["q"], nq, nkv, d, out, kp, vp, c["table"], c["cu"], c["kv"], 0, B, splits, part_o,
+                            part_ml, d ** -0.5, window, None, None, eps, cos_sin, pos.to(torch.int32).to(DEV),
+                            slots.to(torch.int32).to(DEV))
+    return
+  ops.attn_decode_front(c["q"], nq, nkv, d, out, kp, vp, c["table"], c["cu"], c["kv"], 0, B, splits, part_o, part_ml,
+                        d ** -0.5, window, qw.to(DEV) if with_norm else None, kw.to(DEV) if with_norm else None, eps,
+                        cos_sin, pos.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV))
+  torch.testing.assert_close(out.double().cpu(), want.double(), rtol=1.6e-2, atol=1e-2)
+  assert torch.equal(c["q"], before)                     # the projection is read only
+  k_after, v_after = kp.float().cpu(), vp.float().cpu().transpose(2, 3)
+  changed_k = (k_after != kc).any(-1)
+  for b in range(B):
+    page, off = int(slots[b]) // P, int(slots[b]) % P
+    torch.testing.assert_close(k_after[page, :, off], k[b], rtol=1e-2, atol=1e-2)
+    assert torch.equal(v_after[page, :, off], v[b])
+    changed_k[page, :, off] = False
+  assert not bool(changed_k.any())                       # no other slot was written
