@@ -36,6 +36,7 @@ class EngineConfig:
   max_num_batched_tokens: int = 8192          # token budget of one step (reference: max_extend_len)
   enable_chunked_prefill: bool = True
   enforce_eager: bool = False                 # True: never replay decode steps from HIP graphs
+  enable_overlap: bool = True                 # launch a step before the last one's tokens are read back
   eos: Optional[int] = None                   # None: from config.json
   seed: int = 0
   device: str = "cuda:0"

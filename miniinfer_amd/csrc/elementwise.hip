@@ -9,11 +9,14 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding
+// A negative id -(r + 1) stands for a token that an earlier kernel on the stream left in future[r] (the row of the
+// last step's sampling output): the engine launches a step before it has read the tokens of the one before.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
-                             int H, int V) {
+                             int H, int V, const int* __restrict__ future, int num_future) {
   const int t = blockIdx.x;
-  const int id = ids[t];
+  int id = ids[t];
+  if (id < 0 && future && -(id + 1) < num_future) id = future[-(id + 1)];
   const bool ok = id >= 0 && id < V;
   const T* row = table + (int64_t)(ok ? id : 0) * H;
   float* o = out + (int64_t)t * H;
@@ -21,14 +24,14 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
 }
 
 MI_EXPORT int mi_embed(int dtype, const void* table, const int* ids, float* out, int T, int H, int V,
-                       hipStream_t stream) {
-  MI_REQUIRE(T >= 0 && H > 0 && V > 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+                       const int* future, int num_future, hipStream_t stream) {
+  MI_REQUIRE(T >= 0 && H > 0 && V > 0 && num_future >= 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
   if (T == 0) return 0;
   const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
   if (dtype == MI_DTYPE_F32)
-    embed_kernel<float><<<T, threads, 0, stream>>>((const float*)table, ids, out, H, V);
+    embed_kernel<float><<<T, threads, 0, stream>>>((const float*)table, ids, out, H, V, future, num_future);
   else if (dtype == MI_DTYPE_BF16)
-    embed_kernel<bf16><<<T, threads, 0, stream>>>((const bf16*)table, ids, out, H, V);
+    embed_kernel<bf16><<<T, threads, 0, stream>>>((const bf16*)table, ids, out, H, V, future, num_future);
   else
     MI_FAIL("embed: unknown dtype %d", dtype);
   MI_CHECK_LAUNCH("embed");

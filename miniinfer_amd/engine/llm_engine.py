@@ -7,7 +7,10 @@
       outs[0]["token_ids"], outs[0]["text"]
 
 Prompts are lists of token ids (always) or strings (when the model folder holds a tokenizer.json).
-One synchronous loop: schedule, step, sample, update; no processes, no server.
+One loop: schedule, step, sample, update; no processes, no server.  With `enable_overlap` (the default, as in the
+reference: config/engine/config.py:8-77, llm_engine.py:559-700) a step is launched before the tokens of the step
+before it have been read back: they stay on the device, the new step's embedding reads them there, and the host
+catches up while the device works.  What `step()` returns then describes the step before the one it launched.
 """
 
 from __future__ import annotations
@@ -74,6 +77,10 @@ class LLMEngine:
     self._next_number = 0
     self._requests: Dict[str, Request] = {}
     self.num_steps = 0
+    # the launched step whose tokens have not been read back yet: (plan, requests that sample, host buffer, event)
+    self._pending = None
+    self._token_bufs = [torch.zeros(max(1, cfg.max_num_seqs), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+    self._token_turn = 0
 
   # ------------------------------------------------------------------ set-up helpers
   def _pages_from_memory(self, needs) -> int:
@@ -142,17 +149,14 @@ class LLMEngine:
     return rid
 
   def is_finished(self) -> bool:
-    return not self.scheduler.has_unfinished()
+    return self._pending is None and not self.scheduler.has_unfinished()
 
   has_unfinished = property(lambda self: self.scheduler.has_unfinished())
 
   # ------------------------------------------------------------------ one step
-  def step(self) -> StepOutput:
-    """schedule -> run the batch -> sample -> update (miniinfer/engine/llm_engine.py:465-557)."""
-    plan = self.scheduler.schedule()
-    out = StepOutput()
-    if plan is None:
-      return out
+  def _launch(self, plan: ScheduledStep):
+    """Runs the plan's batch and samples, all of it queued on the device; the tokens go to the runner's
+    `future_tokens` and, by a copy that an event marks, to a pinned host buffer."""
     entries = []
     sampling = []
     for e in plan.entries:
@@ -160,17 +164,49 @@ class LLMEngine:
       entries.append(StepEntry(req=e.request.number, tokens=toks, want=[e.num_tokens - 1] if e.samples else []))
       if e.samples:
         sampling.append(e.request)
-    logits = self.runner.step(entries)
+    logits = self.runner.step(entries, allow_future=True)
+    host = event = None
+    if sampling:
+      R = len(sampling)
+      dev = self.runner.future_tokens[:R]
+      self.sampler.sample_into(logits, [r.params for r in sampling], [r.seed for r in sampling],
+                               [len(r.outputs) for r in sampling], dev)
+      self._token_turn ^= 1
+      host = self._token_bufs[self._token_turn][:R]
+      host.copy_(dev, non_blocking=True)
+      event = torch.cuda.Event()
+      event.record()
+    self.scheduler.advance(plan)
+    self.num_steps += 1
+    return plan, sampling, host, event
+
+  def _resolve(self, pending, out: StepOutput) -> None:
+    """Reads a launched step's tokens (waiting for them if need be) and books them."""
+    plan, sampling, host, event = pending
     sampled: Dict[int, int] = {}
     if sampling:
-      toks = self.sampler.sample(logits, [r.params for r in sampling], [r.seed for r in sampling],
-                                 [len(r.outputs) for r in sampling])
-      sampled = {r.number: t for r, t in zip(sampling, toks)}
-    out.finished = self.scheduler.update(plan, sampled)
-    out.num_prefill_tokens = plan.num_prefill_tokens
-    out.num_decode_tokens = plan.num_decode_tokens
-    out.num_preempted = len(plan.preempted)
-    self.num_steps += 1
+      event.synchronize()
+      sampled = {r.number: t for r, t in zip(sampling, host.tolist())}
+    out.finished += self.scheduler.resolve(plan, sampled)
+    out.num_prefill_tokens += plan.num_prefill_tokens
+    out.num_decode_tokens += plan.num_decode_tokens
+    out.num_preempted += len(plan.preempted)
+
+  def step(self) -> StepOutput:
+    """schedule -> run the batch -> sample -> update (miniinfer/engine/llm_engine.py:465-557); with
+    `enable_overlap`, schedule and launch the next step, then read and book the tokens of the one before
+    (llm_engine.py:559-700).  Returns what the booked step did."""
+    out = StepOutput()
+    if not self.config.enable_overlap:
+      plan = self.scheduler.schedule()
+      if plan is not None:
+        self._resolve(self._launch(plan), out)
+      return out
+    plan = self.scheduler.schedule()
+    launched = self._launch(plan) if plan is not None else None
+    if self._pending is not None:
+      self._resolve(self._pending, out)
+    self._pending = launched
     return out
 
   # ------------------------------------------------------------------ generate

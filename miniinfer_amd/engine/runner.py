@@ -45,6 +45,7 @@ class StepContext:
     self.kv_len: torch.Tensor = None         # [B] int32, keys per request after this step
     self.req_slots: torch.Tensor = None      # [B] int32, state slot of each request
     self.logit_rows: torch.Tensor = None     # [R] int32, flattened token rows whose logits are wanted
+    self.future_tokens: Optional[torch.Tensor] = None   # int32: a token id -(r + 1) stands for future_tokens[r]
     self.slots: List[torch.Tensor] = []      # per paged group: [T] int32, page * page_size + offset
     self.block_tables: List[torch.Tensor] = []   # per paged group: [B, W] int32
     # host copies
@@ -124,18 +125,24 @@ class _DecodeGraph:
     cache = runner.cache
     G = len(cache.paged)
     self.layout = _Layout(T=B, B=B, R=B, G=G, W=W)
-    self.stage = torch.zeros(self.layout.total, dtype=torch.int32, pin_memory=True)
-    self.host = self.layout.views(self.stage.numpy())
-    # what never changes: one token per entry, every row's logits
-    self.host["token_req"][:] = np.arange(B, dtype=np.int32)
-    self.host["cu_q"][:] = np.arange(B + 1, dtype=np.int32)
-    self.host["logit_rows"][:] = np.arange(B, dtype=np.int32)
-    self.fill_padding(0)
+    # two pinned staging buffers, used in turn: the copy of one step may still be queued on the stream while the
+    # host lays out the next step (the engine reads a step's tokens only after it has launched the next one)
+    self.stages = [torch.zeros(self.layout.total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+    self.hosts = [self.layout.views(st.numpy()) for st in self.stages]
+    self.turn = 0
+    for self.host in self.hosts:
+      # what never changes: one token per entry, every row's logits
+      self.host["token_req"][:] = np.arange(B, dtype=np.int32)
+      self.host["cu_q"][:] = np.arange(B + 1, dtype=np.int32)
+      self.host["logit_rows"][:] = np.arange(B, dtype=np.int32)
+      self.fill_padding(0)
+    self.stage = self.stages[0]
     self.dev = torch.zeros(self.layout.total, dtype=torch.int32, device=runner.device)
     self.dev.copy_(self.stage)
     ctx = self.layout.context(self.dev, cache, runner.device)
     ctx.q_lens, ctx.kv_lens = [1] * B, [W * cache.page_size] * B   # host-side sizes the kernels are tuned for
     ctx.num_multi, ctx.max_q_len, ctx.max_kv_len = 0, 1, W * cache.page_size
+    ctx.future_tokens = runner.future_tokens
     self.ctx = ctx
     # every entry is padding while warming up and capturing: it reads and writes the scratch page only
     side = torch.cuda.Stream(device=runner.device)
@@ -159,6 +166,12 @@ class _DecodeGraph:
     h["slots"].reshape(G, B)[:, first:] = 0
     h["tables"].reshape(G, B, W)[:, first:, :] = 0
 
+  def next_host(self):
+    """The staging views to lay the next step out in."""
+    self.turn ^= 1
+    self.stage, self.host = self.stages[self.turn], self.hosts[self.turn]
+    return self.host
+
   def run(self) -> torch.Tensor:
     self.dev.copy_(self.stage, non_blocking=True)
     self.graph.replay()
@@ -178,7 +191,12 @@ class ModelRunner:
     self.vocab_size = model.spec.vocab_size
     self.use_graphs = use_graphs and self.device.type == "cuda"
     self._staging: Optional[torch.Tensor] = None
+    self._allow_future = False
     self._graphs: Dict[tuple, _DecodeGraph] = {}
+    # Tokens of the last step's sampling output, by row.  A token id -(r + 1) in a step's entries stands for
+    # future_tokens[r] as it is when the step's embedding kernel runs: whoever samples writes here, and may
+    # launch the next step before reading the tokens back.
+    self.future_tokens = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=self.device)
 
   # ------------------------------------------------------------------ host side of a step
   def _stage(self, n: int) -> torch.Tensor:
@@ -207,7 +225,7 @@ class ModelRunner:
         if not 0 <= w < len(e.tokens):
           raise IndexError(f"request {e.req!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
       for t in e.tokens:
-        if not 0 <= t < self.vocab_size:
+        if not (0 <= t < self.vocab_size or (self._allow_future and -self.future_tokens.numel() <= t < 0)):
           raise ValueError(f"request {e.req!r}: token id {t} is outside [0, {self.vocab_size})")
     order = sorted(range(len(entries)), key=lambda i: 0 if len(entries[i].tokens) > 1 else 1)
     q_lens = [len(entries[i].tokens) for i in order]
@@ -269,13 +287,16 @@ class ModelRunner:
     ctx.q_lens, ctx.kv_lens = q_lens, kv_lens
     ctx.num_multi = sum(1 for n in q_lens if n > 1)
     ctx.max_q_len, ctx.max_kv_len = max(q_lens), max(kv_lens)
+    ctx.future_tokens = self.future_tokens
     return ctx, order, kv_lens
 
   # ------------------------------------------------------------------ the step
   @torch.no_grad()
-  def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+  def step(self, entries: Sequence[StepEntry], allow_future: bool = False) -> torch.Tensor:
     """Runs the entries as one batch.  Returns float32 logits [number of wanted places, vocab] on the
-    device, in the order of the entries and of each entry's `want`."""
+    device, in the order of the entries and of each entry's `want`.  With `allow_future`, a token id -(r + 1)
+    is taken from `future_tokens[r]` on the device."""
+    self._allow_future = allow_future
     if self.use_graphs and len(entries) <= _GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries):
       return self._step_from_graph(entries)
     ctx, order, kv_lens = self.build_context(entries)
@@ -297,7 +318,7 @@ class ModelRunner:
     if g is None:
       g = _DecodeGraph(self, Bb, Wb)
       self._graphs[(Bb, Wb)] = g
-    self._fill(g.host, g.layout, entries, order, q_lens, starts, kv_lens)
+    self._fill(g.next_host(), g.layout, entries, order, q_lens, starts, kv_lens)
     g.fill_padding(B)
     logits = g.run()
     for i, kv in zip(order, kv_lens):

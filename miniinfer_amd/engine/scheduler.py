@@ -15,6 +15,12 @@ and slot are given back and it returns to the head of the waiting queue, keeping
 when it is admitted again it recomputes prompt + outputs as one prompt.  Admission of new requests
 stops while running requests cannot grow.  A request that could never fit the pool alone is refused
 when it is added.
+
+Results come back in two halves, so that the engine can launch the next step before it has read the
+tokens of the last one (the reference's overlap mode schedules step N+1 against placeholders for step N's
+tokens too: miniinfer/engine/future_map.py:1-206, llm_engine.py:559-700): `advance` moves the lengths on
+and appends a placeholder for each token to come (a negative id that names the row of the step's sampling
+output), `resolve` writes the tokens in and finishes requests.  `update` is both at once.
 """
 
 from __future__ import annotations
@@ -37,10 +43,29 @@ class Request:
   num_computed: int = 0           # tokens whose keys and values are in the cache
   finish_reason: Optional[str] = None
   num_preemptions: int = 0
+  pending: int = 0                # sampled tokens that are still placeholders
+  _tokens: Optional[List[int]] = field(default=None, repr=False, compare=False)
 
   @property
   def tokens(self) -> List[int]:
-    return self.prompt + self.outputs
+    """prompt + outputs, kept as one list (it is sliced every step)."""
+    if self._tokens is None or len(self._tokens) != len(self.prompt) + len(self.outputs):
+      self._tokens = self.prompt + self.outputs
+    return self._tokens
+
+  def append_output(self, tok: int) -> None:
+    toks = self.tokens
+    self.outputs.append(tok)
+    toks.append(tok)
+
+  def set_output(self, index: int, tok: int) -> None:
+    toks = self.tokens
+    self.outputs[index] = tok
+    toks[len(self.prompt) + index] = tok
+
+  def truncate_outputs(self, count: int) -> None:
+    del self.outputs[count:]
+    self._tokens = None
 
   @property
   def num_tokens(self) -> int:
@@ -61,6 +86,7 @@ class ScheduledEntry:
   start: int                      # position of the first token of this portion
   num_tokens: int
   samples: bool                   # the portion ends the known tokens: its last logits pick the next token
+  output_index: int = -1          # where in the request's outputs its sampled token goes (set by `advance`)
 
 
 @dataclass
@@ -94,6 +120,9 @@ class Scheduler:
     self.running: List[Request] = []      # in order of admission
     self.finished: List[Request] = []
     self.num_preemptions = 0
+    self.num_unresolved = 0               # sampled tokens launched and not yet written in
+    self._draining: List[Request] = []    # finished, pages still held until their last token is written in
+    self._retired_unadmitted: List[Request] = []
 
   # ------------------------------------------------------------------ requests in
   def add(self, req: Request) -> None:
@@ -114,7 +143,7 @@ class Scheduler:
     self.waiting.append(req)
 
   def has_unfinished(self) -> bool:
-    return bool(self.waiting or self.running)
+    return bool(self.waiting or self.running or self.num_unresolved)
 
   # ------------------------------------------------------------------ one step's plan
   def _pages_for(self, req: Request, new_len: int) -> int:
@@ -129,7 +158,7 @@ class Scheduler:
     self.waiting.appendleft(req)
 
   def schedule(self) -> Optional[ScheduledStep]:
-    if not self.has_unfinished():
+    if not (self.waiting or self.running):
       return None
     budget = self.max_num_batched_tokens
     free = self.cache.num_free_pages()
@@ -185,6 +214,8 @@ class Scheduler:
       budget -= n
 
     if not entries:
+      if self._draining:
+        return None       # finished requests give their pages back as soon as their last token is written in
       if self.running or self.waiting:
         # nothing fits: every running request is stuck on pages and none can be preempted further
         if len(self.running) > 1:
@@ -206,26 +237,69 @@ class Scheduler:
     return max(n, 0)
 
   # ------------------------------------------------------------------ results in
-  def update(self, step: ScheduledStep, sampled: Dict[int, int]) -> List[Request]:
-    """After the step ran: `sampled[request.number]` is the next token of every entry that samples.
-    Returns the requests that finished; their pages and slots are given back here."""
-    done = []
+  def advance(self, step: ScheduledStep) -> None:
+    """The step has been launched: its tokens count as computed, and every entry that samples gets a placeholder
+    -(row + 1) for its token, `row` being its place among the sampling entries of the step.  A request that
+    reaches max_tokens or the model's length with this token leaves the running list now; its pages stay until
+    the token is written in."""
+    row = 0
     for e in step.entries:
       r = e.request
       r.num_computed += e.num_tokens
       if not e.samples:
         continue
-      tok = int(sampled[r.number])
-      r.outputs.append(tok)
-      if not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id:
-        r.finish_reason = "eos"
-      elif len(r.outputs) >= r.params.max_tokens:
-        r.finish_reason = "max_tokens"
-      elif r.num_tokens >= self.max_model_len:
-        r.finish_reason = "length"
-      if r.finished:
-        self.cache.release(r.number)
-        self.running.remove(r)
+      e.output_index = len(r.outputs)
+      r.append_output(-(row + 1))
+      r.pending += 1
+      self.num_unresolved += 1
+      row += 1
+      if r.finish_reason is None:
+        if len(r.outputs) >= r.params.max_tokens:
+          r.finish_reason = "max_tokens"
+        elif r.num_tokens >= self.max_model_len:
+          r.finish_reason = "length"
+        if r.finished and r in self.running:
+          self.running.remove(r)
+          self._draining.append(r)
+
+  def resolve(self, step: ScheduledStep, sampled: Dict[int, int]) -> List[Request]:
+    """`sampled[request.number]` is the token of every entry of `step` that samples.  Writes the tokens in place
+    of their placeholders, ends requests at their end-of-sequence token (placeholders launched after it are
+    dropped), and returns the requests that are finished and have no token outstanding; their pages and slots
+    are given back here."""
+    done = []
+    for e in step.entries:
+      if not e.samples:
+        continue
+      r = e.request
+      r.pending -= 1
+      self.num_unresolved -= 1
+      if e.output_index < len(r.outputs):          # else: dropped after an earlier end-of-sequence token
+        tok = int(sampled[r.number])
+        r.set_output(e.output_index, tok)
+        if not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id:
+          r.finish_reason = "eos"
+          r.truncate_outputs(e.output_index + 1)
+          if r in self.running:
+            self.running.remove(r)
+            self._draining.append(r)
+          elif r in self.waiting:                   # preempted meanwhile: it holds nothing
+            self.waiting.remove(r)
+            self._retired_unadmitted.append(r)
+      if r.finished and r.pending == 0:
+        if r in self._draining:
+          self._draining.remove(r)
+          self.cache.release(r.number)
+        elif r in self._retired_unadmitted:
+          self._retired_unadmitted.remove(r)
+        else:
+          continue
         self.finished.append(r)
         done.append(r)
     return done
+
+  def update(self, step: ScheduledStep, sampled: Dict[int, int]) -> List[Request]:
+    """After the step ran: `sampled[request.number]` is the next token of every entry that samples.
+    Returns the requests that finished; their pages and slots are given back here."""
+    self.advance(step)
+    return self.resolve(step, sampled)

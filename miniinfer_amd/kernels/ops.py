@@ -71,7 +71,7 @@ def _f32(name, t, n=None):
 
 _SIGS = {
   "elementwise": {
-    "mi_embed": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "mi_embed": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
     "mi_add_rmsnorm": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                        c_void_p],
     "mi_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -157,16 +157,20 @@ def _check_pages(what, k_pages, v_pages, nkv, d, dtype):
 
 # ----------------------------------------------------------------------------- embedding
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-  """out[t, :] = float32(table[ids[t], :]).  An id outside the table gives a row of NaN."""
-  _dev(table, ids, out)
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor,
+          future: Optional[torch.Tensor] = None) -> torch.Tensor:
+  """out[t, :] = float32(table[ids[t], :]).  An id outside the table gives a row of NaN.  With `future` (int32),
+  an id -(r + 1) is replaced by future[r] as it stands when the kernel runs."""
+  _dev(table, ids, out, future)
+  _i32("future", future)
   V, H = table.shape
   T = ids.numel()
   _contig("table", table)
   _i32("ids", ids)
   _f32("out", out, T * H)
   lib = _lib("elementwise")
-  _check(lib, lib.mi_embed(dtype_code(table.dtype), _ptr(table), _ptr(ids), _ptr(out), T, H, V, _stream()))
+  _check(lib, lib.mi_embed(dtype_code(table.dtype), _ptr(table), _ptr(ids), _ptr(out), T, H, V, _ptr(future),
+                           0 if future is None else future.numel(), _stream()))
   return out
 
 

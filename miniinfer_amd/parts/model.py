@@ -70,7 +70,7 @@ class DecoderModel(Part):
     """ctx: StepContext.  Returns float32 logits [len(ctx.logit_rows), vocab]."""
     T, H = ctx.num_tokens, self.spec.hidden_size
     residual = torch.empty((T, H), dtype=torch.float32, device=self.ctx.device)
-    ops.embed(self.embedding, ctx.token_ids, residual)
+    ops.embed(self.embedding, ctx.token_ids, residual, future=getattr(ctx, "future_tokens", None))
     h = None
     for run, li in enumerate(self.spec.run_order):
       h, residual = self.blocks[li].forward(h, residual, ctx, ctx.layer_cache(self.cache_index(run)))

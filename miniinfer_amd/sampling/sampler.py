@@ -31,13 +31,20 @@ class Sampler:
   def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
              steps: Sequence[int]) -> List[int]:
     """logits float32 [R, V]; row r is sampled with params[r] from the stream (seeds[r], steps[r])."""
+    out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+    return self.sample_into(logits, params, seeds, steps, out).tolist()
+
+  def sample_into(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
+                  steps: Sequence[int], out: torch.Tensor) -> torch.Tensor:
+    """The same, left on the device in `out` (int32 [R]); nothing waits for the kernel."""
     R = logits.shape[0]
     if not (len(params) == len(seeds) == len(steps) == R):
       raise ValueError("one SamplingParams, seed and step per row of logits")
-    out = torch.empty(R, dtype=torch.int32, device=self.device)
+    if out.numel() != R or out.dtype != torch.int32:
+      raise ValueError("out must hold one int32 per row of logits")
     if all(p.temperature == 0 for p in params):
       ops.sample(logits, None, None, None, None, None, out)
-      return out.tolist()
+      return out
     temp = torch.tensor([p.temperature for p in params], dtype=torch.float32, device=self.device)
     any_k = any(p.top_k > 0 for p in params)
     any_p = any(p.top_p < 1.0 for p in params)
@@ -46,4 +53,4 @@ class Sampler:
     sd = torch.tensor(list(seeds), dtype=torch.int64, device=self.device)
     st = torch.tensor(list(steps), dtype=torch.int64, device=self.device)
     ops.sample(logits, temp, top_k, top_p, sd, st, out)
-    return out.tolist()
+    return out

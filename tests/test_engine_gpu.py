@@ -120,3 +120,40 @@ def test_command_line_generate(tmp_path):
                         capture_output=True, text=True, cwd=root, timeout=300)
   assert proc.returncode == 0, proc.stderr[-2000:]
   assert json.loads(proc.stdout.strip().splitlines()[-1])["token_ids"] == want
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_launching_ahead_of_the_tokens_changes_no_token(tmp_path, dtype):
+  """With `enable_overlap` the engine launches a step before it has read the tokens of the one before (they stay
+  on the device as placeholders' targets).  Same requests, same tokens and finish reasons as the synchronous
+  loop: greedy and seeded sampling, an end-of-sequence token that is found one step late, so few pages that
+  requests are preempted, prompts cut into portions."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "B", dtype=torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+  prompts = [tm.random_tokens(cfg, n, seed=50 + n) for n in (30, 41, 3, 25, 37, 12)]
+  params = [SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True),
+            SamplingParams(temperature=0.9, max_tokens=33, ignore_eos=True, seed=7),
+            SamplingParams(temperature=0.0, max_tokens=30),
+            SamplingParams(temperature=0.7, top_k=20, top_p=0.9, max_tokens=25, seed=11),
+            SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True),
+            SamplingParams(temperature=0.0, max_tokens=28)]
+  results = {}
+  for overlap in (False, True):
+    # the end-of-sequence token is one that the third request produces early in greedy decoding
+    with LLMEngine(model=str(tmp_path / "m"), dtype=dtype, page_size=8, num_pages=15, max_num_seqs=4,
+                   max_num_batched_tokens=48, enable_overlap=overlap, eos=results.get("eos")) as eng:
+      if "eos" not in results:
+        probe = eng.generate([prompts[2]], SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True),
+                             use_tqdm=False)[0]["token_ids"]
+        results["eos"] = probe[3]
+        eng.scheduler.eos_token_id = eng.eos_token_id = probe[3]
+      outs = eng.generate(prompts, params, use_tqdm=False)
+      results[overlap] = [(o["token_ids"], o["finish_reason"]) for o in outs]
+      assert eng.cache.num_free_pages() == eng.cache.num_pages and eng.is_finished()
+      eng.cache.check()
+      if overlap:
+        assert eng.scheduler.num_preemptions > 0, "the test is meant to run out of pages"
+  assert results[True] == results[False]
+  assert results[True][2][1] == "eos" and len(results[True][2][0]) <= 4
+  assert all(t >= 0 for toks, _ in results[True] for t in toks)

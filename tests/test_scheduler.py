@@ -154,3 +154,87 @@ def test_eos_and_length_finish():
                params=SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True))
   run(cache2, sched2, [r3])
   assert r3.outputs == want and r3.finish_reason == "max_tokens"
+
+
+# ---------------------------------------------------------------------------- results that arrive one step late
+
+def run_pipelined(cache, sched, reqs, max_steps=100000):
+  """Drives the scheduler like the engine does when it launches a step before it has read the tokens of the
+  step before: schedule, 'launch' (advance), then resolve the previous step.  The fake model looks a placeholder
+  token -(row + 1) up in the previous step's sampling output, as the embedding kernel does."""
+  for r in reqs:
+    sched.add(r)
+  pending = None          # (plan, tokens by row) of the launched step
+  future = []             # tokens by row of the last launched step
+  steps = 0
+  while sched.has_unfinished():
+    plan = sched.schedule()
+    launched = None
+    if plan is not None:
+      rows = []
+      for e in plan.entries:
+        r = e.request
+        assert e.start == r.num_computed == cache.length(r.number)
+        cache.grow(r.number, e.start + e.num_tokens)
+        cache.commit(r.number, e.start + e.num_tokens)
+        if e.samples:
+          toks = [t if t >= 0 else future[-(t + 1)] for t in r.tokens]
+          assert all(t >= 0 for t in toks), "a placeholder may only name a row of the step before"
+          rows.append((r.number, fake_next(toks)))
+      sched.advance(plan)
+      launched = (plan, rows)
+    if pending is not None:
+      sched.resolve(pending[0], dict(pending[1]))
+    cache.check()
+    if launched is not None:
+      future = [t for _, t in launched[1]]
+    pending = launched
+    steps += 1
+    assert steps < max_steps
+  assert pending is None
+  return steps
+
+
+def test_placeholders_stand_for_tokens_until_they_are_resolved():
+  cache, sched = make(pages=100, budget=32)
+  r = _req(0, 5, 4)
+  sched.add(r)
+  plan = sched.schedule()
+  cache.grow(0, 5)
+  cache.commit(0, 5)
+  sched.advance(plan)
+  assert r.outputs == [-1] and r.pending == 1 and r.num_computed == 5 and sched.has_unfinished()
+  nxt = sched.schedule()                                   # the next step is planned against the placeholder
+  assert [(e.start, e.num_tokens, e.samples) for e in nxt.entries] == [(5, 1, True)]
+  assert r.tokens[5:6] == [-1]
+  assert sched.resolve(plan, {0: 77}) == []
+  assert r.outputs == [77] and r.tokens[-1] == 77 and r.pending == 0
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_late_results_give_the_same_tokens_and_leave_no_page_behind(seed):
+  rnd = random.Random(100 + seed)
+  P = 8
+  reqs = [_req(i, rnd.randint(1, 60), rnd.randint(1, 40), seed=seed) for i in range(10)]
+  biggest = max(-(-(len(r.prompt) + r.params.max_tokens) // P) for r in reqs)
+  cache, sched = make(pages=biggest + rnd.randint(0, 6), P=P, max_seqs=3, budget=rnd.choice([8, 16, 64]))
+  run_pipelined(cache, sched, reqs)
+  for r in reqs:
+    assert r.outputs == expected(r.prompt, r.params.max_tokens) and r.pending == 0
+  assert cache.num_free_pages() == cache.num_pages and cache.num_free_slots() == 3
+  assert sorted(r.number for r in sched.finished) == list(range(10))
+
+
+def test_an_end_of_sequence_token_found_late_drops_the_token_launched_after_it():
+  prompt = [3, 1, 4, 1, 5]
+  want = expected(prompt, 6)
+  eos = want[2]
+  stop = want.index(eos) + 1
+  cache, sched = make(pages=100, eos=eos)
+  r = Request(number=0, request_id="r0", prompt=list(prompt), params=SamplingParams(temperature=0.0, max_tokens=6))
+  other = _req(1, 7, 9)
+  run_pipelined(cache, sched, [r, other])
+  assert r.outputs == want[:stop] and r.finish_reason == "eos" and r.pending == 0
+  assert other.outputs == expected(other.prompt, 9)
+  assert cache.num_free_pages() == 100 and cache.num_free_slots() == 4
+  assert [q.number for q in sched.finished].count(0) == 1
