@@ -34,14 +34,28 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // (arrays of HIP's uint4 class end up in scratch memory)
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int D = HEAD_DIM;
+
+// Register budgets.  Up to head size 128 the decode kernel is held to the registers that let two waves share a
+// SIMD (the compiler would otherwise take a few more and lose a wave to them), and the prefill kernel exists a
+// second time, held to three waves per SIMD at the price of a few spilled registers: that pays when there are
+// more than two workgroups for every compute unit, and costs when there are not.
+#if HEAD_DIM <= 128
+#define DECODE_OCCUPANCY __attribute__((amdgpu_waves_per_eu(2)))
+#define PREFILL_DENSE_OCCUPANCY __attribute__((amdgpu_waves_per_eu(3)))
+#else
+#define DECODE_OCCUPANCY
+#define PREFILL_DENSE_OCCUPANCY
+#endif
 constexpr int KSTEPS = D / 32;          // 16x16x32 products over the head dim
 constexpr bool KREM = (D % 32) != 0;    // plus one more, half of it zeros
 constexpr int QSTEPS = KSTEPS + (KREM ? 1 : 0);
 constexpr int DBLK = D / 16;            // 16-row blocks of O^T
 constexpr int MT = D > 128 ? 2 : 4;     // tiles of 16 keys per macro tile
 constexpr int MKEYS = 16 * MT;          // keys per macro tile
+static_assert(MT % 2 == 0, "the second product takes the tiles in pairs");
 
 // The last 16 dims of a head size that is no multiple of 32 go through the same 16x16x32 product with the
 // upper half of the contraction zeroed: lanes 0..31 hold 8 dims each, lanes 32..63 hold zeros.  (Finishing
@@ -137,33 +151,47 @@ __device__ __forceinline__ void tile_scores(f32x4 (&s)[NB], const bf16x8 (&ka)[Q
   }
 }
 
-// The running softmax over the macro tile that starts at key j0: masks and scales the scores in s[t][nb]
-// (lane: key j0 + 16 t + 4 (lane / 16) + i, column lane % 16), moves the maxima, rescales sums and accumulators,
-// and leaves the probabilities, rounded to bfloat16, in p[t][nb].  c = scale * log2(e).
+// The running softmax over the macro tile that starts at key j0: masks the scores in s[t][nb] (lane: key
+// j0 + 16 t + 4 (lane / 16) + i, column lane % 16), moves the maxima, rescales sums and accumulators, and leaves
+// the probabilities, rounded to bfloat16, in p[t][nb].  c = scale * log2(e) > 0; the scale is folded into the
+// exponent's multiply-add, so a probability costs a max, an fma, an exp2 and an add.
 // pos_hi[nb] / pos_lo[nb]: the last and first key the lane's column of block nb may see (pos_hi < 0: none).
+// Most macro tiles lie wholly inside every column's range; those skip the masking (the test is per wave).
 template <int NB>
 __device__ __forceinline__ void softmax_update(State<NB>& st, f32x4 (&s)[MT][NB], s16x4 (&p)[MT][NB], float c, int j0,
                                                const int (&pos_lo)[NB], const int (&pos_hi)[NB]) {
   const int lane = threadIdx.x & 63;
   const int kbase = j0 + 4 * (lane >> 4);
+  bool inside = true;                    // columns without a query do not matter: their results are dropped
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+    inside = inside && (pos_hi[nb] < 0 || (j0 + MKEYS - 1 <= pos_hi[nb] && j0 >= pos_lo[nb]));
+  const bool full = __all(inside);
   float alpha[NB];
   bool moved = false;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     float tmax = -INFINITY;
+    if (full) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+      for (int t = 0; t < MT; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = kbase + 16 * t + i;
-        const bool ok = key <= pos_hi[nb] && key >= pos_lo[nb];
-        const float v = ok ? s[t][nb][i] * c : -INFINITY;
-        s[t][nb][i] = v;
-        tmax = fmaxf(tmax, v);
-      }
+        for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[t][nb][i]);
+    } else {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kbase + 16 * t + i;
+          const bool ok = key <= pos_hi[nb] && key >= pos_lo[nb];
+          const float v = ok ? s[t][nb][i] : -INFINITY;
+          s[t][nb][i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+    }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(st.m[nb], tmax);
+    const float m_new = fmaxf(st.m[nb], tmax * c);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;    // a column that has seen no key yet
     alpha[nb] = __builtin_amdgcn_exp2f(st.m[nb] - m_use);      // 2^-inf = 0 on the first visible tile
     moved = moved || (m_new != st.m[nb]);
@@ -173,7 +201,7 @@ __device__ __forceinline__ void softmax_update(State<NB>& st, f32x4 (&s)[MT][NB]
       float e[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        e[i] = __builtin_amdgcn_exp2f(s[t][nb][i] - m_use);    // 0 for masked keys
+        e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][nb][i], c, -m_use));    // 0 for masked keys
         psum += e[i];
       }
       p[t][nb] = pack_bf16x4(e[0], e[1], e[2], e[3]);
@@ -194,14 +222,30 @@ __device__ __forceinline__ void softmax_update(State<NB>& st, f32x4 (&s)[MT][NB]
   }
 }
 
-// O^T += V^T P^T for one tile of 16 keys (operands `va`).
+// O^T += V^T P^T for two tiles of 16 keys at once (operands va0 / p0 of one tile, va1 / p1 of the other), as one
+// 16x16x32 product: the order of the contraction index is free as long as both operands agree, so slot 8 q + e of
+// lane group q is key 4 q + e of the first tile for e < 4 and key 4 q + e - 4 of the second for e >= 4, which is
+// where the values' 8-byte reads and the first product's accumulators already are.
+__device__ __forceinline__ bf16x8 join8(const s16x4 lo, const s16x4 hi) {
+  union {
+    s16x4 h[2];
+    bf16x8 v;
+  } u;
+  u.h[0] = lo;
+  u.h[1] = hi;
+  return u.v;
+}
+
 template <int NB>
-__device__ __forceinline__ void tile_values(State<NB>& st, const s16x4 (&va)[DBLK], const s16x4 (&p)[NB]) {
+__device__ __forceinline__ void tile_values(State<NB>& st, const s16x4 (&va0)[DBLK], const s16x4 (&va1)[DBLK],
+                                            const s16x4 (&p0)[NB], const s16x4 (&p1)[NB]) {
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
+  for (int nb = 0; nb < NB; ++nb) {
+    const bf16x8 pb = join8(p0[nb], p1[nb]);
 #pragma unroll
     for (int blk = 0; blk < DBLK; ++blk)
-      st.o[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[blk], p[nb], st.o[nb][blk], 0, 0, 0);
+      st.o[nb][blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(join8(va0[blk], va1[blk]), pb, st.o[nb][blk], 0, 0, 0);
+  }
 }
 
 // Normalises and stores the columns of a wave: token col / gpad of the rows that start at out_base.
@@ -237,14 +281,15 @@ __device__ __forceinline__ void store_output(const State<NB>& st, uint16_t* out_
 #define PREFILL_NB 1
 #endif
 constexpr int LDS_KSTR = D + 8;                  // elements per key row in LDS
-constexpr int LDS_VSTR = MKEYS + 8;              // elements per dim row of the transposed values in LDS
+constexpr int LDS_VSTR = MKEYS + 4;              // elements per dim row of the transposed values in LDS: rows 2 banks
+                                                 // apart, so the 16 rows x 8 bytes of an operand read hit 32 banks
 constexpr int LDS_KCHUNKS = MKEYS * (D / 8);     // 16-byte chunks of a key tile
 constexpr int LDS_VCHUNKS = D * (MKEYS / 8);     // 16-byte chunks of a value tile
 constexpr int LDS_KITER = (LDS_KCHUNKS + 255) / 256;
 constexpr int LDS_VITER = (LDS_VCHUNKS + 255) / 256;
 
 template <int NB>
-__global__ __launch_bounds__(256) void prefill_kernel(
+__device__ __forceinline__ void prefill_body(
     const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ work, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int nq,
@@ -253,8 +298,10 @@ __global__ __launch_bounds__(256) void prefill_kernel(
   __shared__ __attribute__((aligned(16))) uint16_t Vs[D * LDS_VSTR];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int b = work[2 * blockIdx.x], sb = work[2 * blockIdx.x + 1];
-  const int g = blockIdx.y;
+  // The kv head is the fastest grid index: workgroups go round the 8 XCDs by their linear index, so with 8 kv
+  // heads (or a divisor or multiple of 8) all the workgroups that read one head's keys and values share an L2.
+  const int b = work[2 * blockIdx.y], sb = work[2 * blockIdx.y + 1];
+  const int g = blockIdx.x;
   const int G = nq / nkv;
   const int P = 1 << page_shift;
   const int q_begin = cu_q[b];
@@ -292,30 +339,48 @@ __global__ __launch_bounds__(256) void prefill_kernel(
   State<NB> st;
   init_state<NB>(st);
 
-  // this thread's chunks of a macro tile: global -> registers (PREFILL_FETCH), registers -> LDS (PREFILL_STASH)
+  // This thread's chunks of a macro tile: page numbers from the block table (PREFILL_PAGES), global -> registers
+  // (PREFILL_FETCH), registers -> LDS (PREFILL_STASH).  The page numbers are asked for one tile earlier than the
+  // keys and values that need them, so that no step of the loop waits for two dependent loads in a row.
   const int kpp = P < MKEYS ? P : MKEYS;   // keys of a macro tile that lie in one page
   const int cpp = kpp / 8;                 // 16-byte chunks per (page, dim)
   u32x4 pk[LDS_KITER], pv[LDS_VITER];
+  int kpage[LDS_KITER], vpage[LDS_VITER];
+#define PREFILL_KEY_OF_KCHUNK(J0, IT, KEY)                                                                           \
+  int ch = threadIdx.x + 256 * (IT);                                                                                 \
+  ch = ch < LDS_KCHUNKS ? ch : LDS_KCHUNKS - 1; /* threads past the end load the last chunk again, drop it */       \
+  int KEY = (J0) + ch / (D / 8);                                                                                     \
+  KEY = KEY > last ? last : KEY; /* masked keys read valid memory of the request */
+#define PREFILL_KEY_OF_VCHUNK(J0, IT, KEY)                                                                           \
+  int ch = threadIdx.x + 256 * (IT);                                                                                 \
+  ch = ch < LDS_VCHUNKS ? ch : LDS_VCHUNKS - 1;                                                                      \
+  /* chunk -> (page of the tile, dim, run of 8 keys): consecutive threads read consecutive memory of a page */      \
+  const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);                                          \
+  int KEY = (J0) + page_i * kpp + 8 * part;                                                                          \
+  KEY = KEY > last ? (last & ~7) : KEY; /* a run of 8 keys lies in one page */
+#define PREFILL_PAGES(J0)                                                                                            \
+  {                                                                                                                  \
+    _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
+      PREFILL_KEY_OF_KCHUNK(J0, it, key)                                                                             \
+      kpage[it] = bt[key >> page_shift];                                                                             \
+    }                                                                                                                \
+    _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
+      PREFILL_KEY_OF_VCHUNK(J0, it, key)                                                                             \
+      (void)dim;                                                                                                     \
+      vpage[it] = bt[key >> page_shift];                                                                             \
+    }                                                                                                                \
+  }
 #define PREFILL_FETCH(J0)                                                                                            \
   {                                                                                                                  \
     _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
-      int ch = threadIdx.x + 256 * it;                                                                               \
-      ch = ch < LDS_KCHUNKS ? ch : LDS_KCHUNKS - 1; /* threads past the end load the last chunk again, drop it */   \
-      int key = (J0) + ch / (D / 8);                                                                                 \
-      key = key > last ? last : key; /* masked keys read valid memory of the request */                             \
-      const int64_t page = bt[key >> page_shift];                                                                    \
-      pk[it] = *reinterpret_cast<const u32x4*>(k_pages + ((page * nkv + g) * P + (key & (P - 1))) * D +              \
+      PREFILL_KEY_OF_KCHUNK(J0, it, key)                                                                             \
+      pk[it] = *reinterpret_cast<const u32x4*>(k_pages + (((int64_t)kpage[it] * nkv + g) * P + (key & (P - 1))) * D + \
                                                8 * (ch % (D / 8)));                                                  \
     }                                                                                                                \
     _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
-      int ch = threadIdx.x + 256 * it;                                                                               \
-      ch = ch < LDS_VCHUNKS ? ch : LDS_VCHUNKS - 1;                                                                  \
-      /* chunk -> (page of the tile, dim, run of 8 keys): consecutive threads read consecutive memory of a page */  \
-      const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);                                      \
-      int key = (J0) + page_i * kpp + 8 * part;                                                                      \
-      key = key > last ? (last & ~7) : key; /* a run of 8 keys lies in one page */                                  \
-      const int64_t page = bt[key >> page_shift];                                                                    \
-      pv[it] = *reinterpret_cast<const u32x4*>(v_pages + ((page * nkv + g) * D + dim) * P + (key & (P - 1)));        \
+      PREFILL_KEY_OF_VCHUNK(J0, it, key)                                                                             \
+      pv[it] = *reinterpret_cast<const u32x4*>(v_pages + (((int64_t)vpage[it] * nkv + g) * D + dim) * P +            \
+                                               (key & (P - 1)));                                                     \
     }                                                                                                                \
   }
 #define PREFILL_STASH()                                                                                              \
@@ -327,16 +392,25 @@ __global__ __launch_bounds__(256) void prefill_kernel(
     _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
       const int ch = threadIdx.x + 256 * it;                                                                         \
       const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);                                      \
-      if (ch < LDS_VCHUNKS) *reinterpret_cast<u32x4*>(Vs + dim * LDS_VSTR + page_i * kpp + 8 * part) = pv[it];       \
+      if (ch < LDS_VCHUNKS) { /* rows are 8-byte aligned only: two 64-bit writes */                                  \
+        u32x2* dst = reinterpret_cast<u32x2*>(Vs + dim * LDS_VSTR + page_i * kpp + 8 * part);                        \
+        dst[0] = u32x2{pv[it][0], pv[it][1]};                                                                        \
+        dst[1] = u32x2{pv[it][2], pv[it][3]};                                                                        \
+      }                                                                                                              \
     }                                                                                                                \
   }
 
+  PREFILL_PAGES(wg_lo)
   PREFILL_FETCH(wg_lo)
+  PREFILL_PAGES(wg_lo + MKEYS)
   for (int j0 = wg_lo; j0 < wg_hi; j0 += MKEYS) {
     __syncthreads();                    // every wave is done with the tile that is in LDS
     PREFILL_STASH()
     __syncthreads();
-    if (j0 + MKEYS < wg_hi) PREFILL_FETCH(j0 + MKEYS)
+    if (j0 + MKEYS < wg_hi) {
+      PREFILL_FETCH(j0 + MKEYS)
+      PREFILL_PAGES(j0 + 2 * MKEYS)
+    }
     if (j0 >= w_hi || j0 + MKEYS <= w_lo) continue;      // nothing this wave can see (same for all its lanes)
     f32x4 s[MT][NB];
     s16x4 p[MT][NB];
@@ -348,18 +422,45 @@ __global__ __launch_bounds__(256) void prefill_kernel(
     }
     softmax_update<NB>(st, s, p, c, j0, pos_lo, pos_hi);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      s16x4 va[DBLK];
+    for (int t = 0; t < MT; t += 2) {
+      s16x4 va[2][DBLK];
 #pragma unroll
-      for (int blk = 0; blk < DBLK; ++blk)
-        va[blk] = *reinterpret_cast<const s16x4*>(Vs + (16 * blk + (lane & 15)) * LDS_VSTR + 16 * t + 4 * (lane >> 4));
-      tile_values<NB>(st, va, p[t]);
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int blk = 0; blk < DBLK; ++blk)
+          va[u][blk] = *reinterpret_cast<const s16x4*>(Vs + (16 * blk + (lane & 15)) * LDS_VSTR + 16 * (t + u) +
+                                                       4 * (lane >> 4));
+      tile_values<NB>(st, va[0], va[1], p[t], p[t + 1]);
     }
   }
+#undef PREFILL_PAGES
+#undef PREFILL_KEY_OF_KCHUNK
+#undef PREFILL_KEY_OF_VCHUNK
 #undef PREFILL_FETCH
 #undef PREFILL_STASH
   store_output<NB>(st, out + (int64_t)(q_begin + tok0) * out_row_stride, out_row_stride, gpad, g * G, pos_hi);
 }
+
+#define PREFILL_ARGS                                                                                                 \
+  const uint16_t *__restrict__ q, int64_t q_row_stride, uint16_t *__restrict__ out, int64_t out_row_stride,          \
+      const uint16_t *__restrict__ k_pages, const uint16_t *__restrict__ v_pages, const int *__restrict__ block_table, \
+      int table_width, const int *__restrict__ work, const int *__restrict__ cu_q, const int *__restrict__ kv_len,   \
+      int nq, int nkv, int gpad, int page_shift, float scale, int window
+#define PREFILL_PASS                                                                                                 \
+  q, q_row_stride, out, out_row_stride, k_pages, v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv,     \
+      gpad, page_shift, scale, window
+
+template <int NB>
+__global__ __launch_bounds__(256) void prefill_kernel(PREFILL_ARGS) {
+  prefill_body<NB>(PREFILL_PASS);
+}
+
+template <int NB>
+__global__ __launch_bounds__(256) PREFILL_DENSE_OCCUPANCY void prefill_dense_kernel(PREFILL_ARGS) {
+  prefill_body<NB>(PREFILL_PASS);
+}
+#undef PREFILL_ARGS
+#undef PREFILL_PASS
 
 // ---------------------------------------------------------------- decode: one new token per entry, keys split
 // Grid (num_splits, nkv, entries), DECODE_WAVES waves per workgroup.  The macro tiles of a split go round-robin to
@@ -392,7 +493,7 @@ struct DecodeFront {
 __device__ __forceinline__ float bf16_at(const uint16_t* p) { return __uint_as_float((uint32_t)(*p) << 16); }
 
 template <bool FRONT>
-__global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
+__global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_kernel(
     const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int first_entry,
@@ -544,7 +645,7 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) void decode_kernel(
     for (int t = 0; t < MT; ++t) tile_scores<1>(s[t], ka[t], qr);
     softmax_update<1>(st, s, p, c, j0, pos_lo, pos_hi);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) tile_values<1>(st, va[t], p[t]);
+    for (int t = 0; t < MT; t += 2) tile_values<1>(st, va[t], va[t + 1], p[t], p[t + 1]);
     mt += DECODE_WAVES;
     if (mt < t1) DECODE_FETCH(mt)
   }
@@ -713,6 +814,11 @@ static int check_common(const char* what, int nq, int nkv, int page_size, int64_
   return 0;
 }
 
+static int check_scale(const char* what, float scale) {
+  MI_REQUIRE(scale > 0.f, "%s: the softmax scale must be positive, got %g", what, (double)scale);
+  return 0;
+}
+
 static int log2_of(int v) {
   int s = 0;
   while ((1 << s) < v) ++s;
@@ -744,14 +850,29 @@ MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, in
                               int num_work, const int* cu_q, const int* kv_len, int nq, int nkv, int page_size,
                               float scale, int window, hipStream_t stream) {
   if (check_common("attn_prefill", nq, nkv, page_size, q_row_stride, out_row_stride, table_width)) return 1;
+  if (check_scale("attn_prefill", scale)) return 1;
   MI_REQUIRE(num_work >= 0 && window >= 0, "attn_prefill: bad work count or window");
-  MI_REQUIRE(nkv <= 65535, "attn_prefill: grid too large");
+  MI_REQUIRE(num_work <= 65535, "attn_prefill: %d work items; the grid takes at most 65535", num_work);
   if (num_work == 0) return 0;
-  dim3 grid(num_work, nkv);
-  prefill_kernel<PREFILL_NB><<<grid, 256, 0, stream>>>(
-      (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
-      (const uint16_t*)v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv, group_pad(nq, nkv),
-      log2_of(page_size), scale, window);
+  dim3 grid(nkv, num_work);
+  static int compute_units = 0;
+  if (compute_units == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        compute_units <= 0)
+      compute_units = 256;
+  }
+  if ((int64_t)num_work * nkv > 2 * (int64_t)compute_units)
+    prefill_dense_kernel<PREFILL_NB><<<grid, 256, 0, stream>>>(
+        (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
+        (const uint16_t*)v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv, group_pad(nq, nkv),
+        log2_of(page_size), scale, window);
+  else
+    prefill_kernel<PREFILL_NB><<<grid, 256, 0, stream>>>(
+        (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
+        (const uint16_t*)v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv, group_pad(nq, nkv),
+        log2_of(page_size), scale, window);
   MI_CHECK_LAUNCH("attn_prefill");
   return 0;
 }
@@ -764,6 +885,7 @@ MI_EXPORT int mi_attn_decode(const void* q, int64_t q_row_stride, void* out, int
                              float* part_ml, int nq, int nkv, int page_size, float scale, int window,
                              hipStream_t stream) {
   if (check_common("attn_decode", nq, nkv, page_size, q_row_stride, out_row_stride, table_width)) return 1;
+  if (check_scale("attn_decode", scale)) return 1;
   MI_REQUIRE(num_entries >= 0 && first_entry >= 0 && window >= 0, "attn_decode: bad entry range or window");
   MI_REQUIRE(num_splits >= 1 && num_splits <= 1024, "attn_decode: %d splits", num_splits);
   MI_REQUIRE(num_entries <= 65535 && nkv <= 65535, "attn_decode: grid too large");
@@ -794,6 +916,7 @@ MI_EXPORT int mi_attn_decode_front(const void* qkv, int64_t qkv_row_stride, void
                                    const float* cos_sin, int rotary_dim, int max_pos, const int* positions,
                                    const int* slots, hipStream_t stream) {
   if (check_common("attn_decode_front", nq, nkv, page_size, qkv_row_stride, out_row_stride, table_width)) return 1;
+  if (check_scale("attn_decode_front", scale)) return 1;
   MI_REQUIRE(qkv_row_stride >= (int64_t)(nq + 2 * nkv) * D, "attn_decode_front: row stride %lld holds no q | k | v",
              (long long)qkv_row_stride);
   MI_REQUIRE(num_entries >= 0 && first_entry >= 0 && window >= 0, "attn_decode_front: bad entry range or window");

@@ -74,6 +74,33 @@ __device__ __forceinline__ void store2(bf16* p, float a, float b) {   // v_cvt_p
   *reinterpret_cast<uint32_t*>(p) = *reinterpret_cast<const uint32_t*>(&r);
 }
 
+// four values at once (a 64-bit or 128-bit access)
+typedef float mi_f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t mi_u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+  const mi_f32x4 x = *reinterpret_cast<const mi_f32x4*>(p);
+  v[0] = x[0];
+  v[1] = x[1];
+  v[2] = x[2];
+  v[3] = x[3];
+}
+__device__ __forceinline__ void load4(const bf16* p, float (&v)[4]) {
+  const mi_u32x2 u = *reinterpret_cast<const mi_u32x2*>(p);
+  v[0] = __uint_as_float(u[0] << 16);
+  v[1] = __uint_as_float(u[0] & 0xffff0000u);
+  v[2] = __uint_as_float(u[1] << 16);
+  v[3] = __uint_as_float(u[1] & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
+  *reinterpret_cast<mi_f32x4*>(p) = mi_f32x4{v[0], v[1], v[2], v[3]};
+}
+__device__ __forceinline__ void store4(bf16* p, const float (&v)[4]) {
+  const mi_f32x2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
+  const mi_bf16x2 a = __builtin_convertvector(lo, mi_bf16x2), b = __builtin_convertvector(hi, mi_bf16x2);
+  *reinterpret_cast<mi_u32x2*>(p) = mi_u32x2{*reinterpret_cast<const uint32_t*>(&a), *reinterpret_cast<const uint32_t*>(&b)};
+}
+
 template <typename T>
 __device__ __forceinline__ T from_float(float x);
 template <>

@@ -79,23 +79,6 @@ __global__ void add_rmsnorm_kernel(const TX* __restrict__ x, float* __restrict__
 
 // The same with every value held in registers: one read of x, residual and w (all loads issued together), one
 // reduction, one write.  Each thread takes CH chunks of 4 consecutive elements; N must be a multiple of 4.
-__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
-  const float4 t = *reinterpret_cast<const float4*>(p);
-  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-}
-__device__ __forceinline__ void load4(const bf16* p, float (&v)[4]) {
-  const uint2 t = *reinterpret_cast<const uint2*>(p);
-  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
-  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
-}
-__device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
-  *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
-}
-__device__ __forceinline__ void store4(bf16* p, const float (&v)[4]) {
-  store2(p, v[0], v[1]);
-  store2(p + 2, v[2], v[3]);
-}
-
 template <typename TX, typename TY, int CH>
 __global__ void add_rmsnorm_reg_kernel(const TX* __restrict__ x, float* __restrict__ residual,
                                        const float* __restrict__ w, TY* __restrict__ y, const int* __restrict__ rows,
@@ -260,9 +243,9 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_strid
                                           const float* __restrict__ cos_sin, int rotary_dim, int max_pos,
                                           const int* __restrict__ positions, T* __restrict__ k_pages,
                                           T* __restrict__ v_pages, const int* __restrict__ slots, int page_shift,
-                                          int num_tokens) {
+                                          int num_tokens, int heads) {
+  // heads = nq + 2 nkv, or nq + nkv when value_cache_write_kernel copies the values
   const int lane = threadIdx.x & (MI_WAVE - 1);
-  const int heads = nq + 2 * nkv;
   const int64_t wid = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + threadIdx.x / MI_WAVE;
   if (wid >= (int64_t)num_tokens * heads) return;
   const int t = (int)(wid / heads);
@@ -375,6 +358,139 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_strid
   }
 }
 
+// The same norm and rotation for many tokens whose heads are rotated whole (rotary_dim == d, or no rotation) and
+// whose values go through value_cache_write_kernel.  LPH lanes share a head: a lane takes 4 neighbouring rotation
+// pairs (j .. j + 3, each with its partner d/2 further on) in 64-bit or 128-bit accesses, so a wave holds 64 / LPH
+// heads of one token at a time, and two such sets in flight.  LPH is the power of two >= d / 8.
+template <typename T, int LPH>
+__global__ void qk_norm_rope_many_kernel(T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
+                                         const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+                                         const float* __restrict__ cos_sin, int max_pos,
+                                         const int* __restrict__ positions, T* __restrict__ k_pages,
+                                         const int* __restrict__ slots, int page_shift, int num_tokens) {
+  constexpr int HPS = MI_WAVE / LPH;     // heads per set
+  constexpr int SETS = 2;
+  const int lane = threadIdx.x & (MI_WAVE - 1);
+  const int sub = lane / LPH, ln = lane % LPH;
+  const int heads = nq + nkv;
+  const int groups = (heads + HPS * SETS - 1) / (HPS * SETS);
+  const int64_t wid = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + threadIdx.x / MI_WAVE;
+  if (wid >= (int64_t)num_tokens * groups) return;
+  const int t = (int)(wid / groups);
+  const int h0 = (int)(wid - (int64_t)t * groups) * HPS * SETS;
+  const int half = d / 2;
+  const int j = 4 * ln;
+  const bool ok = j < half;
+  int pos = (cos_sin && positions) ? positions[t] : 0;
+  const int slot = k_pages ? slots[t] : 0;
+  T* row = qkv + (int64_t)t * row_stride;
+  float xa[SETS][4], xb[SETS][4];
+#pragma unroll
+  for (int s = 0; s < SETS; ++s) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) xa[s][c] = xb[s][c] = 0.f;
+    const T* src = row + (int64_t)min(h0 + s * HPS + sub, heads - 1) * d;
+    if (ok) {
+      load4(src + j, xa[s]);
+      load4(src + j + half, xb[s]);
+    }
+  }
+  float wqa[4] = {1.f, 1.f, 1.f, 1.f}, wqb[4] = {1.f, 1.f, 1.f, 1.f}, wka[4] = {1.f, 1.f, 1.f, 1.f},
+        wkb[4] = {1.f, 1.f, 1.f, 1.f};
+  if (ok && qw) {
+    load4(qw + j, wqa);
+    load4(qw + j + half, wqb);
+  }
+  if (ok && kw) {
+    load4(kw + j, wka);
+    load4(kw + j + half, wkb);
+  }
+  pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+  float cv[4] = {1.f, 1.f, 1.f, 1.f}, sv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (ok && cos_sin) {
+    const float* cs = cos_sin + (int64_t)pos * d;
+    load4(cs + j, cv);
+    load4(cs + half + j, sv);
+  }
+  const int P = 1 << page_shift;
+#pragma unroll
+  for (int s = 0; s < SETS; ++s) {
+    const int h = h0 + s * HPS + sub;
+    const bool live = h < heads;
+    const bool is_key = h >= nq;
+    const float* w = is_key ? kw : qw;
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) ss += xa[s][c] * xa[s][c] + xb[s][c] * xb[s][c];
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, MI_WAVE);   // over the head's lanes
+    const float rstd = w ? rsqrtf(ss / (float)d + eps) : 1.f;
+    float o1[4], o2[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float a = xa[s][c] * rstd * (is_key ? wka[c] : wqa[c]);
+      const float b2 = xb[s][c] * rstd * (is_key ? wkb[c] : wqb[c]);
+      o1[c] = a * cv[c] - b2 * sv[c];
+      o2[c] = b2 * cv[c] + a * sv[c];
+    }
+    if (ok && live) {
+      T* src = row + (int64_t)h * d;
+      store4(src + j, o1);
+      store4(src + j + half, o2);
+      if (is_key && k_pages) {
+        T* dst = k_pages + ((((int64_t)(slot >> page_shift)) * nkv + (h - nq)) * P + (slot & (P - 1))) * d;
+        store4(dst + j, o1);
+        store4(dst + j + half, o2);
+      }
+    }
+  }
+}
+
+// The values of many tokens into their transposed pages [page][kv head][dim][slot in page].  A workgroup takes 16
+// consecutive tokens of one kv head.  Consecutive tokens of a request lie side by side in a page, so each half
+// of 8 tokens whose slots are consecutive and start at a multiple of 8 is written as one run of 8 per dim (16 bytes
+// in bfloat16) instead of 8 scattered elements; any other half falls back to single elements.
+template <typename T>
+__global__ void value_cache_write_kernel(const T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
+                                         T* __restrict__ v_pages, const int* __restrict__ slots, int page_shift,
+                                         int num_tokens) {
+  const int g = blockIdx.y;
+  const int P = 1 << page_shift;
+  for (int hf = 0; hf < 2; ++hf) {
+    const int t0 = blockIdx.x * 16 + 8 * hf;
+    const int n = min(8, num_tokens - t0);
+    if (n <= 0) break;
+    const int slot0 = slots[t0];
+    bool run = n == 8 && P >= 8 && (slot0 & 7) == 0;
+    for (int i = 1; i < n; ++i) run = run && slots[t0 + i] == slot0 + i;
+    const T* src = qkv + (int64_t)t0 * row_stride + (int64_t)(nq + nkv + g) * d;
+    if (run) {      // the same for every thread of the workgroup
+      T* base = v_pages + (((int64_t)(slot0 >> page_shift) * nkv + g) * d) * P + (slot0 & (P - 1));
+      for (int e = threadIdx.x; e < d; e += blockDim.x) {
+        union {
+          T v[8];
+          uint32_t u[2 * sizeof(T)];
+        } pack;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pack.v[i] = src[(int64_t)i * row_stride + e];
+        uint32_t* o = reinterpret_cast<uint32_t*>(base + (int64_t)e * P);
+#pragma unroll
+        for (int i = 0; i < (int)(2 * sizeof(T)); i += 4) {
+          typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+          *reinterpret_cast<u32x4*>(o + i) = u32x4{pack.u[i], pack.u[i + 1], pack.u[i + 2], pack.u[i + 3]};
+        }
+      }
+    } else {
+      for (int idx = threadIdx.x; idx < n * d; idx += blockDim.x) {
+        const int i = idx / d, e = idx - i * d;
+        const int slot = slots[t0 + i];
+        v_pages[(((int64_t)(slot >> page_shift) * nkv + g) * d + e) * P + (slot & (P - 1))] =
+            src[(int64_t)i * row_stride + e];
+      }
+    }
+  }
+}
+
 MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nq, int nkv, int d,
                                     const float* qw, const float* kw, float eps, const float* cos_sin,
                                     int rotary_dim, int max_pos, const int* positions, void* k_pages, void* v_pages,
@@ -396,18 +512,58 @@ MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, in
   int shift = 0;
   while ((1 << shift) < page_size) ++shift;
   const int waves_per_block = 4;
-  const int64_t waves = (int64_t)num_tokens * (nq + 2 * nkv);
+  // many tokens: the values are copied by a kernel of their own that writes runs of slots
+  const bool split_values = v_pages && nkv > 0 && num_tokens >= 32 && page_size >= 8;
+  const int heads = split_values ? nq + nkv : nq + 2 * nkv;
+  const int64_t waves = (int64_t)num_tokens * heads;
   const int blocks = (int)((waves + waves_per_block - 1) / waves_per_block);
-  if (dtype == MI_DTYPE_F32)
-    qk_norm_rope_cache_kernel<float><<<blocks, waves_per_block * MI_WAVE, 0, stream>>>(
-        (float*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (float*)k_pages,
-        (float*)v_pages, slots, shift, num_tokens);
-  else if (dtype == MI_DTYPE_BF16)
-    qk_norm_rope_cache_kernel<bf16><<<blocks, waves_per_block * MI_WAVE, 0, stream>>>(
-        (bf16*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (bf16*)k_pages,
-        (bf16*)v_pages, slots, shift, num_tokens);
-  else
+  const dim3 vgrid((num_tokens + 15) / 16, nkv > 0 ? nkv : 1);
+  const int vthreads = d >= 128 ? 128 : 64;
+  // whole-head rotation of many tokens: LPH lanes per head, the power of two >= d / 8
+  const bool many = (split_values || (nkv == 0 && num_tokens >= 32)) && d % 8 == 0 && (!cos_sin || rotary_dim == d);
+  int lph = 1;
+  while (lph * 8 < d) lph <<= 1;
+  const int heads_per_wave = 2 * (MI_WAVE / lph);
+  const int64_t many_waves = (int64_t)num_tokens * ((nq + nkv + heads_per_wave - 1) / heads_per_wave);
+  const int many_blocks = (int)((many_waves + waves_per_block - 1) / waves_per_block);
+#define MI_LAUNCH_MANY(T, LPH)                                                                                      \
+  qk_norm_rope_many_kernel<T, LPH><<<many_blocks, waves_per_block * MI_WAVE, 0, stream>>>(                          \
+      (T*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, max_pos, positions, (T*)k_pages, slots, shift, num_tokens)
+#define MI_LAUNCH_MANY_ANY(T)                                                                                       \
+  switch (lph) {                                                                                                    \
+    case 1: case 2: MI_LAUNCH_MANY(T, 2); break;                                                                    \
+    case 4: MI_LAUNCH_MANY(T, 4); break;                                                                            \
+    case 8: MI_LAUNCH_MANY(T, 8); break;                                                                            \
+    case 16: MI_LAUNCH_MANY(T, 16); break;                                                                          \
+    default: MI_LAUNCH_MANY(T, 32); break;                                                                          \
+  }
+  if (dtype == MI_DTYPE_F32) {
+    if (many) {
+      MI_LAUNCH_MANY_ANY(float)
+    } else {
+      qk_norm_rope_cache_kernel<float><<<blocks, waves_per_block * MI_WAVE, 0, stream>>>(
+          (float*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (float*)k_pages,
+          (float*)v_pages, slots, shift, num_tokens, heads);
+    }
+    if (split_values)
+      value_cache_write_kernel<float><<<vgrid, vthreads, 0, stream>>>((const float*)qkv, row_stride, nq, nkv, d,
+                                                                      (float*)v_pages, slots, shift, num_tokens);
+  } else if (dtype == MI_DTYPE_BF16) {
+    if (many) {
+      MI_LAUNCH_MANY_ANY(bf16)
+    } else {
+      qk_norm_rope_cache_kernel<bf16><<<blocks, waves_per_block * MI_WAVE, 0, stream>>>(
+          (bf16*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (bf16*)k_pages,
+          (bf16*)v_pages, slots, shift, num_tokens, heads);
+    }
+    if (split_values)
+      value_cache_write_kernel<bf16><<<vgrid, vthreads, 0, stream>>>((const bf16*)qkv, row_stride, nq, nkv, d,
+                                                                     (bf16*)v_pages, slots, shift, num_tokens);
+  } else {
     MI_FAIL("qk_norm_rope_cache: unknown dtype %d", dtype);
+  }
+#undef MI_LAUNCH_MANY_ANY
+#undef MI_LAUNCH_MANY
   MI_CHECK_LAUNCH("qk_norm_rope_cache");
   return 0;
 }

@@ -109,16 +109,24 @@ def _rope_ref(x, pos, theta, rotary_dim):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T", [11, 75])
 @pytest.mark.parametrize("nq,nkv,d,rd,P", [(6, 3, 48, 48, 16), (4, 4, 128, 128, 8), (5, 1, 16, 16, 4), (2, 2, 80, 32, 16)])
-def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P):
+def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P, T):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(4)
-  T, pages, max_pos, theta, eps = 11, 9, 300, 12345.0, 1e-5
+  pages, max_pos, theta, eps = 12 + 2 * T // P, 300, 12345.0, 1e-5
   qkv = torch.randn(T, (nq + 2 * nkv) * d, generator=g).to(dtype)
   qw = 1 + 0.1 * torch.randn(d, generator=g)
   kw = 1 + 0.1 * torch.randn(d, generator=g)
   pos = torch.randint(0, max_pos, (T,), generator=g)
   slots = torch.randperm(pages * P, generator=g)[:T] + P   # never page 0
+  if T > 32:
+    # like a prompt's portion: runs of consecutive slots (one starts in the middle of a page), then scattered ones
+    slots[:29] = torch.arange(29) + 3 * P + 5
+    slots[29:50] = torch.arange(21) + ((3 * P + 5 + 29) // P + 2) * P
+    rest = [x for x in range(P, (pages + 1) * P) if x not in set(slots[:50].tolist())]
+    slots[50:] = torch.tensor(rest)[torch.randperm(len(rest), generator=g)[:T - 50]]
+  assert len(set(slots.tolist())) == T
   j = torch.arange(0, rd, 2, dtype=torch.float32)
   ang = torch.outer(torch.arange(max_pos, dtype=torch.float32), 1.0 / theta ** (j / rd))
   table = torch.cat((ang.cos(), ang.sin()), -1)
