@@ -26,6 +26,8 @@ def _engine_args(p):
   p.add_argument("--max-num-batched-tokens", type=int, default=8192, help="token budget of one step")
   p.add_argument("--no-chunked-prefill", action="store_true")
   p.add_argument("--eager", action="store_true", help="never replay decode steps from HIP graphs")
+  p.add_argument("--no-overlap", action="store_true",
+                 help="read each step's tokens back before the next step is launched")
   p.add_argument("--seed", type=int, default=0)
 
 
@@ -34,7 +36,8 @@ def _engine(args):
   return LLMEngine(model=args.model, dtype=args.dtype, max_num_seqs=args.max_num_seqs,
                    max_model_len=args.max_model_len, page_size=args.page_size, num_pages=args.num_pages,
                    max_num_batched_tokens=args.max_num_batched_tokens,
-                   enable_chunked_prefill=not args.no_chunked_prefill, enforce_eager=args.eager, seed=args.seed)
+                   enable_chunked_prefill=not args.no_chunked_prefill, enforce_eager=args.eager, enable_overlap=not args.no_overlap,
+                   seed=args.seed)
 
 
 def cmd_generate(args) -> int:

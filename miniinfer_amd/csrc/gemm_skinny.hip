@@ -313,9 +313,6 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
   return 0;
 }
 
-// Tuning knob for experiments: waves per workgroup (0 = chosen from the shape).
-static int g_waves_override = 0;
-MI_EXPORT void mi_gemm_skinny_set_waves(int waves) { g_waves_override = waves; }
 
 // A [M, K], C [M, N] bfloat16 or float32; W [N, K], or with gate_up the fused matrix [2 N, K].
 MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
@@ -335,7 +332,6 @@ MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t ld
   if (waves > 16) waves = 16;
   if (waves > steps / 2) waves = steps / 2;
   if (waves < 1) waves = 1;
-  if (g_waves_override > 0) waves = g_waves_override;
   const int MB = (M + 15) / 16;
   size_t lds = waves > 1 ? (size_t)waves * RB * MB * 1024 : 0;
   while (lds > 64 * 1024 && waves > 1) {     // the default LDS allotment of a workgroup
