@@ -28,7 +28,11 @@ CSRC = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)),
 
 # packed 32-bit float instructions are switched off for every kernel of this library
 HIPCC_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+               # MFMA results stay in ordinary vector registers: the kernels here read every product's
+               # accumulators with vector instructions at once, and copies to and from the accumulation
+               # registers were a third of the attention loop's instructions
+               "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
