@@ -139,8 +139,10 @@ def main() -> int:
   mid_context = args.context + args.warmup + args.steps // 2
   bytes_step = decode_bytes(cfg, layers, args.batch, mid_context, esize)
   achieved = bytes_step / sec / 1e9
+  shape_name = {"qwen3-0.6b": "Qwen3-0.6B", "qwen3-8b": "Qwen3-8B", "qwen3-32b": "Qwen3-32B"}.get(args.preset, args.preset)
   rec = {
-    "metric": "decode tok/s @ batch 8, 2,048-token contexts, Qwen3-0.6B shape", "value": round(value, 2),
+    "metric": f"decode tok/s @ batch {args.batch}, {args.context:,}-token contexts, {shape_name} shape",
+    "value": round(value, 2),
     "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4),
     "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
     "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (seeded random token ids, random weights)",

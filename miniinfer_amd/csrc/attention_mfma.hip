@@ -342,62 +342,72 @@ __device__ __forceinline__ void prefill_body(
   // This thread's chunks of a macro tile: page numbers from the block table (PREFILL_PAGES), global -> registers
   // (PREFILL_FETCH), registers -> LDS (PREFILL_STASH).  The page numbers are asked for one tile earlier than the
   // keys and values that need them, so that no step of the loop waits for two dependent loads in a row.
+  // Everything about a chunk that does not change from tile to tile is worked out once: which key of the tile
+  // and which 16 bytes of it (keys), which dim and which run of 8 keys (values; chunk -> (page of the tile, dim,
+  // run) so that consecutive threads read consecutive memory of a page), and where it goes in LDS.
   const int kpp = P < MKEYS ? P : MKEYS;   // keys of a macro tile that lie in one page
   const int cpp = kpp / 8;                 // 16-byte chunks per (page, dim)
   u32x4 pk[LDS_KITER], pv[LDS_VITER];
   int kpage[LDS_KITER], vpage[LDS_VITER];
-#define PREFILL_KEY_OF_KCHUNK(J0, IT, KEY)                                                                           \
-  int ch = threadIdx.x + 256 * (IT);                                                                                 \
-  ch = ch < LDS_KCHUNKS ? ch : LDS_KCHUNKS - 1; /* threads past the end load the last chunk again, drop it */       \
-  int KEY = (J0) + ch / (D / 8);                                                                                     \
-  KEY = KEY > last ? last : KEY; /* masked keys read valid memory of the request */
-#define PREFILL_KEY_OF_VCHUNK(J0, IT, KEY)                                                                           \
-  int ch = threadIdx.x + 256 * (IT);                                                                                 \
-  ch = ch < LDS_VCHUNKS ? ch : LDS_VCHUNKS - 1;                                                                      \
-  /* chunk -> (page of the tile, dim, run of 8 keys): consecutive threads read consecutive memory of a page */      \
-  const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);                                          \
-  int KEY = (J0) + page_i * kpp + 8 * part;                                                                          \
-  KEY = KEY > last ? (last & ~7) : KEY; /* a run of 8 keys lies in one page */
+  int k_key[LDS_KITER], k_col[LDS_KITER], k_lds[LDS_KITER];    // key in the tile, first element, LDS element offset
+  int v_key[LDS_VITER], v_dim[LDS_VITER], v_lds[LDS_VITER];    // first key of the run in the tile, dim, LDS offset
+#pragma unroll
+  for (int it = 0; it < LDS_KITER; ++it) {
+    int ch = threadIdx.x + 256 * it;
+    k_lds[it] = ch < LDS_KCHUNKS ? (ch / (D / 8)) * LDS_KSTR + 8 * (ch % (D / 8)) : -1;
+    ch = ch < LDS_KCHUNKS ? ch : LDS_KCHUNKS - 1;   // threads past the end load the last chunk again and drop it
+    k_key[it] = ch / (D / 8);
+    k_col[it] = 8 * (ch % (D / 8));
+  }
+#pragma unroll
+  for (int it = 0; it < LDS_VITER; ++it) {
+    int ch = threadIdx.x + 256 * it;
+    const bool live = ch < LDS_VCHUNKS;
+    ch = live ? ch : LDS_VCHUNKS - 1;
+    const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);
+    v_key[it] = page_i * kpp + 8 * part;
+    v_dim[it] = dim;
+    v_lds[it] = live ? dim * LDS_VSTR + page_i * kpp + 8 * part : -1;
+  }
+  const uint16_t* kbase = k_pages + (int64_t)g * P * D;     // + page * page_stride + (slot in page) * D + element
+  const uint16_t* vbase = v_pages + (int64_t)g * D * P;     // + page * page_stride + dim * P + slot in page
+  const int page_stride = nkv * P * D;                      // elements; a page of one layer is far below 2^31
 #define PREFILL_PAGES(J0)                                                                                            \
   {                                                                                                                  \
     _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
-      PREFILL_KEY_OF_KCHUNK(J0, it, key)                                                                             \
+      const int key = min((J0) + k_key[it], last); /* masked keys read valid memory of the request */               \
       kpage[it] = bt[key >> page_shift];                                                                             \
     }                                                                                                                \
     _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
-      PREFILL_KEY_OF_VCHUNK(J0, it, key)                                                                             \
-      (void)dim;                                                                                                     \
+      int key = (J0) + v_key[it];                                                                                    \
+      key = key > last ? (last & ~7) : key; /* a run of 8 keys lies in one page */                                  \
       vpage[it] = bt[key >> page_shift];                                                                             \
     }                                                                                                                \
   }
 #define PREFILL_FETCH(J0)                                                                                            \
   {                                                                                                                  \
     _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
-      PREFILL_KEY_OF_KCHUNK(J0, it, key)                                                                             \
-      pk[it] = *reinterpret_cast<const u32x4*>(k_pages + (((int64_t)kpage[it] * nkv + g) * P + (key & (P - 1))) * D + \
-                                               8 * (ch % (D / 8)));                                                  \
+      const int key = min((J0) + k_key[it], last);                                                                   \
+      pk[it] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kpage[it] * page_stride +                            \
+                                               ((key & (P - 1)) * D + k_col[it]));                                   \
     }                                                                                                                \
     _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
-      PREFILL_KEY_OF_VCHUNK(J0, it, key)                                                                             \
-      pv[it] = *reinterpret_cast<const u32x4*>(v_pages + (((int64_t)vpage[it] * nkv + g) * D + dim) * P +            \
-                                               (key & (P - 1)));                                                     \
+      int key = (J0) + v_key[it];                                                                                    \
+      key = key > last ? (last & ~7) : key;                                                                          \
+      pv[it] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)vpage[it] * page_stride +                            \
+                                               (v_dim[it] * P + (key & (P - 1))));                                   \
     }                                                                                                                \
   }
 #define PREFILL_STASH()                                                                                              \
   {                                                                                                                  \
-    _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
-      const int ch = threadIdx.x + 256 * it;                                                                         \
-      if (ch < LDS_KCHUNKS) *reinterpret_cast<u32x4*>(Ks + (ch / (D / 8)) * LDS_KSTR + 8 * (ch % (D / 8))) = pk[it]; \
-    }                                                                                                                \
-    _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
-      const int ch = threadIdx.x + 256 * it;                                                                         \
-      const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);                                      \
-      if (ch < LDS_VCHUNKS) { /* rows are 8-byte aligned only: two 64-bit writes */                                  \
-        u32x2* dst = reinterpret_cast<u32x2*>(Vs + dim * LDS_VSTR + page_i * kpp + 8 * part);                        \
+    _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it)                                                         \
+      if (k_lds[it] >= 0) *reinterpret_cast<u32x4*>(Ks + k_lds[it]) = pk[it];                                        \
+    _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it)                                                         \
+      if (v_lds[it] >= 0) { /* rows are 8-byte aligned only: two 64-bit writes */                                    \
+        u32x2* dst = reinterpret_cast<u32x2*>(Vs + v_lds[it]);                                                       \
         dst[0] = u32x2{pv[it][0], pv[it][1]};                                                                        \
         dst[1] = u32x2{pv[it][2], pv[it][3]};                                                                        \
       }                                                                                                              \
-    }                                                                                                                \
   }
 
   PREFILL_PAGES(wg_lo)
@@ -434,8 +444,6 @@ __device__ __forceinline__ void prefill_body(
     }
   }
 #undef PREFILL_PAGES
-#undef PREFILL_KEY_OF_KCHUNK
-#undef PREFILL_KEY_OF_VCHUNK
 #undef PREFILL_FETCH
 #undef PREFILL_STASH
   store_output<NB>(st, out + (int64_t)(q_begin + tok0) * out_row_stride, out_row_stride, gpad, g * G, pos_hi);
