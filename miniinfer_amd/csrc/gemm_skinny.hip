@@ -25,11 +25,28 @@ __device__ __forceinline__ bf16x8 zero_bf16x8() {
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.f + expf(-g)); }
 
+// Two optional halves of an RMS norm that sits between two products, so that the norm needs no kernel of its own.
+// After the first product (`residual` set): instead of C, the workgroup adds its result to the 32-bit residual
+// stream in place, r[m][n] += result, writes the next product's left operand a_out[m][n] = bf16(r[m][n] * w[n]),
+// and the sum of r[m][n]^2 over its own columns n to ss_out[blockIdx.x][m] (rows of 64).
+// Before the second product's result is stored (`row_ss` set): row m is scaled by rsqrt(sum_p row_ss[p][m] / K +
+// eps), the norm's missing factor (K, the length of the normed rows, is this product's K).
+struct NormHalves {
+  const float* row_ss;      // [ss_parts][64]
+  int ss_parts;
+  float eps;
+  float* residual;          // [M, N] float32, leading dimension N
+  const float* norm_weight; // [N]
+  uint16_t* a_out;          // [M, N] bfloat16, leading dimension N
+  float* ss_out;            // [gridDim.x][64]
+};
+
 template <int MB, int RB, bool OUT_F32, bool GATE_UP>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __restrict__ A, int64_t lda,
                                                            const uint16_t* __restrict__ W, int64_t ldw,
-                                                           void* __restrict__ C, int64_t ldc, int M, int N, int K) {
-  extern __shared__ float red[];   // [waves][RB * MB][256]
+                                                           void* __restrict__ C, int64_t ldc, int M, int N, int K,
+                                                           NormHalves nh) {
+  extern __shared__ float red[];   // [(waves + 1) / 2][RB * MB][256], then (norm halves) [OB * 256] squares, [waves][64] sums
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
@@ -61,6 +78,30 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     const int m = 16 * mb + (lane & 15);
     mok[mb] = m < M;
     arow[mb] = A + (int64_t)(mok[mb] ? m : 0) * lda;
+  }
+
+  // What the norm halves read is asked for before the weights, so that the end of the kernel does not wait for
+  // memory again: the partial sums of squares of row (thread % 64), parts (thread / 64), + waves, ...; and the
+  // residual and norm weight of the first two result elements this thread will finish.
+  constexpr int OBLK = GATE_UP ? MB : RB * MB;
+  float my_ss = 0.f;
+  if (nh.row_ss) {
+    const int m = threadIdx.x & 63;
+    for (int p = wave; p < nh.ss_parts; p += nw) my_ss += nh.row_ss[(int64_t)p * 64 + m];
+  }
+  float r_pre[2] = {0.f, 0.f}, w_pre[2] = {0.f, 0.f};
+  if (nh.residual) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = threadIdx.x + j * blockDim.x;
+      const int blk = e >> 8, ln = (e & 255) >> 2, i = e & 3;
+      const int n = n0 + 16 * (blk / MB) + 4 * (ln >> 4) + i;
+      const int m = 16 * (blk % MB) + (ln & 15);
+      if (e < OBLK * 256 && n < N && m < M) {
+        r_pre[j] = nh.residual[(int64_t)m * N + n];
+        w_pre[j] = nh.norm_weight[n];
+      }
+    }
   }
 
   // Steps are taken CH at a time: first every load of the chunk is issued (weights, and the raw left operand),
@@ -98,47 +139,79 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     }
   }
 
-  // lane holds C^T[n0 + 16 rb + 4 (lane / 16) + i][16 mb + lane % 16]
+  // lane holds C^T[n0 + 16 rb + 4 (lane / 16) + i][16 mb + lane % 16].  The waves' blocks are added through LDS in
+  // two rounds, which halves the LDS they need: the upper half of the waves leaves its blocks there, the lower
+  // half adds them to its own (each lane the very words it holds) and leaves the sums; then the workgroup's
+  // threads share out the elements of the result.
   constexpr int OB = GATE_UP ? MB : RB * MB;          // output blocks of the workgroup
-  if (nw > 1) {
+  const int hw = (nw + 1) / 2;                        // waves whose sums stay in LDS
+  float* sq = red + hw * RB * MB * 256;               // [OB * 256] squares of the new residual (norm halves only)
+  float* ss_part = sq + OB * 256;                     // [waves][64]
+  if (wave >= hw) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
-        *reinterpret_cast<f32x4*>(red + ((wave * RB * MB + rb * MB + mb) * 64 + lane) * 4) = acc[rb][mb];
-    __syncthreads();
-    // element e of the workgroup's result: block e / 256, lane (e % 256) / 4, register e % 4
-    for (int e = threadIdx.x; e < OB * 256; e += blockDim.x) {
-      const int blk = e >> 8, r = e & 255;
-      float v = 0.f, u = 0.f;
-      for (int w = 0; w < nw; ++w) {
-        v += red[(w * RB * MB + blk) * 256 + r];
-        if (GATE_UP) u += red[(w * RB * MB + MB + blk) * 256 + r];
+        *reinterpret_cast<f32x4*>(red + (((wave - hw) * RB * MB + rb * MB + mb) * 64 + lane) * 4) = acc[rb][mb];
+  }
+  if (nh.row_ss) ss_part[wave * 64 + lane] = my_ss;
+  __syncthreads();
+  if (wave < hw) {
+    const bool partner = wave + hw < nw;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        f32x4* p = reinterpret_cast<f32x4*>(red + ((wave * RB * MB + rb * MB + mb) * 64 + lane) * 4);
+        *p = partner ? *p + acc[rb][mb] : acc[rb][mb];
       }
-      if (GATE_UP) v = silu_f(v) * u;
-      const int ln = r >> 2, i = r & 3;
-      const int n = n0 + 16 * (GATE_UP ? 0 : blk / MB) + 4 * (ln >> 4) + i;
-      const int m = 16 * (blk % MB) + (ln & 15);
-      if (n < N && m < M) {
-        if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n] = v;
-        else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n] = float_to_bf16_bits(v);
-      }
+  }
+  __syncthreads();
+  // element e of the workgroup's result: block e / 256, lane (e % 256) / 4, register e % 4
+  for (int e = threadIdx.x; e < OB * 256; e += blockDim.x) {
+    const int blk = e >> 8, r = e & 255;
+    float v = 0.f, u = 0.f;
+    for (int w = 0; w < hw; ++w) {
+      v += red[(w * RB * MB + blk) * 256 + r];
+      if (GATE_UP) u += red[(w * RB * MB + MB + blk) * 256 + r];
     }
-  } else {
-#pragma unroll
-    for (int ob = 0; ob < OB; ++ob) {
-      const int rb = GATE_UP ? 0 : ob / MB, mb = ob % MB;
-      const int m = 16 * mb + (lane & 15);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + 16 * rb + 4 * (lane >> 4) + i;
-        float v = acc[rb][mb][i];
-        if (GATE_UP) v = silu_f(v) * acc[GATE_UP ? 1 : 0][mb][i];
-        if (n < N && m < M) {
-          if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n] = v;
-          else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n] = float_to_bf16_bits(v);
-        }
+    const int ln = r >> 2, i = r & 3;
+    const int n = n0 + 16 * (GATE_UP ? 0 : blk / MB) + 4 * (ln >> 4) + i;
+    const int m = 16 * (blk % MB) + (ln & 15);
+    if (nh.row_ss) {
+      float total = 0.f;
+      for (int w = 0; w < nw; ++w) total += ss_part[w * 64 + m];
+      const float rstd = rsqrtf(total / (float)K + nh.eps);
+      v *= rstd;
+      u *= rstd;
+    }
+    if (GATE_UP) v = silu_f(v) * u;
+    const bool live = n < N && m < M;
+    if (nh.residual) {
+      float rv = 0.f;
+      if (live) {
+        const int j = (e - (int)threadIdx.x) / (int)blockDim.x;
+        const float r_old = j == 0 ? r_pre[0] : (j == 1 ? r_pre[1] : nh.residual[(int64_t)m * N + n]);
+        const float w_n = j == 0 ? w_pre[0] : (j == 1 ? w_pre[1] : nh.norm_weight[n]);
+        rv = r_old + v;
+        nh.residual[(int64_t)m * N + n] = rv;
+        nh.a_out[(int64_t)m * N + n] = float_to_bf16_bits(rv * w_n);
       }
+      sq[e] = rv * rv;
+    } else if (live) {
+      if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n] = v;
+      else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n] = float_to_bf16_bits(v);
+    }
+  }
+  if (nh.residual) {
+    // row m's squares over this workgroup's columns, summed in a fixed order by one thread
+    __syncthreads();
+    for (int m = threadIdx.x; m < 16 * MB; m += blockDim.x) {
+      float total = 0.f;
+      for (int rb = 0; rb < (GATE_UP ? 1 : RB); ++rb)
+        for (int q = 0; q < 4; ++q)
+          for (int i = 0; i < 4; ++i) total += sq[(rb * MB + (m >> 4)) * 256 + 4 * ((m & 15) + 16 * q) + i];
+      nh.ss_out[(int64_t)blockIdx.x * 64 + m] = total;
     }
   }
 }
@@ -291,15 +364,20 @@ MI_EXPORT int mi_norm_gemm_skinny(int gate_up, const float* R, const void* X, fl
   return 0;
 }
 
+static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up) {
+  const int OB = gate_up ? MB : RB * MB;
+  return ((size_t)((waves + 1) / 2) * RB * MB * 256 + (size_t)OB * 256 + (size_t)waves * 64) * sizeof(float);
+}
+
 template <int MB, int RB>
 static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
-                  int64_t ldc, int M, int N, int K, int waves, hipStream_t stream) {
+                  int64_t ldc, int M, int N, int K, int waves, const NormHalves& nh, hipStream_t stream) {
   const dim3 grid(gate_up ? (N + 15) / 16 : (N + 16 * RB - 1) / (16 * RB));
   const dim3 block(64 * waves);
-  const size_t lds = waves > 1 ? (size_t)waves * RB * MB * 256 * sizeof(float) : 0;
+  const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up);
 #define GO(F32, GU)                                                                                              \
   gemm_skinny_kernel<MB, RB, F32, GU><<<grid, block, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, \
-                                                                    ldw, C, ldc, M, N, K)
+                                                                    ldw, C, ldc, M, N, K, nh)
   if (gate_up) {
     if constexpr (RB == 2) {
       if (out_f32) GO(true, true);
@@ -313,15 +391,29 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
   return 0;
 }
 
+// Workgroups of the launch for an [N, K] matrix (the number of rows of 64 that `ss_out` must hold).
+MI_EXPORT int mi_gemm_skinny_groups(int gate_up, int N) {
+  const int row_blocks = (N + 15) / 16;
+  const int RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
+  return gate_up ? row_blocks : (row_blocks + RB - 1) / RB;
+}
 
 // A [M, K], C [M, N] bfloat16 or float32; W [N, K], or with gate_up the fused matrix [2 N, K].
-MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
-                             int64_t ldc, int M, int N, int K, hipStream_t stream) {
+// Norm halves (see NormHalves; all optional): row_ss [ss_parts][64] and eps scale the rows of the result;
+// residual [M, N] float32 + norm_weight [N] + a_out [M, N] bfloat16 + ss_out [groups][64] replace C.
+MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw,
+                                void* C, int64_t ldc, int M, int N, int K, const float* row_ss, int ss_parts,
+                                float eps, float* residual, const float* norm_weight, void* a_out, float* ss_out,
+                                hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);
   MI_REQUIRE(lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: row strides (%lld, %lld) must be multiples of 8", (long long)lda,
              (long long)ldw);
-  MI_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_skinny: leading dimensions too small");
+  MI_REQUIRE(lda >= K && ldw >= K, "gemm_skinny: leading dimensions too small");
+  MI_REQUIRE(residual || (C && ldc >= N), "gemm_skinny: no result buffer");
+  MI_REQUIRE(!residual || (norm_weight && a_out && ss_out && !gate_up),
+             "gemm_skinny: the residual form needs norm_weight, a_out and ss_out, and no gate|up");
+  MI_REQUIRE(!row_ss || ss_parts > 0, "gemm_skinny: row_ss without parts");
   if (M == 0) return 0;
   const int row_blocks = (N + 15) / 16;
   const int RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
@@ -333,18 +425,21 @@ MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t ld
   if (waves > steps / 2) waves = steps / 2;
   if (waves < 1) waves = 1;
   const int MB = (M + 15) / 16;
-  size_t lds = waves > 1 ? (size_t)waves * RB * MB * 1024 : 0;
-  while (lds > 64 * 1024 && waves > 1) {     // the default LDS allotment of a workgroup
-    waves /= 2;
-    lds = waves > 1 ? (size_t)waves * RB * MB * 1024 : 0;
-  }
+  while (skinny_lds_bytes(waves, RB, MB, gate_up != 0) > 64 * 1024 && waves > 1) waves /= 2;   // the default LDS allotment
+  const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \
-    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, stream);              \
+    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, nh, stream);          \
     MI_CHECK_LAUNCH("gemm_skinny");                                                                           \
     return 0;                                                                                                 \
   }
   CASE(1, 1) CASE(2, 1) CASE(3, 1) CASE(4, 1) CASE(1, 2) CASE(2, 2) CASE(3, 2) CASE(4, 2)
 #undef CASE
   MI_FAIL("gemm_skinny: no instance for M=%d", M);
+}
+
+MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                             int64_t ldc, int M, int N, int K, hipStream_t stream) {
+  return mi_gemm_skinny_ex(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, nullptr, 0, 0.f, nullptr, nullptr,
+                           nullptr, nullptr, stream);
 }

@@ -14,7 +14,7 @@ import torch
 
 from ..kernels import ops
 from .base import (BuildContext, NORMS, POSITIONS, PagedKV, ParamSpec, Part, Source, register_mixer)
-from .linear import linear
+from .linear import PendingLinear, linear
 
 
 class PagedAttention(Part):
@@ -62,6 +62,11 @@ class PagedAttention(Part):
 
   # ------------------------------------------------------------------ one step
   def forward(self, x, ctx, cache) -> torch.Tensor:
+    return self.forward_lazy(x, ctx, cache).materialize()
+
+  def forward_lazy(self, x, ctx, cache) -> PendingLinear:
+    """The same with the output projection left pending, so that the block can fold the add and the next norm
+    into it."""
     T = x.shape[0]
     qkv = linear(x, self.qkv_weight)
     table = self.position.rotary_table()
@@ -71,7 +76,7 @@ class PagedAttention(Part):
       # a step of decoded tokens only: the attention kernel norms, rotates and caches by itself
       out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
       self._attend_decode(qkv, out, ctx, cache, 0, ctx.num_requests, front=(table, eps))
-      return linear(out, self.o_weight)
+      return PendingLinear(out, self.o_weight)
     if self.shares_kv:
       # only queries of its own: they are normed and rotated; the borrowed pages are read, never written
       ops.qk_norm_rope_cache(qkv, self.nq, 0, self.d, self.q_norm.weight if self.q_norm is not None else None, None,
@@ -84,7 +89,7 @@ class PagedAttention(Part):
         eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
     out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
     self._attend(qkv, out, ctx, cache)
-    return linear(out, self.o_weight)
+    return PendingLinear(out, self.o_weight)
 
   def _attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx, cache) -> None:
     nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0

@@ -35,18 +35,22 @@ class PreNormBlock(Part):
     Returns (this block's pending output, the residual stream), which may be a new buffer.
 
     A part that sets `takes_deferred_norm` gets its input as a DeferredNorm and may fuse the add and the norm into
-    its own first kernel; any other part gets the normed tensor."""
+    its own first kernel; any other part gets the normed tensor.  A part that has `forward_lazy` may return its
+    last product still pending (`PendingLinear`); the pending output (h, and what this returns) goes into the next
+    norm as it is."""
     x = self.mixer_norm.defer(h, residual)
     if not getattr(self.mixer, "takes_deferred_norm", False):
       x.materialize()
-    a = self.mixer.forward(x if getattr(self.mixer, "takes_deferred_norm", False) else x.value, ctx, cache)
+    run = getattr(self.mixer, "forward_lazy", self.mixer.forward)
+    a = run(x if getattr(self.mixer, "takes_deferred_norm", False) else x.value, ctx, cache)
     if not x.consumed:
       x.materialize()       # a mixer that ignored its input still leaves the residual updated
     residual = x.residual
     y = self.ff_norm.defer(a, residual)
     if not getattr(self.feed_forward, "takes_deferred_norm", False):
       y.materialize()
-    m = self.feed_forward.forward(y if getattr(self.feed_forward, "takes_deferred_norm", False) else y.value, ctx)
+    run = getattr(self.feed_forward, "forward_lazy", self.feed_forward.forward)
+    m = run(y if getattr(self.feed_forward, "takes_deferred_norm", False) else y.value, ctx)
     if not y.consumed:
       y.materialize()
     return m, y.residual

@@ -16,12 +16,61 @@ import torch
 from ..kernels import ops
 
 
+class PendingLinear:
+  """a @ W^T that has not been computed yet.  A part may hand this to the block instead of a tensor
+  (`forward_lazy`): when a norm and another product follow, the add to the residual stream and the norm are
+  split between the two products' kernels (`_fuse_norm`) and need none of their own; anyone else calls
+  `materialize()`."""
+
+  def __init__(self, a: torch.Tensor, weight: torch.Tensor):
+    self.a = a
+    self.weight = weight
+    self.value: Optional[torch.Tensor] = None
+
+  @property
+  def shape(self):
+    return (self.a.shape[0], self.weight.shape[0])
+
+  @property
+  def dtype(self):
+    return self.a.dtype
+
+  @property
+  def device(self):
+    return self.a.device
+
+  def materialize(self) -> torch.Tensor:
+    if self.value is None:
+      self.value = linear(self.a, self.weight)
+    return self.value
+
+
+def as_tensor(x) -> Optional[torch.Tensor]:
+  """A tensor from what a part returned: a tensor, None, or a pending product."""
+  return x.materialize() if isinstance(x, PendingLinear) else x
+
+
 def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]:
-  """The product of a deferred norm with `weight` in one kernel, when the shapes allow it."""
+  """The product of a deferred norm with `weight` without a kernel for the norm, when the shapes allow it."""
   M = d.residual.shape[0]
-  if d.consumed or d.dtype != torch.bfloat16 or not ops.norm_gemm_supported(M, d.residual, d.x, weight):
+  if d.consumed or d.dtype != torch.bfloat16:
     return None
   N = weight.shape[0] // 2 if gate_up else weight.shape[0]
+  if isinstance(d.x, PendingLinear) and d.x.value is None:
+    # The branch's last product is still pending: its kernel adds to the residual stream in place and leaves
+    # bfloat16(residual * norm weight) and partial sums of squares; this product's kernel scales its rows by them.
+    p = d.x
+    if ops.gemm_skinny_into_norm_supported(p.a, p.weight, d.residual, d.norm.weight) \
+        and weight.dtype == torch.bfloat16 and weight.shape[1] == d.residual.shape[1] and weight.stride(1) == 1 \
+        and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0:
+      operand, row_ss = ops.gemm_skinny_into_norm(p.a, p.weight, d.residual, d.norm.weight)
+      out = torch.empty((M, N), dtype=torch.bfloat16, device=d.device)
+      ops.gemm_skinny_scaled(operand, weight, out, row_ss, d.norm.eps, gate_up=gate_up)
+      d.fused(d.residual)
+      return out
+    d.x = p.materialize()
+  if not ops.norm_gemm_supported(M, d.residual, d.x, weight):
+    return None
   out = torch.empty((M, N), dtype=torch.bfloat16, device=d.device)
   new_res = torch.empty_like(d.residual) if d.x is not None else None
   ops.norm_gemm_skinny(d.residual, d.x, d.norm.weight, d.norm.eps, weight, out, residual_out=new_res,

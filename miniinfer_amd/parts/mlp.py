@@ -8,7 +8,7 @@ from typing import List, Optional
 import torch
 
 from .base import BuildContext, ParamSpec, Part, Source, register_feed_forward
-from .linear import gate_up_activation, linear
+from .linear import PendingLinear, gate_up_activation
 
 
 class GatedMLP(Part):
@@ -32,7 +32,11 @@ class GatedMLP(Part):
     ]
 
   def forward(self, x, ctx) -> torch.Tensor:
-    return linear(gate_up_activation(x, self.gate_up_weight), self.down_weight)
+    return self.forward_lazy(x, ctx).materialize()
+
+  def forward_lazy(self, x, ctx) -> PendingLinear:
+    """The same with the down projection left pending, so that the block can fold the add and the next norm into it."""
+    return PendingLinear(gate_up_activation(x, self.gate_up_weight), self.down_weight)
 
 
 register_feed_forward("gated_mlp", GatedMLP)

@@ -15,7 +15,7 @@ import torch
 from ..config.spec import ModelSpec
 from ..kernels import ops
 from .base import BLOCKS, NORMS, BuildContext, ParamSpec, Part, Source
-from .linear import linear
+from .linear import as_tensor, linear
 
 
 class DecoderModel(Part):
@@ -77,5 +77,5 @@ class DecoderModel(Part):
     R = ctx.num_logit_rows
     if R == 0:
       return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.ctx.device)
-    x = self.final_norm.forward_residual(h, residual, rows=ctx.logit_rows)
+    x = self.final_norm.forward_residual(as_tensor(h), residual, rows=ctx.logit_rows)
     return linear(x, self.head if self.head is not None else self.embedding, out_dtype=torch.float32)

@@ -11,9 +11,10 @@ from .base import BuildContext, ParamSpec, Part, register_norm
 
 
 class DeferredNorm:
-  """norm(residual + x) that has not been computed yet.  A consumer that can fuse the add and the norm into its
-  own first kernel takes the pieces (`linear` and `gate_up_activation` do, for few rows); any other calls
-  `materialize()`.  After either, `residual` is the updated residual stream (it may be a new buffer)."""
+  """norm(residual + x) that has not been computed yet; x is a tensor, None, or a pending product.  A consumer
+  that can fuse the add and the norm into its own first kernel takes the pieces (`linear` and `gate_up_activation`
+  do, for few rows); any other calls `materialize()`.  After either, `residual` is the updated residual stream (it
+  may be a new buffer, or the old one updated in place)."""
 
   def __init__(self, norm: "RMSNorm", x: Optional[torch.Tensor], residual: torch.Tensor):
     self.norm = norm
@@ -38,6 +39,8 @@ class DeferredNorm:
     if self.value is None:
       if self.consumed:
         raise RuntimeError("a deferred norm was fused into one product and then asked for again")
+      if hasattr(self.x, "materialize"):       # a product that a part left pending
+        self.x = self.x.materialize()
       self.value = self.norm.forward_residual(self.x, self.residual)
       self.consumed = True
     return self.value

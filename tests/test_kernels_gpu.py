@@ -442,3 +442,35 @@ def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, win
     assert torch.equal(v_after[page, :, off], v[b])
     changed_k[page, :, off] = False
   assert not bool(changed_k.any())                       # no other slot was written
+
+
+@pytest.mark.parametrize("M,N,K,N2,gate_up", [(8, 1024, 2048, 6144, True), (1, 80, 96, 112, False), (16, 1024, 3072, 4096, False),
+                                               (40, 136, 264, 200, True), (64, 1024, 2048, 3072, False), (5, 88, 40, 24, False)])
+def test_norm_split_between_two_products(M, N, K, N2, gate_up):
+  """residual += a W1^T; y = rmsnorm(residual) * w; out = y W2^T (or the gated activation of it), the add and the
+  norm done half in the first product's kernel and half in the second's.  Against 64-bit arithmetic with the
+  kernels' rounding points restated: the second product's left operand is bfloat16(residual * w), and the row's
+  rsqrt(mean square + eps) scales its 32-bit sums."""
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(31)
+  eps = 3e-6
+  a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+  w1 = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(DEV)
+  r = (torch.randn(M, N, generator=g) * 2).to(DEV)
+  nw = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+  w2 = (torch.randn(2 * N2 if gate_up else N2, N, generator=g) * 0.1).bfloat16().to(DEV)
+  want_r = r.double() + a.double() @ w1.double().T
+  r_dev = r.clone()
+  operand, row_ss = ops.gemm_skinny_into_norm(a, w1, r_dev, nw)
+  torch.testing.assert_close(r_dev.double(), want_r, rtol=1e-5, atol=1e-4)
+  torch.testing.assert_close(operand.double(), (r_dev.double() * nw.double()).bfloat16().double(), rtol=1e-2, atol=1e-6)
+  torch.testing.assert_close(row_ss[:, :M].sum(0).double(), r_dev.double().pow(2).sum(-1), rtol=1e-5, atol=1e-5)
+  out = torch.empty(M, N2, dtype=torch.bfloat16, device=DEV)
+  ops.gemm_skinny_scaled(operand, w2, out, row_ss, eps, gate_up=gate_up)
+  rstd = torch.rsqrt(r_dev.double().pow(2).mean(-1, keepdim=True) + eps)
+  y = (operand.double() @ w2.double().T) * rstd
+  # ... which is the norm followed by the product, up to the operand's rounding
+  torch.testing.assert_close(y, torch.nn.functional.rms_norm(want_r, (N,), nw.double(), eps) @ w2.double().T,
+                             rtol=3e-2, atol=3e-2 * float(y.abs().max()))
+  want = torch.nn.functional.silu(y[:, :N2]) * y[:, N2:] if gate_up else y
+  torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
