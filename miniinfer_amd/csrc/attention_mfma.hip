@@ -288,16 +288,32 @@ constexpr int LDS_VCHUNKS = D * (MKEYS / 8);     // 16-byte chunks of a value ti
 constexpr int LDS_KITER = (LDS_KCHUNKS + 255) / 256;
 constexpr int LDS_VITER = (LDS_VCHUNKS + 255) / 256;
 
-template <int NB>
+// KG = 1: as described.  KG = 2: the workgroup has 8 waves and walks two macro tiles per step, staged side by side;
+// waves 0-3 take the first of each pair, waves 4-7 the second, for the same 4 query blocks, and at the end wave
+// w + 4 hands its running softmax state to wave w through LDS.  That halves the number of dependent steps of the
+// workgroup with the most keys, which is what a short prompt's launch waits for.
+template <int NB, int KG>
 __device__ __forceinline__ void prefill_body(
     const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ work, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int nq,
     int nkv, int gpad, int page_shift, float scale, int window) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[MKEYS * LDS_KSTR];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[D * LDS_VSTR];
+  constexpr int KS_TILE = MKEYS * LDS_KSTR, VS_TILE = D * LDS_VSTR;
+  __shared__ __attribute__((aligned(16))) uint16_t tiles[KG * (KS_TILE + VS_TILE)];   // keys, then values
+  uint16_t* Ks_all = tiles;
+  uint16_t* Vs_all = tiles + KG * KS_TILE;
+  static_assert((KG * KS_TILE) % 8 == 0, "the value tiles start on a 16-byte boundary");
+  static_assert(KG == 1 || (size_t)(KS_TILE + VS_TILE) * KG * 2 >= (size_t)4 * NB * (DBLK * 64 * 4 + 128) * 4,
+                "the tiles' LDS must hold four waves' states at the end");
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int kgroup = (threadIdx.x >> 6) >> 2;            // which macro tile of a step this wave multiplies
+  const int wave = (threadIdx.x >> 6) & 3;               // its query block within the workgroup
+  const int tid = threadIdx.x & 255;                     // the thread's place among those that stage one macro tile
+  const int stage = threadIdx.x >> 8;                    // and which macro tile of a step they stage
+  uint16_t* Ks = Ks_all + kgroup * KS_TILE;
+  uint16_t* Vs = Vs_all + kgroup * VS_TILE;
+  uint16_t* Ks_stage = Ks_all + stage * KS_TILE;
+  uint16_t* Vs_stage = Vs_all + stage * VS_TILE;
   // The kv head is the fastest grid index: workgroups go round the 8 XCDs by their linear index, so with 8 kv
   // heads (or a divisor or multiple of 8) all the workgroups that read one head's keys and values share an L2.
   const int b = work[2 * blockIdx.y], sb = work[2 * blockIdx.y + 1];
@@ -353,7 +369,7 @@ __device__ __forceinline__ void prefill_body(
   int v_key[LDS_VITER], v_dim[LDS_VITER], v_lds[LDS_VITER];    // first key of the run in the tile, dim, LDS offset
 #pragma unroll
   for (int it = 0; it < LDS_KITER; ++it) {
-    int ch = threadIdx.x + 256 * it;
+    int ch = tid + 256 * it;
     k_lds[it] = ch < LDS_KCHUNKS ? (ch / (D / 8)) * LDS_KSTR + 8 * (ch % (D / 8)) : -1;
     ch = ch < LDS_KCHUNKS ? ch : LDS_KCHUNKS - 1;   // threads past the end load the last chunk again and drop it
     k_key[it] = ch / (D / 8);
@@ -361,7 +377,7 @@ __device__ __forceinline__ void prefill_body(
   }
 #pragma unroll
   for (int it = 0; it < LDS_VITER; ++it) {
-    int ch = threadIdx.x + 256 * it;
+    int ch = tid + 256 * it;
     const bool live = ch < LDS_VCHUNKS;
     ch = live ? ch : LDS_VCHUNKS - 1;
     const int part = ch % cpp, dim = (ch / cpp) % D, page_i = ch / (cpp * D);
@@ -401,27 +417,31 @@ __device__ __forceinline__ void prefill_body(
 #define PREFILL_STASH()                                                                                              \
   {                                                                                                                  \
     _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it)                                                         \
-      if (k_lds[it] >= 0) *reinterpret_cast<u32x4*>(Ks + k_lds[it]) = pk[it];                                        \
+      if (k_lds[it] >= 0) *reinterpret_cast<u32x4*>(Ks_stage + k_lds[it]) = pk[it];                                  \
     _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it)                                                         \
       if (v_lds[it] >= 0) { /* rows are 8-byte aligned only: two 64-bit writes */                                    \
-        u32x2* dst = reinterpret_cast<u32x2*>(Vs + v_lds[it]);                                                       \
+        u32x2* dst = reinterpret_cast<u32x2*>(Vs_stage + v_lds[it]);                                                 \
         dst[0] = u32x2{pv[it][0], pv[it][1]};                                                                        \
         dst[1] = u32x2{pv[it][2], pv[it][3]};                                                                        \
       }                                                                                                              \
   }
 
-  PREFILL_PAGES(wg_lo)
-  PREFILL_FETCH(wg_lo)
-  PREFILL_PAGES(wg_lo + MKEYS)
-  for (int j0 = wg_lo; j0 < wg_hi; j0 += MKEYS) {
-    __syncthreads();                    // every wave is done with the tile that is in LDS
+  // a thread stages the macro tile `stage` of every step; a wave multiplies the macro tile `kgroup` of every step
+  constexpr int STEP = MKEYS * KG;
+  const int s_off = MKEYS * stage, c_off = MKEYS * kgroup;
+  PREFILL_PAGES(wg_lo + s_off)
+  PREFILL_FETCH(wg_lo + s_off)
+  PREFILL_PAGES(wg_lo + STEP + s_off)
+  for (int j0 = wg_lo; j0 < wg_hi; j0 += STEP) {
+    __syncthreads();                    // every wave is done with the tiles that are in LDS
     PREFILL_STASH()
     __syncthreads();
-    if (j0 + MKEYS < wg_hi) {
-      PREFILL_FETCH(j0 + MKEYS)
-      PREFILL_PAGES(j0 + 2 * MKEYS)
+    if (j0 + STEP < wg_hi) {
+      PREFILL_FETCH(j0 + STEP + s_off)
+      PREFILL_PAGES(j0 + 2 * STEP + s_off)
     }
-    if (j0 >= w_hi || j0 + MKEYS <= w_lo) continue;      // nothing this wave can see (same for all its lanes)
+    const int jt = j0 + c_off;          // this wave's macro tile
+    if (jt >= w_hi || jt + MKEYS <= w_lo) continue;      // nothing this wave can see (same for all its lanes)
     f32x4 s[MT][NB];
     s16x4 p[MT][NB];
 #pragma unroll
@@ -430,7 +450,7 @@ __device__ __forceinline__ void prefill_body(
       load_row(ka, Ks + (16 * t + (lane & 15)) * LDS_KSTR, true);
       tile_scores<NB>(s[t], ka, qr);
     }
-    softmax_update<NB>(st, s, p, c, j0, pos_lo, pos_hi);
+    softmax_update<NB>(st, s, p, c, jt, pos_lo, pos_hi);
 #pragma unroll
     for (int t = 0; t < MT; t += 2) {
       s16x4 va[2][DBLK];
@@ -446,6 +466,38 @@ __device__ __forceinline__ void prefill_body(
 #undef PREFILL_PAGES
 #undef PREFILL_FETCH
 #undef PREFILL_STASH
+  if constexpr (KG == 2) {
+    // wave w + 4 leaves its state where the tiles were; wave w folds it into its own (log-sum-exp rule, base 2)
+    __syncthreads();
+    float* hand = reinterpret_cast<float*>(Ks_all) + wave * NB * (DBLK * 256 + 128);
+    if (kgroup == 1) {
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        float* h = hand + nb * (DBLK * 256 + 128);
+#pragma unroll
+        for (int blk = 0; blk < DBLK; ++blk) *reinterpret_cast<f32x4*>(h + (blk * 64 + lane) * 4) = st.o[nb][blk];
+        h[DBLK * 256 + lane] = st.m[nb];
+        h[DBLK * 256 + 64 + lane] = st.l[nb];
+      }
+    }
+    __syncthreads();
+    if (kgroup == 1) return;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const float* h = hand + nb * (DBLK * 256 + 128);
+      const float m1 = h[DBLK * 256 + lane], l1 = h[DBLK * 256 + 64 + lane];
+      const float m_new = fmaxf(st.m[nb], m1);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float a0 = __builtin_amdgcn_exp2f(st.m[nb] - m_use), a1 = __builtin_amdgcn_exp2f(m1 - m_use);
+      st.m[nb] = m_new;
+      st.l[nb] = st.l[nb] * a0 + l1 * a1;
+#pragma unroll
+      for (int blk = 0; blk < DBLK; ++blk) {
+        const f32x4 o1 = *reinterpret_cast<const f32x4*>(h + (blk * 64 + lane) * 4);
+        st.o[nb][blk] = st.o[nb][blk] * a0 + o1 * a1;
+      }
+    }
+  }
   store_output<NB>(st, out + (int64_t)(q_begin + tok0) * out_row_stride, out_row_stride, gpad, g * G, pos_hi);
 }
 
@@ -459,13 +511,13 @@ __device__ __forceinline__ void prefill_body(
       gpad, page_shift, scale, window
 
 template <int NB>
-__global__ __launch_bounds__(256) void prefill_kernel(PREFILL_ARGS) {
-  prefill_body<NB>(PREFILL_PASS);
+__global__ __launch_bounds__(512) void prefill_kernel(PREFILL_ARGS) {      // few workgroups: 8 waves, two tiles a step
+  prefill_body<NB, 2>(PREFILL_PASS);
 }
 
 template <int NB>
 __global__ __launch_bounds__(256) PREFILL_DENSE_OCCUPANCY void prefill_dense_kernel(PREFILL_ARGS) {
-  prefill_body<NB>(PREFILL_PASS);
+  prefill_body<NB, 1>(PREFILL_PASS);
 }
 #undef PREFILL_ARGS
 #undef PREFILL_PASS
@@ -856,8 +908,10 @@ MI_EXPORT int mi_attn_prefill_tokens_per_block(int nq, int nkv) {
 MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, int64_t out_row_stride, const void* k_pages,
                               const void* v_pages, const int* block_table, int table_width, const int* work,
                               int num_work, const int* cu_q, const int* kv_len, int nq, int nkv, int page_size,
-                              float scale, int window, hipStream_t stream) {
+                              float scale, int window, int variant, hipStream_t stream) {
+  // variant: 0 = chosen from the grid's size; 1 = 8 waves, two macro tiles a step; 2 = 4 waves, three waves a SIMD
   if (check_common("attn_prefill", nq, nkv, page_size, q_row_stride, out_row_stride, table_width)) return 1;
+  MI_REQUIRE(variant >= 0 && variant <= 2, "attn_prefill: variant %d", variant);
   if (check_scale("attn_prefill", scale)) return 1;
   MI_REQUIRE(num_work >= 0 && window >= 0, "attn_prefill: bad work count or window");
   MI_REQUIRE(num_work <= 65535, "attn_prefill: %d work items; the grid takes at most 65535", num_work);
@@ -871,13 +925,13 @@ MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, in
         compute_units <= 0)
       compute_units = 256;
   }
-  if ((int64_t)num_work * nkv > 2 * (int64_t)compute_units)
+  if (variant == 2 || (variant == 0 && (int64_t)num_work * nkv > 2 * (int64_t)compute_units))
     prefill_dense_kernel<PREFILL_NB><<<grid, 256, 0, stream>>>(
         (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
         (const uint16_t*)v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv, group_pad(nq, nkv),
         log2_of(page_size), scale, window);
   else
-    prefill_kernel<PREFILL_NB><<<grid, 256, 0, stream>>>(
+    prefill_kernel<PREFILL_NB><<<grid, 512, 0, stream>>>(
         (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
         (const uint16_t*)v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv, group_pad(nq, nkv),
         log2_of(page_size), scale, window);

@@ -91,7 +91,7 @@ _SIGS = {
 
 _SIGS["attention_mfma"] = {
   "mi_attn_prefill": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
-                      c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                      c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
   "mi_attn_decode": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                      c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
   "mi_attn_decode_front": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
@@ -139,10 +139,6 @@ def _check(lib, rc):
   if rc != 0:
     raise KernelError(lib.mi_last_error().decode())
 
-
-def modules_for(spec_kinds=()):
-  """(name, defines) of every shared object the plain kernel set needs."""
-  return [("elementwise", ()), ("gemm", ()), ("attention", ())]
 
 
 def _check_pages(what, k_pages, v_pages, nkv, d, dtype):
@@ -514,11 +510,17 @@ def _attn_common(what, q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, 
   return B
 
 
+_PREFILL_VARIANTS = {"auto": 0, "two_tiles": 1, "dense": 2}
+
+
 def attn_prefill(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
                  v_pages: torch.Tensor, block_table: torch.Tensor, work: torch.Tensor, cu_q: torch.Tensor,
-                 kv_len: torch.Tensor, scale: float, window: int = 0) -> None:
+                 kv_len: torch.Tensor, scale: float, window: int = 0, variant: str = "auto") -> None:
   """MFMA attention of the entries named in `work` [n, 2] = (entry, block of `attn_prefill_tokens_per_block` query
-  tokens within it).  Other arguments as `paged_attention`."""
+  tokens within it).  Other arguments as `paged_attention`.  variant: "auto" (by the number of work items),
+  "two_tiles" (8 waves a workgroup, for few work items) or "dense" (4 waves, three waves a SIMD)."""
+  if variant not in _PREFILL_VARIANTS:
+    raise KernelError(f"attn_prefill: variant {variant!r}; known: {sorted(_PREFILL_VARIANTS)}")
   _attn_common("attn_prefill", q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len)
   _dev(work)
   _i32("work", work)
@@ -527,7 +529,8 @@ def attn_prefill(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, 
   lib = _lib("attention_mfma", (("HEAD_DIM", d),))
   _check(lib, lib.mi_attn_prefill(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages),
                                   _ptr(block_table), block_table.shape[1], _ptr(work), work.shape[0], _ptr(cu_q),
-                                  _ptr(kv_len), nq, nkv, k_pages.shape[2], float(scale), int(window), _stream()))
+                                  _ptr(kv_len), nq, nkv, k_pages.shape[2], float(scale), int(window),
+                                  _PREFILL_VARIANTS[variant], _stream()))
 
 
 def attn_decode(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
