@@ -17,7 +17,10 @@ from random import Random
 
 
 def _engine_args(p):
-  p.add_argument("--model", required=True, help="folder with config.json and *.safetensors")
+  p.add_argument("--model", default=None, help="folder with config.json and *.safetensors")
+  p.add_argument("--preset", default=None,
+                 help="instead of --model: a named shape (see `random-model`) with random weights drawn on the device")
+  p.add_argument("--num-hidden-layers", type=int, default=None, help="with --preset: fewer layers than the shape has")
   p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
   p.add_argument("--max-num-seqs", type=int, default=4, help="most sequences in a batch")
   p.add_argument("--max-model-len", type=int, default=512, help="most tokens of one sequence")
@@ -33,7 +36,13 @@ def _engine_args(p):
 
 def _engine(args):
   from miniinfer_amd import LLMEngine
-  return LLMEngine(model=args.model, dtype=args.dtype, max_num_seqs=args.max_num_seqs,
+  extra = {}
+  if (args.model is None) == (args.preset is None):
+    raise SystemExit("give exactly one of --model and --preset")
+  if args.preset is not None:
+    from miniinfer_amd.presets import preset
+    extra = dict(model_config=preset(args.preset, args.num_hidden_layers), random_weights_seed=args.seed)
+  return LLMEngine(model=args.model or "", **extra, dtype=args.dtype, max_num_seqs=args.max_num_seqs,
                    max_model_len=args.max_model_len, page_size=args.page_size, num_pages=args.num_pages,
                    max_num_batched_tokens=args.max_num_batched_tokens,
                    enable_chunked_prefill=not args.no_chunked_prefill, enforce_eager=args.eager, enable_overlap=not args.no_overlap,

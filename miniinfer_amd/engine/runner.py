@@ -154,6 +154,21 @@ class _DecodeGraph:
     self.graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(self.graph):
       self.logits = runner.model.forward(ctx)
+    self.ok = True
+    if B > _LIBRARY_FREE_ROWS:
+      # Beyond the rows this library's own product kernels take, the captured step holds library products.  What a
+      # library records into a graph is its own affair (clears of a workspace have replayed wrongly): the graph is
+      # replayed a few times, with eager work in between, against the eager result of the same (padding) inputs,
+      # and a graph that does not reproduce it is not used.
+      want = runner.model.forward(ctx).clone()
+      for _ in range(3):
+        self.graph.replay()
+        got = self.logits.clone()
+        torch.cuda.synchronize()
+        if not torch.allclose(got, want, rtol=1e-3, atol=1e-3):
+          self.ok = False
+          break
+        want = runner.model.forward(ctx).clone()
 
   def fill_padding(self, first: int) -> None:
     """Entries first.. are padding: token 0 at position 0 of a request of one key in the scratch page."""
@@ -178,12 +193,13 @@ class _DecodeGraph:
     return self.logits
 
 
-_GRAPH_BATCHES = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64)
+_GRAPH_BATCHES = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
+_LIBRARY_FREE_ROWS = 64       # up to here every product of a decode step is one of this library's kernels
 
 
 class ModelRunner:
   def __init__(self, model: DecoderModel, cache: CacheManager, use_graphs: bool = False):
-    """use_graphs: replay steps that hold only single decoded tokens (at most 64 of them) from HIP graphs,
+    """use_graphs: replay steps that hold only single decoded tokens (at most 256 of them) from HIP graphs,
     captured on demand per (batch bucket, block-table width bucket)."""
     self.model = model
     self.cache = cache
@@ -299,6 +315,9 @@ class ModelRunner:
     self._allow_future = allow_future
     if self.use_graphs and len(entries) <= _GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries):
       return self._step_from_graph(entries)
+    return self._step_eager(entries)
+
+  def _step_eager(self, entries: Sequence[StepEntry]) -> torch.Tensor:
     ctx, order, kv_lens = self.build_context(entries)
     logits = self.model.forward(ctx)
     for i, kv in zip(order, kv_lens):
@@ -318,6 +337,8 @@ class ModelRunner:
     if g is None:
       g = _DecodeGraph(self, Bb, Wb)
       self._graphs[(Bb, Wb)] = g
+    if not g.ok:
+      return self._step_eager(entries)
     self._fill(g.next_host(), g.layout, entries, order, q_lens, starts, kv_lens)
     g.fill_padding(B)
     logits = g.run()

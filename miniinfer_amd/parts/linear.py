@@ -94,6 +94,13 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
   if ops.gemm_skinny_supported(x, weight):
     # few rows (decode): the time is the time to stream the weights; this library's MFMA kernel
     return ops.gemm_skinny(x, weight, torch.empty((M, N), dtype=out_dtype, device=x.device))
+  if out_dtype == torch.float32 and M > ops.SKINNY_MAX_ROWS and ops.gemm_skinny_supported(x[:1], weight):
+    # 32-bit results from bfloat16 operands for more rows (the logits of many requests): the same kernel, 64 rows
+    # at a time; the weights stream once per 64 rows, which is still far quicker than the FMA kernel
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    for r0 in range(0, M, ops.SKINNY_MAX_ROWS):
+      ops.gemm_skinny(x[r0:r0 + ops.SKINNY_MAX_ROWS], weight, out[r0:r0 + ops.SKINNY_MAX_ROWS])
+    return out
   if x.dtype == torch.float32 or out_dtype != x.dtype:
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     return ops.gemm_nt(x, weight, out)

@@ -74,3 +74,37 @@ def test_engine_generates_the_same_with_and_without_graphs(tmp_path):
       res.append([o["token_ids"] for o in eng.generate(prompts, sps, use_tqdm=False)])
       assert bool(eng.runner._graphs) == (not eager)
   assert res[0] == res[1]
+
+
+def test_graphs_of_many_requests_hold_library_products_and_still_equal_eager_steps(tmp_path):
+  """Beyond 64 single tokens the products of a bfloat16 step are library calls, recorded into the graph with
+  whatever the library adds to them.  Each graph checks itself against the eager step when it is made; here
+  80 and then 100 requests decode for several steps through both paths, with eager work between the replays."""
+  from miniinfer_amd.cache.manager import CacheManager
+  from miniinfer_amd.engine.runner import ModelRunner, StepEntry
+  from miniinfer_amd.weights import load_model
+  cfg, _ = tm.make_model(str(tmp_path / "m"), "A", seed=8, dtype=torch.bfloat16, std=0.05)
+  runners = []
+  for graphs in (False, True):
+    model, _ = load_model(str(tmp_path / "m"), torch.bfloat16, "cuda:0")
+    cache = CacheManager(model.cache_needs(), page_size=16, num_pages=260, max_requests=128,
+                         max_model_len=model.spec.max_positions, dtype=torch.bfloat16, device="cuda:0")
+    runners.append(ModelRunner(model, cache, use_graphs=graphs))
+  outs = [[], []]
+  for k, rn in enumerate(runners):
+    live = []
+    for r in range(100):
+      if r == 80:
+        for t in range(4):
+          outs[k].append(rn.step([StepEntry(q, [(7 * q + t) % cfg["vocab_size"]], [0]) for q in live]).float().cpu())
+      rn.cache.admit(r)
+      rn.step([StepEntry(r, tm.random_tokens(cfg, 3 + r % 9, seed=r), [])])      # eager prompt step
+      live.append(r)
+    for t in range(4, 9):
+      outs[k].append(rn.step([StepEntry(q, [(7 * q + t) % cfg["vocab_size"]], [0]) for q in live]).float().cpu())
+      torch.cuda.synchronize()
+  assert {b for b, _ in runners[1]._graphs} == {96, 128}
+  assert all(g.ok for g in runners[1]._graphs.values()), "a graph with library products did not reproduce the eager step"
+  for e, g in zip(*outs):
+    assert e.shape == g.shape
+    assert float((e - g).abs().max()) <= 2e-2 * max(float(e.abs().max()), 1.0)
