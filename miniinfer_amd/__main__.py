@@ -107,7 +107,9 @@ def cmd_throughput(args) -> int:
     engine.generate(prompts=prompts, sampling_params=sps, use_tqdm=False)
     dt = time.time() - t0
   total = sum(sp.max_tokens for sp in sps)
-  print(f"[miniinfer_amd] Total: {total}tok, Time: {dt:.2f}s, Throughput: {total / dt:.2f}tok/s")
+  total_in = sum(len(p) for p in prompts)
+  print(f"[miniinfer_amd] Total: {total}tok, Time: {dt:.2f}s, Throughput: {total / dt:.2f}tok/s "
+        f"(input {total_in}tok, {total_in / dt:.2f}tok/s)")
   return 0
 
 
