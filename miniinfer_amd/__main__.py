@@ -103,6 +103,7 @@ def cmd_throughput(args) -> int:
                           max_tokens=rnd.randint(min(100, args.max_output_len), args.max_output_len))
            for _ in range(args.num_seqs)]
     engine.generate(prompts=[prompts[0][:8]], sampling_params=SamplingParams(), use_tqdm=False)   # warm-up
+    engine.warm_up(min(args.num_seqs, args.max_num_seqs), min(args.max_model_len, args.max_input_len + args.max_output_len))
     t0 = time.time()
     engine.generate(prompts=prompts, sampling_params=sps, use_tqdm=False)
     dt = time.time() - t0

@@ -148,6 +148,11 @@ class LLMEngine:
     self._requests[rid] = req
     return rid
 
+  def warm_up(self, max_num_seqs: Optional[int] = None, max_tokens: Optional[int] = None) -> int:
+    """Captures the decode graphs ahead of their first use (every batch bucket up to `max_num_seqs`, every table
+    width up to `max_tokens` tokens a request; defaults: the engine's limits).  Returns the number of graphs."""
+    return self.runner.capture_graphs(max_num_seqs or self.config.max_num_seqs, max_tokens or self.max_model_len)
+
   def is_finished(self) -> bool:
     return self._pending is None and not self.scheduler.has_unfinished()
 

@@ -317,6 +317,33 @@ class ModelRunner:
       return self._step_from_graph(entries)
     return self._step_eager(entries)
 
+  def graph_buckets(self, num_requests: int, num_tokens: int):
+    """(batch bucket, block-table width bucket) of the graph that a step of `num_requests` single tokens replays
+    when the longest of them holds `num_tokens` tokens."""
+    cache = self.cache
+    Bb = next(b for b in _GRAPH_BATCHES if b >= num_requests)
+    W = max(1, -(-num_tokens // cache.page_size))
+    Wb = max(16, 1 << (W - 1).bit_length())
+    return Bb, min(Wb, max(cache.max_pages_per_request, W))
+
+  @torch.no_grad()
+  def capture_graphs(self, max_requests: int, max_tokens: int) -> int:
+    """Captures, ahead of their first use, the graphs of every batch bucket up to `max_requests` and every width
+    bucket up to `max_tokens` tokens (the reference captures its graphs when the engine starts:
+    miniinfer/engine/llm_engine.py:281-313).  Returns how many graphs there are."""
+    if not self.use_graphs:
+      return 0
+    widths = sorted({self.graph_buckets(1, n)[1] for n in
+                     [self.cache.page_size * (16 << i) for i in range(32) if self.cache.page_size * (16 << i) < max_tokens]
+                     + [max_tokens]})
+    for b in _GRAPH_BATCHES:
+      if b > max(1, max_requests) and b != self.graph_buckets(max(1, max_requests), 1)[0]:
+        continue
+      for w in widths:
+        if (b, w) not in self._graphs:
+          self._graphs[(b, w)] = _DecodeGraph(self, b, w)
+    return len(self._graphs)
+
   def _step_eager(self, entries: Sequence[StepEntry]) -> torch.Tensor:
     ctx, order, kv_lens = self.build_context(entries)
     logits = self.model.forward(ctx)
@@ -329,10 +356,7 @@ class ModelRunner:
     cache = self.cache
     order, q_lens, starts, kv_lens = self._plan(entries)     # all single tokens: order is the given order
     B = len(entries)
-    Bb = next(b for b in _GRAPH_BATCHES if b >= B)
-    W = max(1, max(-(-kv // cache.page_size) for kv in kv_lens))
-    Wb = max(16, 1 << (W - 1).bit_length())
-    Wb = min(Wb, max(cache.max_pages_per_request, W))
+    Bb, Wb = self.graph_buckets(B, max(kv_lens))
     g = self._graphs.get((Bb, Wb))
     if g is None:
       g = _DecodeGraph(self, Bb, Wb)

@@ -71,8 +71,10 @@ def test_engine_generates_the_same_with_and_without_graphs(tmp_path):
   for eager in (True, False):
     with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, num_pages=64, max_num_seqs=4,
                    enforce_eager=eager) as eng:
+      captured = eng.warm_up()            # every batch bucket up to max_num_seqs, every table width of the model
+      assert (captured == 0) if eager else (captured >= 3 and all(g.ok for g in eng.runner._graphs.values()))
       res.append([o["token_ids"] for o in eng.generate(prompts, sps, use_tqdm=False)])
-      assert bool(eng.runner._graphs) == (not eager)
+      assert len(eng.runner._graphs) == captured, "a step needed a graph that warm_up had not made"
   assert res[0] == res[1]
 
 
