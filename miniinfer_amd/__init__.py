@@ -11,7 +11,7 @@ from .sampling import SamplingParams
 
 def __getattr__(name):
   # the engine pulls in the kernels; keep `import miniinfer_amd` light
-  if name == "LLMEngine":
-    from .engine import LLMEngine
-    return LLMEngine
+  if name in ("LLMEngine", "RequestOutput"):
+    from .engine import llm_engine
+    return getattr(llm_engine, name)
   raise AttributeError(name)

@@ -42,6 +42,18 @@ class StepOutput:
   num_preempted: int = 0
 
 
+@dataclass
+class RequestOutput:
+  """One new token of one request, as `stream_generate` yields it (miniinfer/engine/llm_engine.py:49-59)."""
+  request_id: str
+  delta_text: str
+  full_text: str
+  token_id: int
+  output_token_ids: List[int]
+  finished: bool
+  finish_reason: Optional[str]
+
+
 class LLMEngine:
   def __init__(self, model: str, model_config=None, random_weights_seed: Optional[int] = None, **kwargs):
     """model: a folder with config.json and *.safetensors.  With `model_config` (a typed configuration)
@@ -247,3 +259,38 @@ class LLMEngine:
       text = self.tokenizer.decode(r.outputs) if self.tokenizer is not None else ""
       results.append({"text": text, "token_ids": list(r.outputs), "request_id": rid, "finish_reason": r.finish_reason})
     return results
+
+  def stream_generate(self, prompts, sampling_params: Union[SamplingParams, Sequence[SamplingParams], None] = None):
+    """The same requests, yielded token by token as they are booked: a `RequestOutput` for every new token of
+    every request, the last one of a request with `finished` set (miniinfer/engine/llm_engine.py:1341-1400).
+    Tokens of one request come in order; requests interleave as the steps produce them."""
+    if isinstance(prompts, str) or (len(prompts) > 0 and isinstance(prompts[0], int)):
+      prompts = [prompts]
+    if sampling_params is None:
+      sampling_params = SamplingParams()
+    if isinstance(sampling_params, SamplingParams):
+      sampling_params = [sampling_params] * len(prompts)
+    if len(sampling_params) != len(prompts):
+      raise ValueError("one SamplingParams for all prompts, or one per prompt")
+    rids = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+    live = {rid: self._requests[rid] for rid in rids}
+    sent = {rid: 0 for rid in rids}
+    texts = {rid: "" for rid in rids}
+    while live:
+      if not self.is_finished():
+        self.step()
+      for rid in list(live):
+        r = live[rid]
+        ready = len(r.outputs) - r.pending           # placeholders of tokens still on the device sit at the end
+        done = r.finished and r.pending == 0
+        for i in range(sent[rid], ready):
+          full = self.tokenizer.decode(r.outputs[:i + 1]) if self.tokenizer is not None else ""
+          last = done and i == ready - 1
+          yield RequestOutput(request_id=rid, delta_text=full[len(texts[rid]):], full_text=full, token_id=r.outputs[i],
+                              output_token_ids=list(r.outputs[:i + 1]), finished=last,
+                              finish_reason=r.finish_reason if last else None)
+          texts[rid] = full
+        sent[rid] = ready
+        if done:
+          del live[rid]
+          self._requests.pop(rid, None)

@@ -157,3 +157,25 @@ def test_launching_ahead_of_the_tokens_changes_no_token(tmp_path, dtype):
   assert results[True] == results[False]
   assert results[True][2][1] == "eos" and len(results[True][2][0]) <= 4
   assert all(t >= 0 for toks, _ in results[True] for t in toks)
+
+
+def test_stream_generate_yields_every_token_once_and_in_order(tmp_path):
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "A")
+  prompts = [tm.random_tokens(cfg, n, seed=70 + n) for n in (5, 23, 11)]
+  sps = [SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=True),
+         SamplingParams(temperature=0.8, max_tokens=14, ignore_eos=True, seed=2),
+         SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)]
+  for overlap in (True, False):
+    with LLMEngine(model=str(tmp_path / "m"), dtype="float32", num_pages=32, max_num_seqs=4, enable_overlap=overlap) as eng:
+      whole = eng.generate(prompts, sps, use_tqdm=False)
+      seen, ended = {}, {}
+      for out in eng.stream_generate(prompts, sps):
+        toks = seen.setdefault(out.request_id, [])
+        toks.append(out.token_id)
+        assert out.output_token_ids == toks and out.request_id not in ended
+        if out.finished:
+          ended[out.request_id] = out.finish_reason
+      assert [seen[r] for r in sorted(seen, key=lambda r: int(r.split("-")[1]))] == [o["token_ids"] for o in whole]
+      assert list(ended.values()) == ["max_tokens"] * 3 and eng.is_finished()
+      assert eng.cache.num_free_pages() == eng.cache.num_pages
