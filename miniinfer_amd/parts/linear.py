@@ -80,7 +80,9 @@ def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]
 
 
 def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-  """x: a tensor [M, K], or a DeferredNorm (the add and the norm are then fused into the product if possible)."""
+  """x: a tensor [M, K], a pending product, or a DeferredNorm (the add and the norm are then fused into the product
+  if possible)."""
+  x = as_tensor(x)
   if hasattr(x, "materialize"):
     if out_dtype in (None, torch.bfloat16):
       y = _fuse_norm(x, weight, gate_up=False)
@@ -110,6 +112,7 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
 def gate_up_activation(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
   """silu(x Wg^T) * (x Wu^T) for a fused gate|up matrix [2 I, K]: one kernel for few rows (the activation is made
   from the 32-bit sums in the product's epilogue), product and activation kernels otherwise."""
+  x = as_tensor(x)
   if hasattr(x, "materialize"):
     y = _fuse_norm(x, gate_up_weight, gate_up=True)
     if y is not None:
