@@ -45,13 +45,17 @@ template <int MB, int RB, bool OUT_F32, bool GATE_UP>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __restrict__ A, int64_t lda,
                                                            const uint16_t* __restrict__ W, int64_t ldw,
                                                            void* __restrict__ C, int64_t ldc, int M, int N, int K,
-                                                           NormHalves nh) {
+                                                           int rpg, NormHalves nh) {
   extern __shared__ float red[];   // [(waves + 1) / 2][RB * MB][256], then (norm halves) [OB * 256] squares, [waves][64] sums
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   // GATE_UP: RB == 2, row block 0 = gate rows n0.., row block 1 = up rows N + n0..; N counts output columns
-  const int n0 = GATE_UP ? blockIdx.x * 16 : blockIdx.x * 16 * RB;
+  // rpg: rows of W per workgroup when RB == 1 (16, or fewer so that a matrix of few rows still gives every compute
+  // unit a workgroup: the lanes of the other rows then load nothing and their results are dropped)
+  const int n0 = GATE_UP ? blockIdx.x * 16 : (RB == 1 ? blockIdx.x * rpg : blockIdx.x * 16 * RB);
+  const int n_end = min(N, n0 + (GATE_UP ? 16 : (RB == 1 ? rpg : 16 * RB)));
+  const bool w_live = GATE_UP || RB > 1 || (lane & 15) < rpg;
   const int steps = (K + 31) / 32;
   const int spw = (steps + nw - 1) / nw;
   const int s_begin = wave * spw;
@@ -97,7 +101,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       const int blk = e >> 8, ln = (e & 255) >> 2, i = e & 3;
       const int n = n0 + 16 * (blk / MB) + 4 * (ln >> 4) + i;
       const int m = 16 * (blk % MB) + (ln & 15);
-      if (e < OBLK * 256 && n < N && m < M) {
+      if (e < OBLK * 256 && n < n_end && m < M) {
         r_pre[j] = nh.residual[(int64_t)m * N + n];
         w_pre[j] = nh.norm_weight[n];
       }
@@ -115,7 +119,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       const int k = 32 * (s0 + c) + 8 * (lane >> 4);
       const bool kok = (s0 + c < s_end) && k < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) w[c][rb] = kok ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
+      for (int rb = 0; rb < RB; ++rb)
+        w[c][rb] = (kok && w_live) ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const bool ok = kok && mok[mb];
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       u *= rstd;
     }
     if (GATE_UP) v = silu_f(v) * u;
-    const bool live = n < N && m < M;
+    const bool live = n < n_end && m < M;
     if (nh.residual) {
       float rv = 0.f;
       if (live) {
@@ -369,15 +374,34 @@ static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up) {
   return ((size_t)((waves + 1) / 2) * RB * MB * 256 + (size_t)OB * 256 + (size_t)waves * 64) * sizeof(float);
 }
 
+// Rows of W per workgroup and workgroups of the launch.  A matrix of few rows is cut finer than the 16 rows of a
+// matrix-core tile when the left operand has at most 16 rows (with more, the operand's re-reads per workgroup
+// would outweigh what the extra workgroups gain).
+struct SkinnyGrid {
+  int RB, rpg, groups;
+};
+
+static SkinnyGrid skinny_grid(bool gate_up, int N, int M) {
+  const int row_blocks = (N + 15) / 16;
+  SkinnyGrid g;
+  g.RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
+  g.rpg = 16;
+  if (!gate_up && g.RB == 1 && M <= 16)
+    while (g.rpg > 4 && (N + g.rpg - 1) / g.rpg < 256) g.rpg /= 2;
+  g.groups = gate_up ? row_blocks : (g.RB == 1 ? (N + g.rpg - 1) / g.rpg : (row_blocks + g.RB - 1) / g.RB);
+  return g;
+}
+
 template <int MB, int RB>
 static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
-                  int64_t ldc, int M, int N, int K, int waves, const NormHalves& nh, hipStream_t stream) {
-  const dim3 grid(gate_up ? (N + 15) / 16 : (N + 16 * RB - 1) / (16 * RB));
+                  int64_t ldc, int M, int N, int K, int waves, const SkinnyGrid& sg, const NormHalves& nh,
+                  hipStream_t stream) {
+  const dim3 grid(sg.groups);
   const dim3 block(64 * waves);
   const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up);
 #define GO(F32, GU)                                                                                              \
   gemm_skinny_kernel<MB, RB, F32, GU><<<grid, block, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, \
-                                                                    ldw, C, ldc, M, N, K, nh)
+                                                                    ldw, C, ldc, M, N, K, sg.rpg, nh)
   if (gate_up) {
     if constexpr (RB == 2) {
       if (out_f32) GO(true, true);
@@ -391,12 +415,8 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
   return 0;
 }
 
-// Workgroups of the launch for an [N, K] matrix (the number of rows of 64 that `ss_out` must hold).
-MI_EXPORT int mi_gemm_skinny_groups(int gate_up, int N) {
-  const int row_blocks = (N + 15) / 16;
-  const int RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
-  return gate_up ? row_blocks : (row_blocks + RB - 1) / RB;
-}
+// Workgroups of the launch for M rows and an [N, K] matrix (the number of rows of 64 that `ss_out` must hold).
+MI_EXPORT int mi_gemm_skinny_groups(int gate_up, int N, int M) { return skinny_grid(gate_up != 0, N, M).groups; }
 
 // A [M, K], C [M, N] bfloat16 or float32; W [N, K], or with gate_up the fused matrix [2 N, K].
 // Norm halves (see NormHalves; all optional): row_ss [ss_parts][64] and eps scale the rows of the result;
@@ -415,9 +435,8 @@ MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t
              "gemm_skinny: the residual form needs norm_weight, a_out and ss_out, and no gate|up");
   MI_REQUIRE(!row_ss || ss_parts > 0, "gemm_skinny: row_ss without parts");
   if (M == 0) return 0;
-  const int row_blocks = (N + 15) / 16;
-  const int RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
-  const int groups = gate_up ? row_blocks : (row_blocks + RB - 1) / RB;
+  const SkinnyGrid sg = skinny_grid(gate_up != 0, N, M);
+  const int RB = sg.RB, groups = sg.groups;
   const int steps = (K + 31) / 32;
   // enough waves to fill the chip, at least 2 steps of K per wave, at most 16 waves per workgroup
   int waves = (4096 + groups - 1) / groups;
@@ -429,7 +448,7 @@ MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t
   const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \
-    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, nh, stream);          \
+    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, stream);          \
     MI_CHECK_LAUNCH("gemm_skinny");                                                                           \
     return 0;                                                                                                 \
   }

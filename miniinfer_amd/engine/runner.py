@@ -21,6 +21,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, LayerCache
+from ..kernels import ops
 from ..parts import DecoderModel
 
 
@@ -194,7 +195,7 @@ class _DecodeGraph:
 
 
 _GRAPH_BATCHES = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
-_LIBRARY_FREE_ROWS = 64       # up to here every product of a decode step is one of this library's kernels
+_LIBRARY_FREE_ROWS = ops.SKINNY_OWN_ROWS     # up to here every product of a decode step is one of this library's kernels
 
 
 class ModelRunner:

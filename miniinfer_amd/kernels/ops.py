@@ -108,7 +108,7 @@ _SIGS["gemm_skinny"] = {
 _SIGS["gemm_skinny"]["mi_gemm_skinny_ex"] = [c_int, c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int,
                                              c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p,
                                              c_void_p, c_void_p]
-_SIGS["gemm_skinny"]["mi_gemm_skinny_groups"] = [c_int, c_int]
+_SIGS["gemm_skinny"]["mi_gemm_skinny_groups"] = [c_int, c_int, c_int]
 _SIGS["gemm_skinny"]["mi_norm_gemm_skinny"] = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                                c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]
 
@@ -281,6 +281,16 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor
 
 
 SKINNY_MAX_ROWS = 64
+SKINNY_OWN_ROWS = 16                 # up to here the weight-streaming kernel is the quicker one for every matrix
+SKINNY_OWN_ELEMENTS = 8 << 20        # and for more rows (up to SKINNY_MAX_ROWS) while the matrix is smaller than this
+
+
+def skinny_preferred(num_rows: int, n: int, k: int) -> bool:
+  """Whether a product of `num_rows` rows with an [n, k] matrix goes to `gemm_skinny` rather than to the library.
+  Each wave of that kernel reads the left operand's rows for its own slice of k again, so beyond 16 rows its
+  loads are mostly left operand; on matrices of tens of MB the library's kernels (which split k across workgroups)
+  then stream the weights about twice as fast, which outweighs the norm and activation kernels that fusing saved."""
+  return num_rows <= SKINNY_OWN_ROWS or (num_rows <= SKINNY_MAX_ROWS and n * k < SKINNY_OWN_ELEMENTS)
 
 
 def gemm_skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -357,7 +367,7 @@ def gemm_skinny_into_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tens
   M = a.shape[0]
   N, K = w.shape
   lib = _lib("gemm_skinny")
-  parts = lib.mi_gemm_skinny_groups(0, N)
+  parts = lib.mi_gemm_skinny_groups(0, N, M)
   operand = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
   row_ss = torch.empty((parts, 64), dtype=torch.float32, device=a.device)
   _check(lib, lib.mi_gemm_skinny_ex(0, 0, _ptr(a), a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), None,

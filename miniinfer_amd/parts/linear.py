@@ -55,12 +55,15 @@ def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]
   M = d.residual.shape[0]
   if d.consumed or d.dtype != torch.bfloat16:
     return None
+  if not ops.skinny_preferred(M, weight.shape[0], weight.shape[1]):
+    return None
   N = weight.shape[0] // 2 if gate_up else weight.shape[0]
   if isinstance(d.x, PendingLinear) and d.x.value is None:
     # The branch's last product is still pending: its kernel adds to the residual stream in place and leaves
     # bfloat16(residual * norm weight) and partial sums of squares; this product's kernel scales its rows by them.
     p = d.x
-    if ops.gemm_skinny_into_norm_supported(p.a, p.weight, d.residual, d.norm.weight) \
+    if ops.skinny_preferred(M, p.weight.shape[0], p.weight.shape[1]) \
+        and ops.gemm_skinny_into_norm_supported(p.a, p.weight, d.residual, d.norm.weight) \
         and weight.dtype == torch.bfloat16 and weight.shape[1] == d.residual.shape[1] and weight.stride(1) == 1 \
         and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0:
       operand, row_ss = ops.gemm_skinny_into_norm(p.a, p.weight, d.residual, d.norm.weight)
@@ -93,7 +96,7 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
   M, N = x.shape[0], weight.shape[0]
   if not x.is_cuda:
     raise ops.KernelError("miniinfer_amd runs on the GPU only")
-  if ops.gemm_skinny_supported(x, weight):
+  if ops.gemm_skinny_supported(x, weight) and (out_dtype == torch.float32 or ops.skinny_preferred(M, N, x.shape[1])):
     # few rows (decode): the time is the time to stream the weights; this library's MFMA kernel
     return ops.gemm_skinny(x, weight, torch.empty((M, N), dtype=out_dtype, device=x.device))
   if out_dtype == torch.float32 and M > ops.SKINNY_MAX_ROWS and ops.gemm_skinny_supported(x[:1], weight):
@@ -119,7 +122,7 @@ def gate_up_activation(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.T
       return y
     x = x.materialize()
   M, inter = x.shape[0], gate_up_weight.shape[0] // 2
-  if ops.gemm_skinny_supported(x, gate_up_weight):
+  if ops.gemm_skinny_supported(x, gate_up_weight) and ops.skinny_preferred(M, 2 * inter, x.shape[1]):
     return ops.gemm_skinny(x, gate_up_weight, torch.empty((M, inter), dtype=x.dtype, device=x.device), gate_up=True)
   gu = linear(x, gate_up_weight)
   act = torch.empty((M, inter), dtype=x.dtype, device=x.device)

@@ -319,7 +319,8 @@ def test_mfma_attention_finds_a_far_key_and_respects_the_window_edge():
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (8, 4096, 1024), (16, 1024, 3072), (17, 500, 80), (64, 6144, 1024),
-                                   (3, 151936, 256), (33, 48, 2048), (5, 130, 88), (64, 1000, 40)])
+                                   (3, 151936, 256), (33, 48, 2048), (5, 130, 88), (64, 1000, 40), (7, 2050, 64),
+                                   (16, 1001, 512)])
 def test_gemm_skinny(M, N, K, out_dtype):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(9)
@@ -446,7 +447,8 @@ def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, win
 
 
 @pytest.mark.parametrize("M,N,K,N2,gate_up", [(8, 1024, 2048, 6144, True), (1, 80, 96, 112, False), (16, 1024, 3072, 4096, False),
-                                               (40, 136, 264, 200, True), (64, 1024, 2048, 3072, False), (5, 88, 40, 24, False)])
+                                               (40, 136, 264, 200, True), (64, 1024, 2048, 3072, False), (5, 88, 40, 24, False),
+                                               (12, 2056, 96, 160, True)])
 def test_norm_split_between_two_products(M, N, K, N2, gate_up):
   """residual += a W1^T; y = rmsnorm(residual) * w; out = y W2^T (or the gated activation of it), the add and the
   norm done half in the first product's kernel and half in the second's.  Against 64-bit arithmetic with the

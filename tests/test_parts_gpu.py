@@ -119,9 +119,16 @@ def test_gated_mlp_alone(dtype):
                             plain.swiglu(x.float(), wg.float(), wu.float(), wd.float()), atol=1e-3)
 
 
+@pytest.mark.parametrize("library_products", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_block_alone(dtype):
-  """One block on a residual stream: r += attn(norm(r)); r += mlp(norm(r)) with the adds deferred into the norms."""
+def test_block_alone(dtype, library_products, monkeypatch):
+  """One block on a residual stream: r += attn(norm(r)); r += mlp(norm(r)) with the adds deferred into the norms.
+  With `library_products`, products of more than 16 rows go the way they go for large matrices: to the library,
+  with norm and activation kernels of their own."""
+  from miniinfer_amd.kernels import ops
+  if library_products:
+    monkeypatch.setattr(ops, "SKINNY_OWN_ELEMENTS", 0)
+    assert ops.skinny_preferred(16, 64, 64) and not ops.skinny_preferred(17, 64, 64)
   from miniinfer_amd.cache import CacheManager
   from miniinfer_amd.config import Qwen3Config, model_spec_of
   from miniinfer_amd.engine.runner import StepEntry
