@@ -28,17 +28,19 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.f + expf(-g)); 
 // Two optional halves of an RMS norm that sits between two products, so that the norm needs no kernel of its own.
 // After the first product (`residual` set): instead of C, the workgroup adds its result to the 32-bit residual
 // stream in place, r[m][n] += result, writes the next product's left operand a_out[m][n] = bf16(r[m][n] * w[n]),
-// and the sum of r[m][n]^2 over its own columns n to ss_out[blockIdx.x][m] (rows of 64).
+// and the sum of r[m][n]^2 over its own columns n to ss_out[blockIdx.x][m] (rows of SS_ROW(M) entries: 16 when
+// there are at most 16 rows, so that many small workgroups do not leave the next kernel a long table to read).
 // Before the second product's result is stored (`row_ss` set): row m is scaled by rsqrt(sum_p row_ss[p][m] / K +
 // eps), the norm's missing factor (K, the length of the normed rows, is this product's K).
+#define SS_ROW(rows) ((rows) <= 16 ? 16 : 64)
 struct NormHalves {
-  const float* row_ss;      // [ss_parts][64]
+  const float* row_ss;      // [ss_parts][SS_ROW(M)]
   int ss_parts;
   float eps;
   float* residual;          // [M, N] float32, leading dimension N
   const float* norm_weight; // [N]
   uint16_t* a_out;          // [M, N] bfloat16, leading dimension N
-  float* ss_out;            // [gridDim.x][64]
+  float* ss_out;            // [gridDim.x][SS_ROW(M)]
 };
 
 template <int MB, int RB, bool OUT_F32, bool GATE_UP>
@@ -85,13 +87,14 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   }
 
   // What the norm halves read is asked for before the weights, so that the end of the kernel does not wait for
-  // memory again: the partial sums of squares of row (thread % 64), parts (thread / 64), + waves, ...; and the
-  // residual and norm weight of the first two result elements this thread will finish.
+  // memory again: the partial sums of squares of row (thread % SS), parts (thread / SS), + threads / SS, ...; and
+  // the residual and norm weight of the first two result elements this thread will finish.
   constexpr int OBLK = GATE_UP ? MB : RB * MB;
+  constexpr int SS = SS_ROW(16 * MB);
   float my_ss = 0.f;
   if (nh.row_ss) {
-    const int m = threadIdx.x & 63;
-    for (int p = wave; p < nh.ss_parts; p += nw) my_ss += nh.row_ss[(int64_t)p * 64 + m];
+    const int m = threadIdx.x % SS;
+    for (int p = threadIdx.x / SS; p < nh.ss_parts; p += blockDim.x / SS) my_ss += nh.row_ss[(int64_t)p * SS + m];
   }
   float r_pre[2] = {0.f, 0.f}, w_pre[2] = {0.f, 0.f};
   if (nh.residual) {
@@ -151,7 +154,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   constexpr int OB = GATE_UP ? MB : RB * MB;          // output blocks of the workgroup
   const int hw = (nw + 1) / 2;                        // waves whose sums stay in LDS
   float* sq = red + hw * RB * MB * 256;               // [OB * 256] squares of the new residual (norm halves only)
-  float* ss_part = sq + OB * 256;                     // [waves][64]
+  float* ss_part = sq + OB * 256;                     // [waves][64]: each wave's sums by row
   if (wave >= hw) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
@@ -159,7 +162,13 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       for (int mb = 0; mb < MB; ++mb)
         *reinterpret_cast<f32x4*>(red + (((wave - hw) * RB * MB + rb * MB + mb) * 64 + lane) * 4) = acc[rb][mb];
   }
-  if (nh.row_ss) ss_part[wave * 64 + lane] = my_ss;
+  if (nh.row_ss) {
+    if (SS == 16) {                                   // lanes l, l + 16, l + 32, l + 48 hold sums of the same row
+      my_ss += __shfl_xor(my_ss, 16, 64);
+      my_ss += __shfl_xor(my_ss, 32, 64);
+    }
+    ss_part[wave * 64 + lane] = my_ss;
+  }
   __syncthreads();
   if (wave < hw) {
     const bool partner = wave + hw < nw;
@@ -216,7 +225,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       for (int rb = 0; rb < (GATE_UP ? 1 : RB); ++rb)
         for (int q = 0; q < 4; ++q)
           for (int i = 0; i < 4; ++i) total += sq[(rb * MB + (m >> 4)) * 256 + 4 * ((m & 15) + 16 * q) + i];
-      nh.ss_out[(int64_t)blockIdx.x * 64 + m] = total;
+      nh.ss_out[(int64_t)blockIdx.x * SS + m] = total;
     }
   }
 }
@@ -415,12 +424,13 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
   return 0;
 }
 
-// Workgroups of the launch for M rows and an [N, K] matrix (the number of rows of 64 that `ss_out` must hold).
+// Workgroups of the launch for M rows and an [N, K] matrix: `ss_out` holds that many rows of mi_gemm_skinny_ss_row(M).
 MI_EXPORT int mi_gemm_skinny_groups(int gate_up, int N, int M) { return skinny_grid(gate_up != 0, N, M).groups; }
+MI_EXPORT int mi_gemm_skinny_ss_row(int M) { return SS_ROW(M); }
 
 // A [M, K], C [M, N] bfloat16 or float32; W [N, K], or with gate_up the fused matrix [2 N, K].
-// Norm halves (see NormHalves; all optional): row_ss [ss_parts][64] and eps scale the rows of the result;
-// residual [M, N] float32 + norm_weight [N] + a_out [M, N] bfloat16 + ss_out [groups][64] replace C.
+// Norm halves (see NormHalves; all optional): row_ss [ss_parts][ss_row(M)] and eps scale the rows of the result;
+// residual [M, N] float32 + norm_weight [N] + a_out [M, N] bfloat16 + ss_out [groups][ss_row(M)] replace C.
 MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw,
                                 void* C, int64_t ldc, int M, int N, int K, const float* row_ss, int ss_parts,
                                 float eps, float* residual, const float* norm_weight, void* a_out, float* ss_out,

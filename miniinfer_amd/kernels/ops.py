@@ -109,6 +109,7 @@ _SIGS["gemm_skinny"]["mi_gemm_skinny_ex"] = [c_int, c_int, c_void_p, c_int64, c_
                                              c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p,
                                              c_void_p, c_void_p]
 _SIGS["gemm_skinny"]["mi_gemm_skinny_groups"] = [c_int, c_int, c_int]
+_SIGS["gemm_skinny"]["mi_gemm_skinny_ss_row"] = [c_int]
 _SIGS["gemm_skinny"]["mi_norm_gemm_skinny"] = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                                c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]
 
@@ -327,7 +328,7 @@ def gemm_skinny_scaled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_
                        gate_up: bool = False) -> torch.Tensor:
   """`gemm_skinny` whose rows are scaled by rsqrt(sum_p row_ss[p, m] / K + eps) before they are stored (and, with
   `gate_up`, before the activation): the second half of an RMS norm whose first half `gemm_skinny_into_norm` did.
-  row_ss float32 [parts, 64]."""
+  row_ss float32 [parts, 16] for up to 16 rows, [parts, 64] for more."""
   _dev(a, w, out, row_ss)
   if not gemm_skinny_supported(a, w):
     raise KernelError(f"gemm_skinny does not take a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}")
@@ -339,9 +340,10 @@ def gemm_skinny_scaled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_
     N //= 2
   if tuple(out.shape) != (M, N) or out.stride(1) != 1 or out.dtype not in (torch.bfloat16, torch.float32):
     raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit [{M}, {N}]")
-  if row_ss.dtype != torch.float32 or row_ss.dim() != 2 or row_ss.shape[1] != 64 or not row_ss.is_contiguous():
-    raise KernelError("gemm_skinny_scaled: row_ss must be a contiguous float32 [parts, 64]")
   lib = _lib("gemm_skinny")
+  ss_row = lib.mi_gemm_skinny_ss_row(M)
+  if row_ss.dtype != torch.float32 or row_ss.dim() != 2 or row_ss.shape[1] != ss_row or not row_ss.is_contiguous():
+    raise KernelError(f"gemm_skinny_scaled: row_ss must be a contiguous float32 [parts, {ss_row}] for {M} rows")
   _check(lib, lib.mi_gemm_skinny_ex(1 if out.dtype == torch.float32 else 0, 1 if gate_up else 0, _ptr(a),
                                     a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), _ptr(out),
                                     out.stride(0) if M > 1 else N, M, N, K, _ptr(row_ss), row_ss.shape[0], float(eps),
@@ -359,7 +361,7 @@ def gemm_skinny_into_norm_supported(a: torch.Tensor, w: torch.Tensor, residual: 
 
 def gemm_skinny_into_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor):
   """residual += a @ w^T (in place, 32-bit), and the first half of the RMS norm of the new residual: returns
-  (operand, row_ss) with operand[m, n] = bfloat16(residual[m, n] * norm_weight[n]) and row_ss float32 [parts, 64],
+  (operand, row_ss) with operand[m, n] = bfloat16(residual[m, n] * norm_weight[n]) and row_ss float32 [parts, 16 or 64],
   the sum of squares of row m over each workgroup's columns.  `gemm_skinny_scaled` finishes the norm."""
   _dev(a, w, residual, norm_weight)
   if not gemm_skinny_into_norm_supported(a, w, residual, norm_weight):
@@ -369,7 +371,7 @@ def gemm_skinny_into_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tens
   lib = _lib("gemm_skinny")
   parts = lib.mi_gemm_skinny_groups(0, N, M)
   operand = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
-  row_ss = torch.empty((parts, 64), dtype=torch.float32, device=a.device)
+  row_ss = torch.empty((parts, lib.mi_gemm_skinny_ss_row(M)), dtype=torch.float32, device=a.device)
   _check(lib, lib.mi_gemm_skinny_ex(0, 0, _ptr(a), a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), None,
                                     N, M, N, K, None, 0, 0.0, _ptr(residual), _ptr(norm_weight), _ptr(operand),
                                     _ptr(row_ss), _stream()))
