@@ -105,6 +105,7 @@ def main() -> int:
   ap.add_argument("--layers", type=int, default=None, help="fewer layers than the preset (named in the record)")
   ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
   ap.add_argument("--eager", action="store_true")
+  ap.add_argument("--no-tune", action="store_true", help="choose product kernels by rule instead of timing them at start")
   ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
   ap.add_argument("--only-prefill", action="store_true", help="run only the 2,048-token prefill (for profiling)")
   args = ap.parse_args()
@@ -126,7 +127,7 @@ def main() -> int:
   pages = max_batch * (-(-room // page_size)) + 16
   engine = LLMEngine(model="", model_config=cfg, random_weights_seed=0, dtype=args.dtype, page_size=page_size,
                      num_pages=pages, max_num_seqs=max_batch, max_model_len=max_len, max_num_batched_tokens=8192,
-                     enforce_eager=args.eager)
+                     enforce_eager=args.eager, tune_products=not args.no_tune)
   esize = 2 if args.dtype == "bfloat16" else 4
   if args.only_prefill:
     psec = time_prefill(engine, 2048, reps=max(1, args.steps), seed=2)

@@ -25,6 +25,7 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..config import EngineConfig, load_model_config, model_spec_of
+from ..kernels.tuning import tune_products
 from ..sampling import Sampler, SamplingParams, request_seed
 from ..weights import build_model, fill_random, load_weights
 from .runner import ModelRunner, StepEntry
@@ -72,6 +73,8 @@ class LLMEngine:
       fill_random(self.model, random_weights_seed)
     else:
       load_weights(self.model, cfg.model_path)
+    if cfg.tune_products and self.dtype == torch.bfloat16:
+      tune_products(self.model.products())
     spec = self.model.spec
     self.max_model_len = min(cfg.max_model_len or spec.max_positions, spec.max_positions)
     needs = self.model.cache_needs()

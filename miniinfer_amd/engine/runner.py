@@ -146,21 +146,22 @@ class _DecodeGraph:
     ctx.future_tokens = runner.future_tokens
     self.ctx = ctx
     # every entry is padding while warming up and capturing: it reads and writes the scratch page only
-    side = torch.cuda.Stream(device=runner.device)
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-      runner.model.forward(ctx)
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    self.graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(self.graph):
-      self.logits = runner.model.forward(ctx)
+    before = ops.library_products_run()
+    self.graph, self.logits = self._capture(runner, ctx)
     self.ok = True
-    if B > _LIBRARY_FREE_ROWS:
-      # Beyond the rows this library's own product kernels take, the captured step holds library products.  What a
-      # library records into a graph is its own affair (clears of a workspace have replayed wrongly): the graph is
-      # replayed a few times, with eager work in between, against the eager result of the same (padding) inputs,
-      # and a graph that does not reproduce it is not used.
+    library = ops.library_products_run() != before
+    if library and B <= ops.SKINNY_MAX_ROWS:
+      # The step sends some products of few rows to the library (by measurement of each product alone, or by
+      # rule).  Inside a step that can still lose to this library's own kernels, which need no norm and activation
+      # kernels beside them: the step is captured both ways and the quicker graph is kept.
+      with ops.own_products_only():
+        own_graph, own_logits = self._capture(runner, ctx)
+      if self._replay_ms(own_graph) <= self._replay_ms(self.graph):
+        self.graph, self.logits, library = own_graph, own_logits, False
+    if library and runner.check_graphs:
+      # What a library records into a graph is its own affair (clears of a workspace have replayed wrongly): the
+      # graph is replayed a few times, with eager work in between, against the eager result of the same (padding)
+      # inputs, and a graph that does not reproduce it is not used.
       want = runner.model.forward(ctx).clone()
       for _ in range(3):
         self.graph.replay()
@@ -170,6 +171,33 @@ class _DecodeGraph:
           self.ok = False
           break
         want = runner.model.forward(ctx).clone()
+
+  @staticmethod
+  def _capture(runner: "ModelRunner", ctx):
+    side = ops.side_stream(runner.device)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+      runner.model.forward(ctx)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      logits = runner.model.forward(ctx)
+    return graph, logits
+
+  @staticmethod
+  def _replay_ms(graph) -> float:
+    graph.replay()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = float("inf")
+    for _ in range(3):
+      start.record()
+      graph.replay()
+      end.record()
+      torch.cuda.synchronize()
+      best = min(best, start.elapsed_time(end))
+    return best
 
   def fill_padding(self, first: int) -> None:
     """Entries first.. are padding: token 0 at position 0 of a request of one key in the scratch page."""
@@ -195,7 +223,6 @@ class _DecodeGraph:
 
 
 _GRAPH_BATCHES = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
-_LIBRARY_FREE_ROWS = ops.SKINNY_OWN_ROWS     # up to here every product of a decode step is one of this library's kernels
 
 
 class ModelRunner:
@@ -207,6 +234,7 @@ class ModelRunner:
     self.device = model.ctx.device
     self.vocab_size = model.spec.vocab_size
     self.use_graphs = use_graphs and self.device.type == "cuda"
+    self.check_graphs = True      # replay every captured step against its eager result before it is used
     self._staging: Optional[torch.Tensor] = None
     self._allow_future = False
     self._graphs: Dict[tuple, _DecodeGraph] = {}

@@ -2,10 +2,13 @@
 
     python -m miniinfer_amd.kernels.microbench product --rows 8 --n 25600 --k 5120 --gate-up
     python -m miniinfer_amd.kernels.microbench prefill-attention --tokens 2048 --heads 16 --kv-heads 8 --head-dim 128
+    python -m miniinfer_amd.kernels.microbench decode-attention --batch 8 --context 2048 --heads 16 --kv-heads 8
 
 `product` times the weight-streaming product (`ops.gemm_skinny`) beside the library's product for the same operands;
 the weights cycle through several copies so that they stream from memory, not from a cache.  `prefill-attention`
-times `ops.attn_prefill` for one prompt in both of its variants.  Both print one line per measurement; under
+times `ops.attn_prefill` for one prompt in both of its variants; `decode-attention` times the split-key decode
+kernel and its merge for a batch of requests, with and without the fused norm, rotation and cache write, over
+several caches in turn.  All print one line per measurement; under
 `rocprofv3 --pmc ...` the same commands give the kernels' counters.
 """
 
@@ -17,32 +20,9 @@ import sys
 import torch
 
 from . import ops
+from .tuning import graph_time_us
 
 DEV = "cuda:0"
-
-
-def graph_time_us(fn, calls: int) -> float:
-  """Microseconds per call of `fn`, from one replay of a graph that holds `calls` calls."""
-  fn()
-  torch.cuda.synchronize()
-  side = torch.cuda.Stream()
-  side.wait_stream(torch.cuda.current_stream())
-  with torch.cuda.stream(side):
-    fn()
-  torch.cuda.current_stream().wait_stream(side)
-  torch.cuda.synchronize()
-  g = torch.cuda.CUDAGraph()
-  with torch.cuda.graph(g):
-    for _ in range(calls):
-      fn()
-  g.replay()
-  torch.cuda.synchronize()
-  start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-  start.record()
-  g.replay()
-  end.record()
-  torch.cuda.synchronize()
-  return start.elapsed_time(end) / calls * 1e3
 
 
 def cmd_product(args) -> int:
@@ -95,6 +75,54 @@ def cmd_prefill_attention(args) -> int:
   return 0
 
 
+def cmd_decode_attention(args) -> int:
+  from ..parts.attention import decode_splits
+  nq, nkv, d, P, B, L = args.heads, args.kv_heads, args.head_dim, args.page_size, args.batch, args.context
+  if not ops.mfma_attention_supported(torch.bfloat16, nq, nkv, d, P):
+    print("these sizes go to the plain attention kernel, which this command does not time", file=sys.stderr)
+    return 2
+  per_req = -(-L // P)
+  pages = B * per_req
+  cache_bytes = 2 * pages * nkv * P * d * 2
+  copies = max(2, min(8, (1536 << 20) // cache_bytes))
+  g = torch.Generator(device=DEV).manual_seed(0)
+  caches = [(torch.randn(pages + 1, nkv, P, d, device=DEV, generator=g).bfloat16(),
+             torch.randn(pages + 1, nkv, d, P, device=DEV, generator=g).bfloat16()) for _ in range(copies)]
+  table = (torch.randperm(pages, device=DEV, generator=g) + 1).to(torch.int32).view(B, per_req)
+  qkv = torch.randn(B, (nq + 2 * nkv) * d, device=DEV, generator=g).bfloat16()
+  cu = torch.arange(B + 1, dtype=torch.int32, device=DEV)
+  kv = torch.full((B,), L, dtype=torch.int32, device=DEV)
+  positions = torch.full((B,), L - 1, dtype=torch.int32, device=DEV)
+  slots = (table[:, (L - 1) // P].to(torch.int64) * P + (L - 1) % P).to(torch.int32)
+  weight = torch.ones(d, device=DEV)
+  angles = torch.rand(L, d // 2, device=DEV, generator=g)
+  cos_sin = torch.cat([angles.cos(), angles.sin()], dim=1).contiguous()
+  out = torch.empty(B, nq * d, dtype=torch.bfloat16, device=DEV)
+  tile_keys, waves = ops.attn_decode_geometry(d)
+  splits = args.splits or decode_splits(B * nkv, L, tile_keys, waves)
+  part_o = torch.empty(B * nq * splits * d, device=DEV)
+  part_ml = torch.empty(B * nq * splits * 2, device=DEV)
+  turn = [0]
+
+  def plain():
+    k, v = caches[turn[0] % copies]
+    turn[0] += 1
+    ops.attn_decode(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0)
+
+  def front():
+    k, v = caches[turn[0] % copies]
+    turn[0] += 1
+    ops.attn_decode_front(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0,
+                          weight, weight, 1e-6, cos_sin, positions, slots)
+
+  calls = copies * max(1, args.calls // copies)
+  for name, fn in (("attn_decode", plain), ("attn_decode_front", front)):
+    t = graph_time_us(fn, calls)
+    print(f"{name}: {B} requests of {L} tokens, {nq}/{nkv} heads of {d}, {splits} splits, cache {cache_bytes / 1e6:.1f} MB: "
+          f"{t:.1f} us with the merge, {cache_bytes / t / 1e6:.2f} TB/s")
+  return 0
+
+
 def main(argv=None) -> int:
   ap = argparse.ArgumentParser(prog="python -m miniinfer_amd.kernels.microbench")
   sub = ap.add_subparsers(dest="cmd", required=True)
@@ -113,6 +141,16 @@ def main(argv=None) -> int:
   a.add_argument("--page-size", type=int, default=16)
   a.add_argument("--calls", type=int, default=20)
   a.set_defaults(fn=cmd_prefill_attention)
+  d = sub.add_parser("decode-attention", help="the split-key decode attention and its merge")
+  d.add_argument("--batch", type=int, default=8)
+  d.add_argument("--context", type=int, default=2048)
+  d.add_argument("--heads", type=int, default=16)
+  d.add_argument("--kv-heads", type=int, default=8)
+  d.add_argument("--head-dim", type=int, default=128)
+  d.add_argument("--page-size", type=int, default=16)
+  d.add_argument("--splits", type=int, default=0, help="key ranges per request (default: the engine's choice)")
+  d.add_argument("--calls", type=int, default=24)
+  d.set_defaults(fn=cmd_decode_attention)
   args = ap.parse_args(argv)
   if not torch.cuda.is_available():
     print("miniinfer_amd runs on the GPU only", file=sys.stderr)

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_int64, c_void_p
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
@@ -282,16 +282,83 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor
 
 
 SKINNY_MAX_ROWS = 64
-SKINNY_OWN_ROWS = 16                 # up to here the weight-streaming kernel is the quicker one for every matrix
+SKINNY_OWN_ROWS = 16                 # without a measurement: up to here the weight-streaming kernel for every matrix,
 SKINNY_OWN_ELEMENTS = 8 << 20        # and for more rows (up to SKINNY_MAX_ROWS) while the matrix is smaller than this
+TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_products` times the two candidates
+_PRODUCT_CHOICE: Dict[tuple, bool] = {}  # (rows point, matrix rows, k, gate|up) -> the weight-streaming kernel is quicker
 
 
-def skinny_preferred(num_rows: int, n: int, k: int) -> bool:
-  """Whether a product of `num_rows` rows with an [n, k] matrix goes to `gemm_skinny` rather than to the library.
-  Each wave of that kernel reads the left operand's rows for its own slice of k again, so beyond 16 rows its
-  loads are mostly left operand; on matrices of tens of MB the library's kernels (which split k across workgroups)
-  then stream the weights about twice as fast, which outweighs the norm and activation kernels that fusing saved."""
-  return num_rows <= SKINNY_OWN_ROWS or (num_rows <= SKINNY_MAX_ROWS and n * k < SKINNY_OWN_ELEMENTS)
+def set_product_choice(rows_point: int, matrix_rows: int, k: int, gate_up: bool, own: bool) -> None:
+  _PRODUCT_CHOICE[(rows_point, matrix_rows, k, bool(gate_up))] = bool(own)
+
+
+def product_choice_known(matrix_rows: int, k: int, gate_up: bool) -> bool:
+  return all((p, matrix_rows, k, bool(gate_up)) in _PRODUCT_CHOICE for p in TUNE_ROWS)
+
+
+def clear_product_choices() -> None:
+  _PRODUCT_CHOICE.clear()
+
+
+_SIDE_STREAMS: Dict[int, "torch.cuda.Stream"] = {}
+
+
+def side_stream(device=None) -> "torch.cuda.Stream":
+  """One stream per device beside the current one, for warm-up runs before a graph capture.  It is made once:
+  every further stream a process has used has cost later decode steps time here (a step of 32 requests ran 10%
+  slower after eight streams had been used once), so nothing in this package makes streams freely."""
+  index = torch.device(device).index if device is not None else None
+  if index is None:
+    index = torch.cuda.current_device()
+  if index not in _SIDE_STREAMS:
+    _SIDE_STREAMS[index] = torch.cuda.Stream(device=index)
+  return _SIDE_STREAMS[index]
+
+
+_OWN_ONLY = [False]
+_LIBRARY_PRODUCTS = [0]
+
+
+class own_products_only:
+  """While active, `skinny_preferred` sends every product of up to SKINNY_MAX_ROWS rows to this library's kernel."""
+
+  def __enter__(self):
+    self.was, _OWN_ONLY[0] = _OWN_ONLY[0], True
+    return self
+
+  def __exit__(self, *exc):
+    _OWN_ONLY[0] = self.was
+    return False
+
+
+def library_products_run() -> int:
+  """How many products have gone to the library so far (`linear` counts them with `note_library_product`)."""
+  return _LIBRARY_PRODUCTS[0]
+
+
+def note_library_product() -> None:
+  _LIBRARY_PRODUCTS[0] += 1
+
+
+def skinny_preferred(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> bool:
+  """Whether a product of `num_rows` rows with a [matrix_rows, k] matrix (a fused gate|up matrix counts its 2 I
+  rows) goes to `gemm_skinny` rather than to the library: what `tuning.tune_products` measured for this shape at
+  the next row count of TUNE_ROWS, else a rule.  The rule: each wave of that kernel reads the left operand's rows
+  for its own slice of k again, so beyond 16 rows its loads are mostly left operand; on matrices of tens of MB the
+  library's kernels (which split k across workgroups) then stream the weights about twice as fast, which
+  outweighs the norm and activation kernels that fusing saved."""
+  if num_rows > SKINNY_MAX_ROWS:
+    return False
+  if _OWN_ONLY[0]:
+    return True
+  if _PRODUCT_CHOICE:
+    for p in TUNE_ROWS:
+      if p >= num_rows:
+        c = _PRODUCT_CHOICE.get((p, matrix_rows, k, bool(gate_up)))
+        if c is not None:
+          return c
+        break
+  return num_rows <= SKINNY_OWN_ROWS or matrix_rows * k < SKINNY_OWN_ELEMENTS
 
 
 def gemm_skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:

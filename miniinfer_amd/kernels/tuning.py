@@ -1,0 +1,102 @@
+"""Which kernel runs a product of few rows is measured, not guessed.
+
+For a matrix of tens of MB and a handful of rows there are two candidates: this library's weight-streaming kernel
+(`ops.gemm_skinny`, whose epilogue can take a norm's halves or the gated activation) and the library product
+(hipBLASLt through `torch.matmul`, which splits k across workgroups and so reads the left operand less often, but
+needs the norm and the activation as kernels of their own).  Which is quicker depends on the shape and the number
+of rows in ways no short rule covers, so `tune_products` times both on the model's own matrices once, when an
+engine is built, and `ops.skinny_preferred` then answers from the table.  Matrices below `MIN_ELEMENTS` are not
+timed: there the weight-streaming kernel and its fusions win by the kernels they save.
+"""
+
+from __future__ import annotations
+
+from typing import Callable, Dict, Iterable, List, Optional, Tuple
+
+import torch
+
+from . import ops
+
+MIN_ELEMENTS = 2 << 20
+UNFUSED_US = 3.0          # what a norm or activation kernel of its own costs inside a decode step
+
+
+def graph_time_us(fn: Callable[[], None], calls: int, flush: Optional[torch.Tensor] = None) -> float:
+  """Microseconds per call of `fn`, from one replay of a graph that holds `calls` calls (device time, no launch
+  gaps).  `flush`: a large tensor that is overwritten before the timed replay, so that nothing read is cached."""
+  fn()
+  torch.cuda.synchronize()
+  side = ops.side_stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    fn()
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  g = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(g):
+    for _ in range(calls):
+      fn()
+  g.replay()
+  torch.cuda.synchronize()
+  best = float("inf")
+  start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  for _ in range(2):
+    if flush is not None:
+      flush.zero_()
+    start.record()
+    g.replay()
+    end.record()
+    torch.cuda.synchronize()
+    best = min(best, start.elapsed_time(end) / calls * 1e3)
+  return best
+
+
+def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[Callable[[str], None]] = None) -> int:
+  """products: (weight [N, K] or fused gate|up [2 I, K], is gate|up) of every product that decode steps run; the
+  same shape usually comes once per layer, and the timing walks through all of them in turn so that the weights
+  come from memory as they do in a step.  Fills the table behind `ops.skinny_preferred` for every shape of at
+  least MIN_ELEMENTS and every row count in `ops.TUNE_ROWS`; returns the number of shapes timed."""
+  groups: Dict[tuple, List[torch.Tensor]] = {}
+  for w, gate_up in products:
+    if w is None or w.dtype != torch.bfloat16 or not w.is_cuda or w.dim() != 2 or w.numel() < MIN_ELEMENTS:
+      continue
+    groups.setdefault((w.shape[0], w.shape[1], bool(gate_up)), []).append(w)
+  timed = 0
+  flush = None
+  for (rows_w, K, gate_up), ws in groups.items():
+    N = rows_w // 2 if gate_up else rows_w
+    if ops.product_choice_known(rows_w, K, gate_up):
+      continue
+    probe = torch.zeros(1, K, dtype=torch.bfloat16, device=ws[0].device)
+    if not ops.gemm_skinny_supported(probe, ws[0]):
+      continue
+    if flush is None:
+      flush = torch.empty(512 << 20, dtype=torch.uint8, device=ws[0].device)
+    calls = max(8, min(len(ws), 32))
+    for M in ops.TUNE_ROWS:
+      a = (torch.randn(M, K, device=ws[0].device) * 0.1).bfloat16()
+      out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
+      turn = [0]
+
+      def own():
+        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up)
+        turn[0] += 1
+
+      def library():
+        torch.matmul(a, ws[turn[0] % len(ws)].t())
+        turn[0] += 1
+
+      t_own = graph_time_us(own, calls, flush)
+      t_lib = graph_time_us(library, calls, flush) + (2 if gate_up else 1) * UNFUSED_US
+      ops.set_product_choice(M, rows_w, K, gate_up, t_own <= t_lib)
+      if log is not None:
+        log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: own {t_own:.1f} us, "
+            f"library {t_lib:.1f} us with its extra kernels")
+    timed += 1
+  if timed:
+    # give the timing's buffers back to the driver: what is allocated next (the cache pools) then lies as it would
+    # have without the timing (pools carved out of recycled blocks have streamed measurably slower)
+    del flush
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+  return timed

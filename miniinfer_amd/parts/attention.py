@@ -57,6 +57,9 @@ class PagedAttention(Part):
       out.append((self.spec.tensor_names[5] + ".", self.k_norm))
     return out
 
+  def products(self):
+    return [(self.qkv_weight, False), (self.o_weight, False)]
+
   def cache_requirement(self):
     return PagedKV(num_kv_heads=self.nkv, head_dim=self.d, window=self.window)
 

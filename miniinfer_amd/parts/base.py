@@ -109,6 +109,15 @@ class Part:
     for sub, child in self.children():
       yield from child.named_params(prefix + sub)
 
+  def products(self) -> List[Tuple[torch.Tensor, bool]]:
+    """(matrix, whether it is a fused gate|up matrix) of every product this part and its children run on a step's
+    rows through `linear` / `gate_up_activation`; an engine times the candidates for them once
+    (`kernels.tuning.tune_products`)."""
+    out: List[Tuple[torch.Tensor, bool]] = []
+    for _, child in self.children():
+      out.extend(child.products())
+    return out
+
   def finalize(self) -> None:
     """Called once after all tensors have arrived."""
     for _, child in self.children():

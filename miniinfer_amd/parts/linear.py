@@ -55,7 +55,7 @@ def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]
   M = d.residual.shape[0]
   if d.consumed or d.dtype != torch.bfloat16:
     return None
-  if not ops.skinny_preferred(M, weight.shape[0], weight.shape[1]):
+  if not ops.skinny_preferred(M, weight.shape[0], weight.shape[1], gate_up):
     return None
   N = weight.shape[0] // 2 if gate_up else weight.shape[0]
   if isinstance(d.x, PendingLinear) and d.x.value is None:
@@ -96,9 +96,10 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
   M, N = x.shape[0], weight.shape[0]
   if not x.is_cuda:
     raise ops.KernelError("miniinfer_amd runs on the GPU only")
-  if ops.gemm_skinny_supported(x, weight) and (out_dtype == torch.float32 or ops.skinny_preferred(M, N, x.shape[1])):
-    # few rows (decode): the time is the time to stream the weights; this library's MFMA kernel
-    return ops.gemm_skinny(x, weight, torch.empty((M, N), dtype=out_dtype, device=x.device))
+  if ops.gemm_skinny_supported(x, weight):
+    if out_dtype == torch.float32 or ops.skinny_preferred(M, N, x.shape[1]):
+      # few rows (decode): the time is the time to stream the weights; this library's MFMA kernel
+      return ops.gemm_skinny(x, weight, torch.empty((M, N), dtype=out_dtype, device=x.device))
   if out_dtype == torch.float32 and M > ops.SKINNY_MAX_ROWS and ops.gemm_skinny_supported(x[:1], weight):
     # 32-bit results from bfloat16 operands for more rows (the logits of many requests): the same kernel, 64 rows
     # at a time; the weights stream once per 64 rows, which is still far quicker than the FMA kernel
@@ -109,6 +110,7 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
   if x.dtype == torch.float32 or out_dtype != x.dtype:
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     return ops.gemm_nt(x, weight, out)
+  ops.note_library_product()
   return torch.matmul(x, weight.t())
 
 
@@ -122,7 +124,7 @@ def gate_up_activation(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.T
       return y
     x = x.materialize()
   M, inter = x.shape[0], gate_up_weight.shape[0] // 2
-  if ops.gemm_skinny_supported(x, gate_up_weight) and ops.skinny_preferred(M, 2 * inter, x.shape[1]):
+  if ops.gemm_skinny_supported(x, gate_up_weight) and ops.skinny_preferred(M, 2 * inter, x.shape[1], True):
     return ops.gemm_skinny(x, gate_up_weight, torch.empty((M, inter), dtype=x.dtype, device=x.device), gate_up=True)
   gu = linear(x, gate_up_weight)
   act = torch.empty((M, inter), dtype=x.dtype, device=x.device)

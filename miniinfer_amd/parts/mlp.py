@@ -31,6 +31,9 @@ class GatedMLP(Part):
       ParamSpec("down_weight", (self.hidden, self.inter), (Source(d + ".weight", self.hidden),)),
     ]
 
+  def products(self):
+    return [(self.gate_up_weight, True), (self.down_weight, False)]
+
   def forward(self, x, ctx) -> torch.Tensor:
     return self.forward_lazy(x, ctx).materialize()
 

@@ -129,6 +129,7 @@ def test_block_alone(dtype, library_products, monkeypatch):
   if library_products:
     monkeypatch.setattr(ops, "SKINNY_OWN_ELEMENTS", 0)
     assert ops.skinny_preferred(16, 64, 64) and not ops.skinny_preferred(17, 64, 64)
+    assert not ops.skinny_preferred(65, 64, 64)
   from miniinfer_amd.cache import CacheManager
   from miniinfer_amd.config import Qwen3Config, model_spec_of
   from miniinfer_amd.engine.runner import StepEntry
