@@ -31,6 +31,8 @@ def _engine_args(p):
   p.add_argument("--eager", action="store_true", help="never replay decode steps from HIP graphs")
   p.add_argument("--no-overlap", action="store_true",
                  help="read each step's tokens back before the next step is launched")
+  p.add_argument("--no-tune", action="store_true",
+                 help="choose the kernels of small-batch products by rule instead of timing them at start")
   p.add_argument("--seed", type=int, default=0)
 
 
@@ -46,7 +48,7 @@ def _engine(args):
                    max_model_len=args.max_model_len, page_size=args.page_size, num_pages=args.num_pages,
                    max_num_batched_tokens=args.max_num_batched_tokens,
                    enable_chunked_prefill=not args.no_chunked_prefill, enforce_eager=args.eager, enable_overlap=not args.no_overlap,
-                   seed=args.seed)
+                   tune_products=not args.no_tune, seed=args.seed)
 
 
 def cmd_generate(args) -> int:

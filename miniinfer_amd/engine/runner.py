@@ -149,15 +149,17 @@ class _DecodeGraph:
     before = ops.library_products_run()
     self.graph, self.logits = self._capture(runner, ctx)
     self.ok = True
-    library = ops.library_products_run() != before
-    if library and B <= ops.SKINNY_MAX_ROWS:
+    after = ops.library_products_run()
+    library, avoidable = after[0] != before[0], after[1] != before[1]
+    if avoidable:
       # The step sends some products of few rows to the library (by measurement of each product alone, or by
       # rule).  Inside a step that can still lose to this library's own kernels, which need no norm and activation
       # kernels beside them: the step is captured both ways and the quicker graph is kept.
       with ops.own_products_only():
         own_graph, own_logits = self._capture(runner, ctx)
       if self._replay_ms(own_graph) <= self._replay_ms(self.graph):
-        self.graph, self.logits, library = own_graph, own_logits, False
+        self.graph, self.logits = own_graph, own_logits
+        library = (after[0] - before[0]) > (after[1] - before[1])     # library products that were not avoidable
     if library and runner.check_graphs:
       # What a library records into a graph is its own affair (clears of a workspace have replayed wrongly): the
       # graph is replayed a few times, with eager work in between, against the eager result of the same (padding)

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_int64, c_void_p
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -316,7 +316,7 @@ def side_stream(device=None) -> "torch.cuda.Stream":
 
 
 _OWN_ONLY = [False]
-_LIBRARY_PRODUCTS = [0]
+_LIBRARY_PRODUCTS = [0, 0]
 
 
 class own_products_only:
@@ -331,13 +331,16 @@ class own_products_only:
     return False
 
 
-def library_products_run() -> int:
-  """How many products have gone to the library so far (`linear` counts them with `note_library_product`)."""
-  return _LIBRARY_PRODUCTS[0]
+def library_products_run() -> Tuple[int, int]:
+  """(all, avoidable): how many products have gone to the library so far, and how many of them this library's
+  weight-streaming kernel could have run instead (`linear` counts them with `note_library_product`)."""
+  return _LIBRARY_PRODUCTS[0], _LIBRARY_PRODUCTS[1]
 
 
-def note_library_product() -> None:
+def note_library_product(avoidable: bool = False) -> None:
   _LIBRARY_PRODUCTS[0] += 1
+  if avoidable:
+    _LIBRARY_PRODUCTS[1] += 1
 
 
 def skinny_preferred(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> bool:

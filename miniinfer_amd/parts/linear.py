@@ -96,21 +96,22 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
   M, N = x.shape[0], weight.shape[0]
   if not x.is_cuda:
     raise ops.KernelError("miniinfer_amd runs on the GPU only")
+  avoidable = False
   if ops.gemm_skinny_supported(x, weight):
-    if out_dtype == torch.float32 or ops.skinny_preferred(M, N, x.shape[1]):
+    own = M <= ops.SKINNY_OWN_ROWS if out_dtype == torch.float32 else ops.skinny_preferred(M, N, x.shape[1])
+    avoidable = out_dtype != torch.float32
+    if own:
       # few rows (decode): the time is the time to stream the weights; this library's MFMA kernel
       return ops.gemm_skinny(x, weight, torch.empty((M, N), dtype=out_dtype, device=x.device))
-  if out_dtype == torch.float32 and M > ops.SKINNY_MAX_ROWS and ops.gemm_skinny_supported(x[:1], weight):
-    # 32-bit results from bfloat16 operands for more rows (the logits of many requests): the same kernel, 64 rows
-    # at a time; the weights stream once per 64 rows, which is still far quicker than the FMA kernel
-    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-    for r0 in range(0, M, ops.SKINNY_MAX_ROWS):
-      ops.gemm_skinny(x[r0:r0 + ops.SKINNY_MAX_ROWS], weight, out[r0:r0 + ops.SKINNY_MAX_ROWS])
-    return out
+  if out_dtype == torch.float32 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+    # 32-bit results from bfloat16 operands for more rows (the logits of many requests): the library product with
+    # a 32-bit result (84 us for 64 rows of a [151936, 1024] head against 148 us for the kernel above)
+    ops.note_library_product()
+    return torch.mm(x, weight.t(), out_dtype=torch.float32)
   if x.dtype == torch.float32 or out_dtype != x.dtype:
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     return ops.gemm_nt(x, weight, out)
-  ops.note_library_product()
+  ops.note_library_product(avoidable)
   return torch.matmul(x, weight.t())
 
 
