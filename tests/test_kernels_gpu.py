@@ -291,6 +291,23 @@ def test_mfma_decode_attention_any_number_of_splits(nq, nkv, d, P, window, split
   assert float(out[:5].abs().sum()) == 0.0       # rows of the multi-token entries are not touched
 
 
+@pytest.mark.parametrize("splits", [1, 5])
+@pytest.mark.parametrize("P,long_kv", [(8, 2100), (16, 4200), (16, 4090)])
+def test_mfma_decode_attention_with_long_block_tables(P, long_kv, splits):
+  """Requests of thousands of keys beside short ones: block tables of 263 and of exactly 256 entries."""
+  from miniinfer_amd.kernels import ops
+  nq, nkv, d = 4, 2, 32
+  reqs = [(long_kv - 1, 1), (300, 1), (0, 1)]
+  c = _paged_case(reqs, nq, nkv, d, P, 0, seed=12)
+  assert (c["table"].shape[1] > 256) == (long_kv != 4090)
+  out = torch.zeros(c["T"], nq * d, dtype=torch.bfloat16, device=DEV)
+  part_o = torch.empty(3 * nq * splits * d, dtype=torch.float32, device=DEV)
+  part_ml = torch.empty(3 * nq * splits * 2, dtype=torch.float32, device=DEV)
+  ops.attn_decode(c["q"], nq, nkv, d, out, c["kp"], c["vp"], c["table"], c["cu"], c["kv"], 0, 3, splits, part_o,
+                  part_ml, d ** -0.5, 0)
+  torch.testing.assert_close(out.double().cpu(), c["want"], rtol=1.6e-2, atol=1e-2)
+
+
 def test_mfma_attention_finds_a_far_key_and_respects_the_window_edge():
   """One key among hundreds is made to stand out (its score is far above the rest): the output must be its value.
   With a window that just excludes it, it must vanish; with one that just includes it, it is back."""
