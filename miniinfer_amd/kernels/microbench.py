@@ -3,12 +3,15 @@
     python -m miniinfer_amd.kernels.microbench product --rows 8 --n 25600 --k 5120 --gate-up
     python -m miniinfer_amd.kernels.microbench prefill-attention --tokens 2048 --heads 16 --kv-heads 8 --head-dim 128
     python -m miniinfer_amd.kernels.microbench decode-attention --batch 8 --context 2048 --heads 16 --kv-heads 8
+    python -m miniinfer_amd.kernels.microbench choices --preset qwen3-8b
 
 `product` times the weight-streaming product (`ops.gemm_skinny`) beside the library's product for the same operands;
 the weights cycle through several copies so that they stream from memory, not from a cache.  `prefill-attention`
 times `ops.attn_prefill` for one prompt in both of its variants; `decode-attention` times the split-key decode
 kernel and its merge for a batch of requests, with and without the fused norm, rotation and cache write, over
-several caches in turn.  All print one line per measurement; under
+several caches in turn; `choices` builds a preset's model with random weights and prints what an engine measures
+at its start: the time of the own and of the library kernel for each of the model's products at 1 to 64 rows.
+All print one line per measurement; under
 `rocprofv3 --pmc ...` the same commands give the kernels' counters.
 """
 
@@ -123,6 +126,17 @@ def cmd_decode_attention(args) -> int:
   return 0
 
 
+def cmd_choices(args) -> int:
+  from ..config import model_spec_of
+  from ..presets import preset
+  from ..weights import build_model, fill_random
+  from .tuning import tune_products
+  model = build_model(model_spec_of(preset(args.preset, args.num_hidden_layers)), torch.bfloat16, torch.device(DEV))
+  fill_random(model, 0)
+  tune_products(model.products(), log=print)
+  return 0
+
+
 def main(argv=None) -> int:
   ap = argparse.ArgumentParser(prog="python -m miniinfer_amd.kernels.microbench")
   sub = ap.add_subparsers(dest="cmd", required=True)
@@ -151,6 +165,10 @@ def main(argv=None) -> int:
   d.add_argument("--splits", type=int, default=0, help="key ranges per request (default: the engine's choice)")
   d.add_argument("--calls", type=int, default=24)
   d.set_defaults(fn=cmd_decode_attention)
+  c = sub.add_parser("choices", help="own against library kernel for each product of a preset's model")
+  c.add_argument("--preset", default="qwen3-0.6b")
+  c.add_argument("--num-hidden-layers", type=int, default=None)
+  c.set_defaults(fn=cmd_choices)
   args = ap.parse_args(argv)
   if not torch.cuda.is_available():
     print("miniinfer_amd runs on the GPU only", file=sys.stderr)
