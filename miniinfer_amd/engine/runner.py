@@ -14,6 +14,7 @@ index arrays are built on the host with numpy and reach the device in one copy.
 
 from __future__ import annotations
 
+import warnings
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
@@ -163,14 +164,23 @@ class _DecodeGraph:
     if library and runner.check_graphs:
       # What a library records into a graph is its own affair (clears of a workspace have replayed wrongly): the
       # graph is replayed a few times, with eager work in between, against the eager result of the same (padding)
-      # inputs, and a graph that does not reproduce it is not used.
+      # inputs, and a graph that does not reproduce it is not used.  A library may choose another kernel under
+      # capture than it does eagerly, which moves the result by a rounding of bfloat16 (0.4% of the largest logit
+      # has been seen): the replays must agree with the eager result to within 1.5% of the largest logit, and
+      # with one another exactly, which a stale workspace would not.
       want = runner.model.forward(ctx).clone()
+      bound = 1.5e-2 * max(float(want.abs().max()), 1e-6)
+      first = None
       for _ in range(3):
         self.graph.replay()
         got = self.logits.clone()
         torch.cuda.synchronize()
-        if not torch.allclose(got, want, rtol=1e-3, atol=1e-3):
+        if first is None:
+          first = got
+        if float((got - want).abs().max()) > bound or not torch.equal(got, first):
           self.ok = False
+          warnings.warn(f"the captured decode step for {B} entries does not reproduce the eager step; "
+                        "such steps run without a graph")
           break
         want = runner.model.forward(ctx).clone()
 

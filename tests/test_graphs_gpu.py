@@ -110,3 +110,41 @@ def test_graphs_of_many_requests_hold_library_products_and_still_equal_eager_ste
   for e, g in zip(*outs):
     assert e.shape == g.shape
     assert float((e - g).abs().max()) <= 2e-2 * max(float(e.abs().max()), 1.0)
+
+
+def test_a_step_whose_products_could_go_either_way_is_captured_both_ways(tmp_path, monkeypatch):
+  """With 17 to 64 single tokens a product may go to the library or to this library's own kernel.  When the rule (or
+  the measurement) says library, the runner captures the step both ways and keeps the quicker graph; whichever it
+  keeps reproduces the eager steps."""
+  from miniinfer_amd.cache.manager import CacheManager
+  from miniinfer_amd.engine.runner import ModelRunner, StepEntry
+  from miniinfer_amd.kernels import ops
+  from miniinfer_amd.weights import load_model
+  monkeypatch.setattr(ops, "SKINNY_OWN_ELEMENTS", 0)       # every matrix counts as large: library beyond 16 rows
+  cfg, _ = tm.make_model(str(tmp_path / "m"), "B", seed=9, dtype=torch.bfloat16, std=0.05)
+  runners = []
+  for graphs in (False, True):
+    model, _ = load_model(str(tmp_path / "m"), torch.bfloat16, "cuda:0")
+    cache = CacheManager(model.cache_needs(), page_size=16, num_pages=120, max_requests=32,
+                         max_model_len=model.spec.max_positions, dtype=torch.bfloat16, device="cuda:0")
+    runners.append(ModelRunner(model, cache, use_graphs=graphs))
+  outs = [[], []]
+  counted = []
+  for k, rn in enumerate(runners):
+    live = []
+    for r in range(24):
+      rn.cache.admit(r)
+      rn.step([StepEntry(r, tm.random_tokens(cfg, 2 + r % 11, seed=r), [])])
+      live.append(r)
+    before = ops.library_products_run()
+    for t in range(5):
+      outs[k].append(rn.step([StepEntry(q, [(5 * q + t) % cfg["vocab_size"]], [0]) for q in live]).float().cpu())
+      torch.cuda.synchronize()
+    after = ops.library_products_run()
+    counted.append((after[0] - before[0], after[1] - before[1]))
+  assert counted[0][1] > 0, "the eager steps of 24 rows sent no avoidable product to the library"
+  assert {b for b, _ in runners[1]._graphs} == {24}
+  assert all(g.ok for g in runners[1]._graphs.values())
+  for e, g in zip(*outs):
+    assert e.shape == g.shape
+    assert float((e - g).abs().max()) <= 2e-2 * max(float(e.abs().max()), 1.0)
