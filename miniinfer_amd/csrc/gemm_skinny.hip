@@ -53,11 +53,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   // GATE_UP: RB == 2, row block 0 = gate rows n0.., row block 1 = up rows N + n0..; N counts output columns
-  // rpg: rows of W per workgroup when RB == 1 (16, or fewer so that a matrix of few rows still gives every compute
-  // unit a workgroup: the lanes of the other rows then load nothing and their results are dropped)
-  const int n0 = GATE_UP ? blockIdx.x * 16 : (RB == 1 ? blockIdx.x * rpg : blockIdx.x * 16 * RB);
-  const int n_end = min(N, n0 + (GATE_UP ? 16 : (RB == 1 ? rpg : 16 * RB)));
-  const bool w_live = GATE_UP || RB > 1 || (lane & 15) < rpg;
+  // rpg: rows of W per workgroup and row block when RB == 1 or GATE_UP: 16, or fewer so that the workgroups fill
+  // whole rounds of the compute units (the lanes of the other rows then load nothing and their results are dropped)
+  constexpr bool CUT = GATE_UP || RB == 1;
+  const int n0 = CUT ? blockIdx.x * rpg : blockIdx.x * 16 * RB;
+  const int n_end = min(N, n0 + (CUT ? rpg : 16 * RB));
+  const bool w_live = !CUT || (lane & 15) < rpg;
   const int steps = (K + 31) / 32;
   const int spw = (steps + nw - 1) / nw;
   const int s_begin = wave * spw;
@@ -390,14 +391,32 @@ struct SkinnyGrid {
   int RB, rpg, groups;
 };
 
+static int compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+  }
+  return cus;
+}
+
 static SkinnyGrid skinny_grid(bool gate_up, int N, int M) {
   const int row_blocks = (N + 15) / 16;
   SkinnyGrid g;
   g.RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
   g.rpg = 16;
-  if (!gate_up && g.RB == 1 && M <= 16)
-    while (g.rpg > 4 && (N + g.rpg - 1) / g.rpg < 256) g.rpg /= 2;
-  g.groups = gate_up ? row_blocks : (g.RB == 1 ? (N + g.rpg - 1) / g.rpg : (row_blocks + g.RB - 1) / g.RB);
+  if ((gate_up || g.RB == 1) && M <= 16) {
+    // A workgroup of 16 waves has a compute unit to itself, so the launch runs in rounds of as many workgroups as
+    // there are units, and 320 workgroups take as long as 512.  The rows are shared out so that the last round is
+    // as full as the others: 5,120 rows on 256 units go as 512 groups of 10, 1,024 rows as 256 groups of 4.
+    const int cus = compute_units();
+    const int rounds = (N + 16 * cus - 1) / (16 * cus);
+    const int rpg = (N + cus * rounds - 1) / (cus * rounds);
+    g.rpg = rpg < 4 ? 4 : (rpg > 16 ? 16 : rpg);
+  }
+  g.groups = (gate_up || g.RB == 1) ? (N + g.rpg - 1) / g.rpg : (row_blocks + g.RB - 1) / g.RB;
   return g;
 }
 
