@@ -467,8 +467,11 @@ MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t
   const SkinnyGrid sg = skinny_grid(gate_up != 0, N, M);
   const int RB = sg.RB, groups = sg.groups;
   const int steps = (K + 31) / 32;
-  // enough waves to fill the chip, at least 2 steps of K per wave, at most 16 waves per workgroup
+  // enough waves to fill the chip (where one would do, four: a launch of thousands of workgroups then ends in
+  // smaller pieces; the output head takes 263 instead of 288 us); at least 2 steps of K per wave, at most 16 waves
+  // per workgroup
   int waves = (4096 + groups - 1) / groups;
+  if (waves < 2) waves = 4;
   if (waves > 16) waves = 16;
   if (waves > steps / 2) waves = steps / 2;
   if (waves < 1) waves = 1;
