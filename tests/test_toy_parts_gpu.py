@@ -1,0 +1,269 @@
+"""More generality of the parts, again with toy parts that live only in this file and are registered from outside
+the framework:
+  * a feed-forward with routing (a router in 32-bit, the two best of four small gated experts per token, their
+    weights renormalised),
+  * another position encoding (rotation of half of each head only, by angles of an interpolated position, from a
+    table the part builds itself),
+  * a layer whose attention has no position encoding at all, beside a layer with the ordinary one.
+A second toy architecture made of them is built from a config.json, loaded by tensor name and stepped whole, in
+portions and in mixed batches; its logits must equal a plain whole-sequence statement of the same model."""
+
+import json
+import os
+from dataclasses import dataclass
+from typing import List
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import trace_tools as tt
+
+pytestmark = pytest.mark.gpu
+
+E, TOPK = 4, 2
+
+
+@dataclass(frozen=True)
+class RoutedSpec:
+  hidden_size: int
+  expert_size: int
+  num_experts: int
+  top_k: int
+  kind: str = "toy_routed_experts"
+
+
+@dataclass(frozen=True)
+class SlowPartialRotarySpec:
+  rotary_dim: int          # of each head; the rest passes through
+  theta: float
+  factor: float            # positions are divided by it
+  max_positions: int
+  kind: str = "toy_slow_partial_rotary"
+
+
+def _register():
+  from miniinfer_amd.config import (AttentionSpec, GatedMLPSpec, LayerSpec, ModelSpec, NoPositionSpec, NormSpec,
+                                    RotarySpec, register_architecture)
+  from miniinfer_amd.parts import ParamSpec, Part, register_feed_forward, register_position
+
+  class RoutedExperts(Part):
+    """y_t = sum over the top_k experts e of w_te * down_e( silu(gate_e x_t) * up_e x_t ), w = the softmax of the
+    router's 32-bit logits over all experts, cut to the top_k and renormalised.  Plain torch: a toy, not a kernel."""
+
+    def __init__(self, spec, ctx):
+      self.spec, self.ctx = spec, ctx
+      self.router_weight = self.gate_up = self.down = None
+
+    def param_specs(self):
+      s = self.spec
+      return [ParamSpec.single("router.weight", (s.num_experts, s.hidden_size), storage="float32"),
+              ParamSpec.single("gate_up", (s.num_experts, 2 * s.expert_size, s.hidden_size)),
+              ParamSpec.single("down", (s.num_experts, s.hidden_size, s.expert_size))]
+
+    def forward(self, x, ctx):
+      s = self.spec
+      xf = x.float()
+      probs = torch.softmax(xf @ self.router_weight.float().T, dim=-1)
+      top_w, top_e = probs.topk(s.top_k, dim=-1)
+      top_w = top_w / top_w.sum(-1, keepdim=True)
+      out = torch.zeros_like(xf)
+      for e in range(s.num_experts):
+        gu = xf @ self.gate_up[e].float().T
+        act = torch.nn.functional.silu(gu[:, :s.expert_size]) * gu[:, s.expert_size:]
+        y = act.to(x.dtype).float() @ self.down[e].float().T
+        w = (top_w * (top_e == e)).sum(-1, keepdim=True)
+        out += w * y
+      return out.to(x.dtype)
+
+  register_feed_forward("toy_routed_experts", RoutedExperts)
+
+  class SlowPartialRotary(Part):
+    def __init__(self, spec, ctx):
+      j = torch.arange(0, spec.rotary_dim, 2, dtype=torch.float32)
+      ang = torch.outer(torch.arange(spec.max_positions, dtype=torch.float32) / spec.factor,
+                        1.0 / spec.theta ** (j / spec.rotary_dim))
+      self._table = torch.cat((ang.cos(), ang.sin()), dim=-1).contiguous().to(ctx.device)
+
+    def rotary_table(self):
+      return self._table
+
+  register_position("toy_slow_partial_rotary", SlowPartialRotary)
+
+  @dataclass(frozen=True)
+  class Toy2Config:
+    vocab_size: int
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    intermediate_size: int
+    expert_size: int
+    eps: float
+    theta: float
+    factor: float
+    max_positions: int
+
+    @classmethod
+    def from_dict(cls, raw):
+      return cls(**{k: raw[k] for k in cls.__dataclass_fields__})
+
+    def build_spec(self):
+      H, d = self.hidden_size, self.head_dim
+      norm = NormSpec(size=H, eps=self.eps)
+      positions = (SlowPartialRotarySpec(d // 2, self.theta, self.factor, self.max_positions), NoPositionSpec(),
+                   RotarySpec(rotary_dim=d, theta=self.theta, max_positions=self.max_positions))
+      routed = RoutedSpec(H, self.expert_size, E, TOPK)
+      dense = GatedMLPSpec(hidden_size=H, intermediate_size=self.intermediate_size)
+      layers = tuple(
+        LayerSpec(prefix=f"toy2.layers.{i}.",
+                  mixer=AttentionSpec(hidden_size=H, num_heads=self.num_heads, num_kv_heads=self.num_kv_heads,
+                                      head_dim=d, scale=d ** -0.5, position=positions[i],
+                                      qk_norm=NormSpec(d, self.eps)),
+                  feed_forward=dense if i == 1 else routed, mixer_norm=norm, feed_forward_norm=norm)
+        for i in range(3))
+      return ModelSpec(architecture="Toy2ForCausalLM", vocab_size=self.vocab_size, hidden_size=H, layers=layers,
+                       run_order=(0, 1, 2), final_norm=norm, embedding_name="toy2.embed.weight",
+                       final_norm_prefix="toy2.norm.", head_name="toy2.head.weight", head_optional=True,
+                       optional_name_prefix="", max_positions=self.max_positions)
+
+  register_architecture("Toy2ForCausalLM", Toy2Config)
+
+
+TOY2 = dict(architectures=["Toy2ForCausalLM"], vocab_size=200, hidden_size=40, num_heads=6, num_kv_heads=3, head_dim=32,
+            intermediate_size=56, expert_size=24, eps=3e-6, theta=3000.0, factor=4.0, max_positions=400)
+
+
+def _weights(seed=0, std=0.08):
+  g = torch.Generator().manual_seed(seed)
+  c = TOY2
+  H, V, nq, nkv, d, I, Ie = (c["hidden_size"], c["vocab_size"], c["num_heads"], c["num_kv_heads"], c["head_dim"],
+                             c["intermediate_size"], c["expert_size"])
+  mat = lambda *s: torch.randn(*s, generator=g) * std
+  norm = lambda n: 1 + 0.1 * torch.randn(n, generator=g)
+  w = {"toy2.embed.weight": mat(V, H), "toy2.norm.weight": norm(H)}       # no head: the embedding is the head
+  for i in range(3):
+    p = f"toy2.layers.{i}."
+    w[p + "input_layernorm.weight"] = norm(H)
+    w[p + "post_attention_layernorm.weight"] = norm(H)
+    for n, shape in (("q_proj", (nq * d, H)), ("k_proj", (nkv * d, H)), ("v_proj", (nkv * d, H)), ("o_proj", (H, nq * d))):
+      w[p + f"self_attn.{n}.weight"] = mat(*shape)
+    w[p + "self_attn.q_norm.weight"] = norm(d)
+    w[p + "self_attn.k_norm.weight"] = norm(d)
+    if i == 1:
+      for n, shape in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+        w[p + f"mlp.{n}.weight"] = mat(*shape)
+    else:
+      w[p + "mlp.router.weight"] = mat(E, H) * 40         # decided choices: a third expert is seldom close to the second
+      w[p + "mlp.gate_up"] = mat(E, 2 * Ie, H)
+      w[p + "mlp.down"] = mat(E, H, Ie)
+  return w
+
+
+def _rotate_part(x, ang, rd):
+  """NeoX rotation of the first rd dims of each head (pairs j, j + rd/2); the rest passes through."""
+  return torch.cat((plain.apply_rope_neox(x[..., :rd], ang), x[..., rd:]), dim=-1)
+
+
+def _plain_toy2(tokens: List[int], w, round_act, close_calls=None) -> torch.Tensor:
+  """Whole sequence, no cache, float64.  round_act: the engine's rounding of the experts' activation (identity in
+  the 32-bit mode), the one place where the toy part itself rounds.  close_calls: a list that receives, for every
+  routing decision, (gap between the second and third expert's logit relative to the largest logit, renormalised
+  weight of the second expert)."""
+  w = {k: v.double() for k, v in w.items()}
+  c = TOY2
+  T, nq, nkv, d, Ie = len(tokens), c["num_heads"], c["num_kv_heads"], c["head_dim"], c["expert_size"]
+  pos = torch.arange(T)
+  h = w["toy2.embed.weight"][torch.tensor(tokens)]
+  for i in range(3):
+    p = f"toy2.layers.{i}."
+    x = plain.rms_norm(h, w[p + "input_layernorm.weight"], c["eps"])
+    q = plain.rms_norm((x @ w[p + "self_attn.q_proj.weight"].T).reshape(T, nq, d), w[p + "self_attn.q_norm.weight"], c["eps"])
+    k = plain.rms_norm((x @ w[p + "self_attn.k_proj.weight"].T).reshape(T, nkv, d), w[p + "self_attn.k_norm.weight"], c["eps"])
+    v = (x @ w[p + "self_attn.v_proj.weight"].T).reshape(T, nkv, d)
+    if i == 0:
+      ang = plain.rope_angles(pos.double() / c["factor"], d // 2, c["theta"], torch.float64)
+      q, k = _rotate_part(q, ang, d // 2), _rotate_part(k, ang, d // 2)
+    elif i == 2:
+      ang = plain.rope_angles(pos, d, c["theta"], torch.float64)
+      q, k = plain.apply_rope_neox(q, ang), plain.apply_rope_neox(k, ang)
+    o = plain.grouped_attention(q, k, v, d ** -0.5, plain.causal_mask(T, T, torch.float64))
+    h = h + o.reshape(T, nq * d) @ w[p + "self_attn.o_proj.weight"].T
+    x = plain.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["eps"])
+    if i == 1:
+      h = h + plain.swiglu(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+      continue
+    logits = x @ w[p + "mlp.router.weight"].T
+    probs = torch.softmax(logits, dim=-1)
+    top_w, top_e = probs.topk(TOPK, dim=-1)
+    top_w = top_w / top_w.sum(-1, keepdim=True)
+    if close_calls is not None:
+      ranked = logits.sort(dim=-1, descending=True).values
+      for t in range(T):
+        close_calls.append((float((ranked[t, 1] - ranked[t, 2]) / ranked[t].abs().max()), float(top_w[t, 1])))
+    y = torch.zeros_like(h)
+    for t in range(T):
+      for j in range(TOPK):
+        e = int(top_e[t, j])
+        gu = w[p + "mlp.gate_up"][e] @ x[t]
+        act = round_act(torch.nn.functional.silu(gu[:Ie]) * gu[Ie:])
+        y[t] += top_w[t, j] * (w[p + "mlp.down"][e] @ act)
+    h = h + y
+  return plain.rms_norm(h, w["toy2.norm.weight"], c["eps"]) @ w["toy2.embed.weight"].T
+
+
+def test_partial_rotation_reduces_to_the_whole_one_and_only_distances_count():
+  """What pins the plain statement of the toy position encoding: with rd = d it is the ordinary rotation, and a
+  shift of all positions leaves q.k unchanged."""
+  g = torch.Generator().manual_seed(3)
+  q, k = torch.randn(5, 2, 16, generator=g, dtype=torch.float64), torch.randn(5, 2, 16, generator=g, dtype=torch.float64)
+  pos = torch.arange(5)
+  ang = plain.rope_angles(pos, 16, 100.0, torch.float64)
+  assert torch.equal(_rotate_part(q, ang, 16), plain.apply_rope_neox(q, ang))
+  dots = lambda shift: torch.einsum("ihd,jhd->hij", _rotate_part(q, plain.rope_angles((pos + shift).double() / 4, 8, 100.0, torch.float64), 8),
+                                    _rotate_part(k, plain.rope_angles((pos + shift).double() / 4, 8, 100.0, torch.float64), 8))
+  torch.testing.assert_close(dots(0), dots(37), rtol=1e-9, atol=1e-9)
+  assert not torch.allclose(_rotate_part(q, ang[:, :4], 8)[1:], q[1:])      # and it does rotate
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_routed_feed_forward_and_other_position_encodings_are_registered_built_and_stepped(tmp_path, dtype):
+  from safetensors.torch import save_file
+  _register()
+  from miniinfer_amd.engine.replay import Replayer
+  file_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
+  g = torch.Generator().manual_seed(2)
+  requests = {f"r{i}": torch.randint(0, 200, (n,), generator=g).tolist() for i, n in enumerate((64, 37, 3, 90, 41))}
+  round_act = (lambda a: a) if dtype == "float32" else (lambda a: a.to(torch.bfloat16).double())
+  # Which two experts a token goes to is a discontinuous choice: where the second and the third expert's logits
+  # are within a rounding of bfloat16 of one another and the second carries weight, either choice is right and the
+  # outputs differ by much.  The weights are drawn so that no decision of these requests is such a close call
+  # (the first seed that has none), so that the comparison below can stay as tight as everywhere else.
+  for seed in range(200):
+    w = {k: v.to(file_dtype) for k, v in _weights(seed).items()}
+    calls: list = []
+    want = {r: _plain_toy2(t, {k: v.float() for k, v in w.items()}, round_act, calls).float().numpy()
+            for r, t in requests.items()}
+    if not any(gap < 0.03 and weight > 0.01 for gap, weight in calls):
+      break
+  else:
+    raise AssertionError("no seed without a close routing call")
+  os.makedirs(tmp_path / "toy2")
+  with open(tmp_path / "toy2" / "config.json", "w") as f:
+    json.dump(TOY2, f)
+  save_file({k: v.contiguous() for k, v in w.items()}, str(tmp_path / "toy2" / "model.safetensors"))
+  for steps in (tt.whole(requests), tt.portions(requests), tt.mixed(requests, max_live=3, seed=6)):
+    rp = Replayer(str(tmp_path / "toy2"), dtype, tt.peak_tokens(steps, requests), page_size=16)
+    assert rp.model.head is None                          # the file has no head: the embedding stands in
+    assert len(rp.cache.paged) == 1 and rp.cache.paged[0].layers == [0, 1, 2] and not rp.cache.states
+    outs = []
+    for st in steps:
+      outs.append(rp.step(st))
+      rp.cache.check()
+    assert rp.cache.num_free_pages() == rp.cache.num_pages
+    got = tt.gather(steps, outs, requests, 200)
+    for r in requests:
+      err = np.abs(got[r] - want[r]).max()
+      scale = np.abs(want[r]).max()
+      assert err <= (2e-4 if dtype == "float32" else 4e-2 * scale), f"request {r}: max err {err:.3g} (scale {scale:.3g})"
