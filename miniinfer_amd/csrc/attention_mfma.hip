@@ -799,6 +799,42 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_ker
   }
 }
 
+// Up to FEW splits of one (entry, head): everything is asked for at once, the partial outputs before the maxima
+// and sums that weigh them are known, so the wave waits for memory once.  A lane takes 4 dims and reads every
+// split's (max, sum) itself.
+template <int FEW>
+__device__ __forceinline__ void merge_few(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                          int64_t base, int num_splits, uint16_t* __restrict__ o) {
+  static_assert(D <= 256, "a lane takes 4 of at most 256 dims");
+  const int lane = threadIdx.x;
+  const bool live = 4 * lane < D;
+  const int d0 = live ? 4 * lane : 0;
+  float2 ml[FEW];
+  f32x4 v[FEW];
+#pragma unroll
+  for (int j = 0; j < FEW; ++j) {
+    const int jj = j < num_splits ? j : num_splits - 1;        // a split again instead of a branch
+    ml[j] = *reinterpret_cast<const float2*>(part_ml + (base + jj) * 2);
+    v[j] = *reinterpret_cast<const f32x4*>(part_o + (base + jj) * D + d0);
+  }
+  float M = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < FEW; ++j) M = fmaxf(M, ml[j].x);
+  float L = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < FEW; ++j) {
+    const float w = (j < num_splits && ml[j].x != -INFINITY) ? __builtin_amdgcn_exp2f(ml[j].x - M) : 0.f;
+    L += w * ml[j].y;
+    acc[0] += w * v[j][0];
+    acc[1] += w * v[j][1];
+    acc[2] += w * v[j][2];
+    acc[3] += w * v[j][3];
+  }
+  const float inv = 1.f / L;
+  if (live) *reinterpret_cast<s16x4*>(o + d0) = pack_bf16x4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
+}
+
 // out[token of entry e][head] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s
 // One wave per (entry, head).  The lanes first share out the splits (maximum, weights, sum), then the dims;
 // the loads of a phase do not depend on one another, so they are all in flight together.
@@ -810,39 +846,11 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   const int lane = threadIdx.x;
   const int e = blockIdx.x / nq, head = blockIdx.x % nq;
   const int64_t base = ((int64_t)e * nq + head) * num_splits;
-  constexpr int FEW = 16;
-  if (num_splits <= FEW) {
-    // Few splits (the usual case): everything is asked for at once, the partial outputs before the maxima and
-    // sums that weigh them are known, so the kernel waits for memory once.  A lane takes 4 dims and reads every
-    // split's (max, sum) itself.
-    static_assert(D <= 256, "a lane takes 4 of at most 256 dims");
-    const bool live = 4 * lane < D;
-    const int d0 = live ? 4 * lane : 0;
-    float2 ml[FEW];
-    f32x4 v[FEW];
-#pragma unroll
-    for (int j = 0; j < FEW; ++j) {
-      const int jj = j < num_splits ? j : num_splits - 1;        // a split again instead of a branch
-      ml[j] = *reinterpret_cast<const float2*>(part_ml + (base + jj) * 2);
-      v[j] = *reinterpret_cast<const f32x4*>(part_o + (base + jj) * D + d0);
-    }
-    float M = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < FEW; ++j) M = fmaxf(M, ml[j].x);
-    float L = 0.f;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < FEW; ++j) {
-      const float w = (j < num_splits && ml[j].x != -INFINITY) ? __builtin_amdgcn_exp2f(ml[j].x - M) : 0.f;
-      L += w * ml[j].y;
-      acc[0] += w * v[j][0];
-      acc[1] += w * v[j][1];
-      acc[2] += w * v[j][2];
-      acc[3] += w * v[j][3];
-    }
-    const float inv = 1.f / L;
+  if (num_splits <= 32) {
     uint16_t* o = out + (int64_t)cu_q[first_entry + e] * out_row_stride + (int64_t)head * D;
-    if (live) *reinterpret_cast<s16x4*>(o + d0) = pack_bf16x4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
+    if (num_splits <= 8) merge_few<8>(part_o, part_ml, base, num_splits, o);
+    else if (num_splits <= 16) merge_few<16>(part_o, part_ml, base, num_splits, o);
+    else merge_few<32>(part_o, part_ml, base, num_splits, o);
     return;
   }
   constexpr int MAXR = 16;                       // 64 * 16 = 1024 splits at most

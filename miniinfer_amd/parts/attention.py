@@ -131,20 +131,20 @@ class PagedAttention(Part):
 
 
 def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, waves: int = 4,
-                  target_waves: int = 2048) -> int:
+                  resident_workgroups: int = 512) -> int:
   """Into how many key ranges (workgroups of `waves` waves, each taking macro tiles of `tile_keys` keys in turn) a
-  decoding request is cut.  `target_waves` waves are resident on the chip at once (two workgroups per compute
-  unit): the ranges are as many as still fit in one such round, since a second round that is nearly empty costs as
+  decoding request is cut.  `resident_workgroups` run on the chip at once (two per compute unit, whatever the head
+  size): the ranges are as many as still fit in one such round, since a second round that is nearly empty costs as
   much as a full one (96 kv-head entries: 5 ranges take 27 us, 6 take 32); when one range per entry would leave
-  more than a fifth of the round empty, two are used (384 entries: 77 against 82 us).  At least one macro tile per
-  wave."""
+  more than a fifth of the round empty, two are used (384 entries: 77 against 82 us).  At most 32, which the merge
+  kernel still combines in one pass over memory (one request of 32,768 keys: 34 us with 32 ranges, 47 with 64),
+  and at least one macro tile per wave."""
   tiles = -(-max_keys // tile_keys)
-  room = max(1, target_waves // max(1, waves))        # workgroups per round
   n = max(1, num_head_entries)
-  want = max(1, room // n)
-  if want == 1 and n < room and 5 * n <= 4 * room:
+  want = max(1, resident_workgroups // n)
+  if want == 1 and n < resident_workgroups and 5 * n <= 4 * resident_workgroups:
     want = 2
-  return int(max(1, min(want, max(1, tiles // waves), 256)))
+  return int(max(1, min(want, max(1, tiles // waves), 32)))
 
 
 register_mixer("paged_attention", PagedAttention)
