@@ -1,0 +1,44 @@
+"""Rules that size a launch or pick a kernel, as plain functions of sizes (no GPU)."""
+
+import pytest
+
+
+def test_decode_key_ranges_fill_one_round_and_stay_mergeable_in_one_pass():
+  from miniinfer_amd.parts.attention import decode_splits
+  for waves, tile in ((4, 64), (2, 32)):
+    for entries in (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 256):
+      for kv_heads in (1, 2, 8):
+        for keys in (1, 63, 64, 300, 2048, 8192, 40000, 1 << 20):
+          n = entries * kv_heads
+          s = decode_splits(n, keys, tile, waves)
+          tiles = -(-keys // tile)
+          assert 1 <= s <= 32
+          assert s == 1 or s * waves <= tiles                 # a wave of every range has a tile
+          assert s <= 2 or n * s <= 512                        # more than two ranges only while they fit one round
+  # the cases the rule was measured on
+  assert decode_splits(8 * 8, 2048) == 8 and decode_splits(12 * 8, 2048) == 5 and decode_splits(24 * 8, 2048) == 2
+  assert decode_splits(48 * 8, 2048) == 2 and decode_splits(64 * 8, 2048) == 1
+  assert decode_splits(8, 8192) == 32 and decode_splits(8, 32768) == 32 and decode_splits(8, 2048) == 8
+  assert decode_splits(8 * 4, 2048, 32, 2) == 16 and decode_splits(64 * 4, 2048, 32, 2) == 2
+
+
+def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
+  from miniinfer_amd.kernels import ops
+  ops.clear_product_choices()
+  try:
+    assert ops.skinny_preferred(1, 4096, 4096) and ops.skinny_preferred(16, 51200, 5120, True)
+    assert ops.skinny_preferred(64, 1024, 3072)                       # a small matrix
+    assert not ops.skinny_preferred(17, 4096, 4096)                   # a large one with more than 16 rows
+    assert not ops.skinny_preferred(65, 64, 64)                       # more rows than the kernel takes
+    for p in ops.TUNE_ROWS:
+      ops.set_product_choice(p, 4096, 4096, False, p > 8)
+    assert not ops.skinny_preferred(3, 4096, 4096) and not ops.skinny_preferred(8, 4096, 4096)
+    assert ops.skinny_preferred(9, 4096, 4096) and ops.skinny_preferred(64, 4096, 4096)
+    assert ops.skinny_preferred(3, 4096, 4096, True)                  # another shape: not measured, the rule
+    with ops.own_products_only():
+      assert ops.skinny_preferred(3, 4096, 4096) and ops.skinny_preferred(40, 51200, 5120)
+      assert not ops.skinny_preferred(65, 4096, 4096)
+    assert not ops.skinny_preferred(3, 4096, 4096)
+    assert ops.product_choice_known(4096, 4096, False) and not ops.product_choice_known(4096, 4096, True)
+  finally:
+    ops.clear_product_choices()
