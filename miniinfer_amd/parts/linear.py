@@ -82,6 +82,9 @@ def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]
   return out
 
 
+_MM_TAKES_OUT_DTYPE = [True]     # torch.mm(..., out_dtype=) exists in this torch (found out at the first call)
+
+
 def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
   """x: a tensor [M, K], a pending product, or a DeferredNorm (the add and the norm are then fused into the product
   if possible)."""
@@ -105,9 +108,20 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
       return ops.gemm_skinny(x, weight, torch.empty((M, N), dtype=out_dtype, device=x.device))
   if out_dtype == torch.float32 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
     # 32-bit results from bfloat16 operands for more rows (the logits of many requests): the library product with
-    # a 32-bit result (84 us for 64 rows of a [151936, 1024] head against 148 us for the kernel above)
-    ops.note_library_product()
-    return torch.mm(x, weight.t(), out_dtype=torch.float32)
+    # a 32-bit result (84 us for 64 rows of a [151936, 1024] head against 148 us for the kernel above); where the
+    # library has no such product, the kernel above, 64 rows at a time
+    if _MM_TAKES_OUT_DTYPE[0]:
+      try:
+        y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+        ops.note_library_product()
+        return y
+      except TypeError:
+        _MM_TAKES_OUT_DTYPE[0] = False
+    if ops.gemm_skinny_supported(x[:1], weight):
+      out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+      for r0 in range(0, M, ops.SKINNY_MAX_ROWS):
+        ops.gemm_skinny(x[r0:r0 + ops.SKINNY_MAX_ROWS], weight, out[r0:r0 + ops.SKINNY_MAX_ROWS])
+      return out
   if x.dtype == torch.float32 or out_dtype != x.dtype:
     out = torch.empty((M, N), dtype=out_dtype, device=x.device)
     return ops.gemm_nt(x, weight, out)

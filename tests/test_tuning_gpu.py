@@ -55,3 +55,18 @@ def test_either_choice_gives_the_product(clean_choices, own, M):
   gu = x.double() @ wgu.double().T
   want = torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]
   torch.testing.assert_close(a.double().cpu(), want, rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("library", [True, False])
+@pytest.mark.parametrize("M", [5, 40, 150])
+def test_32_bit_results_from_bfloat16_operands_either_way(M, library, monkeypatch):
+  """The logits' product: this library's kernel for up to 16 rows; beyond, the library's product with a 32-bit
+  result, or (where a torch has none) the own kernel 64 rows at a time."""
+  from miniinfer_amd.parts import linear as lin
+  monkeypatch.setattr(lin, "_MM_TAKES_OUT_DTYPE", [library])
+  g = torch.Generator().manual_seed(M)
+  x = torch.randn(M, 96, generator=g).bfloat16()
+  w = (torch.randn(333, 96, generator=g) * 0.1).bfloat16()
+  y = lin.linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32)
+  assert y.dtype == torch.float32 and tuple(y.shape) == (M, 333)
+  torch.testing.assert_close(y.double().cpu(), x.double() @ w.double().T, rtol=1e-4, atol=1e-3)
