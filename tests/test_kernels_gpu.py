@@ -274,7 +274,7 @@ def test_mfma_prefill_attention(nq, nkv, d, P, window, variant):
   torch.testing.assert_close(out.double().cpu(), c["want"], rtol=1.6e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("splits", [1, 3, 16])
+@pytest.mark.parametrize("splits", [1, 3, 16, 29, 40])
 @pytest.mark.parametrize("nq,nkv,d,P,window", MFMA_SHAPES)
 def test_mfma_decode_attention_any_number_of_splits(nq, nkv, d, P, window, splits):
   from miniinfer_amd.kernels import ops
