@@ -90,7 +90,7 @@ class PagedGroup:
 class StateGroup:
   need: FixedState
   layers: List[int]
-  state: Optional[torch.Tensor] = None  # [len(layers), max_requests, *shape]
+  state: Optional[torch.Tensor] = None  # [len(layers), max_requests + 1, *shape]; the last row is scratch
 
 
 @dataclass
@@ -100,7 +100,7 @@ class LayerCache:
   group: int = -1
   k: Optional[torch.Tensor] = None       # [num_pages + 1, nkv, page_size, d]
   v: Optional[torch.Tensor] = None       # [num_pages + 1, nkv, d, page_size]
-  state: Optional[torch.Tensor] = None   # [max_requests, *shape]
+  state: Optional[torch.Tensor] = None   # [max_requests + 1, *shape]; row max_requests is scratch
   page_size: int = 0
   window: Optional[int] = None
 
@@ -145,6 +145,9 @@ class CacheManager:
       else:
         raise TypeError(f"layer {i}: unknown cache need {need!r}")
     self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
+    # The state row that no request ever gets: padding entries of captured steps read and write it, as they
+    # read and write page 0 of the paged groups.
+    self.scratch_slot = max_requests
     self._slot: Dict[Hashable, int] = {}
     self._length: Dict[Hashable, int] = {}
     if allocate:
@@ -164,7 +167,7 @@ class CacheManager:
       g.k = torch.zeros((n, self.num_pages + 1, h, self.page_size, d), dtype=self.dtype, device=self.device)
       g.v = torch.zeros((n, self.num_pages + 1, h, d, self.page_size), dtype=self.dtype, device=self.device)
     for s in self.states:
-      shape = (len(s.layers), self.max_requests) + tuple(s.need.shape)
+      shape = (len(s.layers), self.max_requests + 1) + tuple(s.need.shape)
       s.state = torch.zeros(shape, dtype=s.need.dtype or self.dtype, device=self.device)
 
   def layer_cache(self, layer: int) -> LayerCache:

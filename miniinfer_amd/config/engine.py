@@ -38,7 +38,7 @@ class EngineConfig:
   enforce_eager: bool = False                 # True: never replay decode steps from HIP graphs
   enable_overlap: bool = True                 # launch a step before the last one's tokens are read back
   tune_products: bool = True                  # time own and library kernels for the model's large products once
-  eos: Optional[int] = None                   # None: from config.json
+  eos: Optional[int] = None                   # None: from generation_config.json, else from config.json
   seed: int = 0
   device: str = "cuda:0"
 

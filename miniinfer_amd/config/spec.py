@@ -100,3 +100,11 @@ class ModelSpec:
   optional_name_prefix: str = "model."  # checkpoints may leave this prefix out
   max_positions: int = 0
   init_std: float = 0.02
+  # The frame around the blocks is data too.  `kind` names the frame class in the frame registry; the default
+  # frame (embedding -> blocks -> final norm -> head) takes the variations below as plain numbers and names.
+  embedding_scale: float = 1.0        # h = E[ids] * embedding_scale
+  position_table_name: Optional[str] = None   # a learned table [max_positions, hidden] whose row of the token's
+                                      # position is added to the embedding (absolute positions)
+  logit_scale: float = 1.0            # logits = (x . head) * logit_scale
+  logit_softcap: Optional[float] = None   # then cap * tanh(logits / cap)
+  kind: str = "decoder"

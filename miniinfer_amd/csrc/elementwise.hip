@@ -11,30 +11,68 @@
 // ---------------------------------------------------------------- embedding
 // A negative id -(r + 1) stands for a token that an earlier kernel on the stream left in future[r] (the row of the
 // last step's sampling output): the engine launches a step before it has read the tokens of the one before.
+// Optional parts of the gather, for model frames that ask for them: `scale` multiplies the row, and a second
+// table `pos_table` [max_pos, H] adds the row of the token's position (learned absolute positions).
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
-                             int H, int V, const int* __restrict__ future, int num_future) {
+                             int H, int V, const int* __restrict__ future, int num_future, float scale,
+                             const T* __restrict__ pos_table, const int* __restrict__ positions, int max_pos) {
   const int t = blockIdx.x;
   int id = ids[t];
   if (id < 0 && future && -(id + 1) < num_future) id = future[-(id + 1)];
-  const bool ok = id >= 0 && id < V;
+  bool ok = id >= 0 && id < V;
   const T* row = table + (int64_t)(ok ? id : 0) * H;
+  const T* prow = nullptr;
+  if (pos_table) {
+    const int p = positions[t];
+    ok = ok && p >= 0 && p < max_pos;
+    prow = pos_table + (int64_t)(ok ? p : 0) * H;
+  }
   float* o = out + (int64_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = ok ? to_float(row[i]) : __builtin_nanf("");
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = to_float(row[i]) * scale;
+    if (prow) v += to_float(prow[i]);
+    o[i] = ok ? v : __builtin_nanf("");
+  }
 }
 
 MI_EXPORT int mi_embed(int dtype, const void* table, const int* ids, float* out, int T, int H, int V,
-                       const int* future, int num_future, hipStream_t stream) {
+                       const int* future, int num_future, float scale, const void* pos_table, const int* positions,
+                       int max_pos, hipStream_t stream) {
   MI_REQUIRE(T >= 0 && H > 0 && V > 0 && num_future >= 0, "embed: bad sizes T=%d H=%d V=%d", T, H, V);
+  MI_REQUIRE(!pos_table || (positions && max_pos > 0), "embed: a position table needs positions");
   if (T == 0) return 0;
   const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
   if (dtype == MI_DTYPE_F32)
-    embed_kernel<float><<<T, threads, 0, stream>>>((const float*)table, ids, out, H, V, future, num_future);
+    embed_kernel<float><<<T, threads, 0, stream>>>((const float*)table, ids, out, H, V, future, num_future, scale,
+                                                   (const float*)pos_table, positions, max_pos);
   else if (dtype == MI_DTYPE_BF16)
-    embed_kernel<bf16><<<T, threads, 0, stream>>>((const bf16*)table, ids, out, H, V, future, num_future);
+    embed_kernel<bf16><<<T, threads, 0, stream>>>((const bf16*)table, ids, out, H, V, future, num_future, scale,
+                                                  (const bf16*)pos_table, positions, max_pos);
   else
     MI_FAIL("embed: unknown dtype %d", dtype);
   MI_CHECK_LAUNCH("embed");
+  return 0;
+}
+
+// ---------------------------------------------------------------- logits: scale and soft cap, in place
+// x = x * scale; with cap > 0 then x = cap * tanh(x / cap).  32-bit logits [R, V] with row stride ld.
+__global__ void logit_transform_kernel(float* __restrict__ x, int64_t ld, int V, float scale, float cap) {
+  float* row = x + (int64_t)blockIdx.y * ld;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < V; i += gridDim.x * blockDim.x) {
+    float v = row[i] * scale;
+    if (cap > 0.f) v = cap * tanhf(v / cap);
+    row[i] = v;
+  }
+}
+
+MI_EXPORT int mi_logit_transform(float* x, int64_t ld, int R, int V, float scale, float cap, hipStream_t stream) {
+  MI_REQUIRE(R >= 0 && V > 0 && ld >= V && cap >= 0.f, "logit_transform: bad sizes R=%d V=%d", R, V);
+  MI_REQUIRE(R <= 65535, "logit_transform: %d rows; the grid takes at most 65535", R);
+  if (R == 0) return 0;
+  const int bx = (V + 1023) / 1024 < 64 ? (V + 1023) / 1024 : 64;
+  logit_transform_kernel<<<dim3(bx, R), 256, 0, stream>>>(x, ld, V, scale, cap);
+  MI_CHECK_LAUNCH("logit_transform");
   return 0;
 }
 

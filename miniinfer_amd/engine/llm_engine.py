@@ -26,6 +26,7 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..config import EngineConfig, load_model_config, model_spec_of
+from ..kernels import ops
 from ..kernels.tuning import tune_products
 from ..sampling import Sampler, SamplingParams, request_seed
 from ..weights import build_model, fill_random, load_weights
@@ -74,6 +75,9 @@ class LLMEngine:
       fill_random(self.model, random_weights_seed)
     else:
       load_weights(self.model, cfg.model_path)
+    # the timed choices between own and library product kernels are process-wide and keyed by shape: an engine
+    # starts from none, so that it never inherits what an earlier engine in the process measured
+    ops.clear_product_choices()
     if cfg.tune_products and self.dtype == torch.bfloat16:
       try:
         tune_products(self.model.products())
@@ -86,7 +90,9 @@ class LLMEngine:
     self.cache = CacheManager(needs, page_size=cfg.page_size, num_pages=self.num_pages, max_requests=cfg.max_num_seqs,
                               max_model_len=self.max_model_len, dtype=self.dtype, device=self.device)
     self.runner = ModelRunner(self.model, self.cache, use_graphs=not cfg.enforce_eager)
-    eos = cfg.eos if cfg.eos is not None else getattr(self.model_config, "eos_token_id", None)
+    eos = cfg.eos if cfg.eos is not None else self._eos_of_folder(cfg.model_path)
+    if eos is None:
+      eos = getattr(self.model_config, "eos_token_id", None)
     self.eos_token_id = eos
     self.scheduler = Scheduler(self.cache, max_num_seqs=cfg.max_num_seqs,
                                max_num_batched_tokens=cfg.max_num_batched_tokens, max_model_len=self.max_model_len,
@@ -103,20 +109,53 @@ class LLMEngine:
 
   # ------------------------------------------------------------------ set-up helpers
   def _pages_from_memory(self, needs) -> int:
-    """Pages from the device memory left after the weights (the reference: utils/memory_utils.py:85-144,
-    which also holds a share back for activations)."""
+    """Pages from the device memory that is free after the weights are loaded, less the share of the device that
+    `gpu_memory_utilization` leaves alone and less what the largest step needs for its activations (the reference
+    holds back a fifth of the free memory for them, whatever the model: utils/memory_utils.py:85-144; here the
+    step's buffers are counted from the model's sizes and the token budget).  Never more pages than
+    `max_num_seqs` requests of `max_model_len` tokens can use."""
     cfg = self.config
     per_page = CacheManager.bytes_per_page(needs, cfg.page_size, self.dtype)
     cap = cfg.max_num_seqs * (-(-self.max_model_len // cfg.page_size))
     if per_page == 0:
       return max(1, cap)
     free, total = torch.cuda.mem_get_info(self.device)
-    usable = free - int(total * (1.0 - cfg.gpu_memory_utilization))
-    usable = int(usable * 0.8)
-    pages = usable // per_page - 1
+    usable = free - int(total * (1.0 - cfg.gpu_memory_utilization)) - self.activation_bytes()
+    pages = usable // per_page - 1            # page 0 of every group is the scratch page
     if pages < 2:
-      raise RuntimeError(f"not enough device memory for a cache: {free >> 20} MiB free, a page costs {per_page} bytes")
+      raise RuntimeError(f"not enough device memory for a cache: {free >> 20} MiB free, the largest step needs "
+                         f"{self.activation_bytes() >> 20} MiB, a page costs {per_page} bytes")
     return int(min(pages, cap))
+
+  def activation_bytes(self) -> int:
+    """An upper estimate of the device memory one step of the full token budget holds beside weights and cache:
+    per token two 32-bit residual rows and, in the activation dtype, the widest rows a block makes (each counted
+    twice, since the allocator keeps a freed buffer of one layer while the next layer's is made), the 32-bit logits
+    of `max_num_seqs` rows with the sampler's scratch, the pools of the captured decode steps, and 256 MiB of slack."""
+    cfg, spec = self.config, self.model.spec
+    esize = 2 if self.dtype == torch.bfloat16 else 4
+    widest = spec.hidden_size
+    for _, part, ps in self.model.named_params():
+      if len(ps.shape) == 2:
+        widest = max(widest, ps.shape[0] if ps.shape[0] != spec.vocab_size else 0)
+    T = cfg.max_num_batched_tokens
+    per_token = 2 * 4 * spec.hidden_size + 2 * esize * (2 * widest + 2 * spec.hidden_size)
+    logits = 3 * 4 * spec.vocab_size * min(cfg.max_num_seqs, 256)
+    graphs = 0 if cfg.enforce_eager else 256 * (per_token + 4 * spec.vocab_size)
+    return int(T * per_token + logits + graphs + (256 << 20))
+
+  @staticmethod
+  def _eos_of_folder(path: str):
+    """`eos_token_id` of the folder's generation_config.json: one id or a list of them; None without the file."""
+    gj = os.path.join(path, "generation_config.json") if path and os.path.isdir(path) else None
+    if not gj or not os.path.isfile(gj):
+      return None
+    import json
+    with open(gj) as f:
+      eos = json.load(f).get("eos_token_id")
+    if isinstance(eos, list):
+      return [int(t) for t in eos] or None
+    return None if eos is None else int(eos)
 
   @staticmethod
   def _load_tokenizer(path: str):

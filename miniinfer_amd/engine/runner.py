@@ -59,6 +59,8 @@ class StepContext:
     self._cache: CacheManager = None
     self._device = None
     self._work: Dict[int, torch.Tensor] = {}
+    self._spare_host: Optional[torch.Tensor] = None   # pinned int32 room behind the step's arrays (work lists)
+    self._spare_used = 0
     self._scratch: Dict[str, torch.Tensor] = {}
 
   def layer_cache(self, layer: int) -> LayerCache:
@@ -72,7 +74,17 @@ class StepContext:
       items = [(b, i) for b in range(self.num_multi) for i in range(-(-self.q_lens[b] // tokens_per_block))]
       # the blocks with the most keys first: they take longest
       items.sort(key=lambda it: -(self.kv_lens[it[0]] - self.q_lens[it[0]] + (it[1] + 1) * tokens_per_block))
-      w = torch.tensor(items, dtype=torch.int32).reshape(-1, 2).to(self._device, non_blocking=True)
+      n = 2 * len(items)
+      if self._spare_host is not None and self._spare_used + n <= self._spare_host.numel():
+        # from the step's pinned staging buffer, so that the copy is queued like the rest of the step's inputs
+        host = self._spare_host[self._spare_used:self._spare_used + n]
+        self._spare_used += n
+        host.copy_(torch.tensor(items, dtype=torch.int32).reshape(-1))
+        w = torch.empty(n, dtype=torch.int32, device=self._device)
+        w.copy_(host, non_blocking=True)
+        w = w.view(-1, 2)
+      else:
+        w = torch.tensor(items, dtype=torch.int32).reshape(-1, 2).to(self._device, non_blocking=True)
       self._work[tokens_per_block] = w
     return w
 
@@ -125,6 +137,7 @@ class _DecodeGraph:
   def __init__(self, runner: "ModelRunner", B: int, W: int):
     self.B, self.W = B, W
     cache = runner.cache
+    self.scratch_slot = cache.scratch_slot
     G = len(cache.paged)
     self.layout = _Layout(T=B, B=B, R=B, G=G, W=W)
     # two pinned staging buffers, used in turn: the copy of one step may still be queued on the stream while the
@@ -212,12 +225,13 @@ class _DecodeGraph:
     return best
 
   def fill_padding(self, first: int) -> None:
-    """Entries first.. are padding: token 0 at position 0 of a request of one key in the scratch page."""
+    """Entries first.. are padding: token 0 at position 0 of a request of one key in the scratch page, whose
+    fixed-size state is the scratch row that no request ever holds."""
     h = self.host
     h["token_ids"][first:] = 0
     h["positions"][first:] = 0
     h["kv_len"][first:] = 1
-    h["req_slots"][first:] = 0
+    h["req_slots"][first:] = self.scratch_slot
     G, B, W = self.layout.G, self.B, self.W
     h["slots"].reshape(G, B)[:, first:] = 0
     h["tables"].reshape(G, B, W)[:, first:, :] = 0
@@ -245,9 +259,15 @@ class ModelRunner:
     self.cache = cache
     self.device = model.ctx.device
     self.vocab_size = model.spec.vocab_size
-    self.use_graphs = use_graphs and self.device.type == "cuda"
+    # a part that cannot be recorded into a graph (one that reads device values on the host, say) declares
+    # `capturable = False`; the steps of a model that holds such a part always run eagerly
+    self.use_graphs = use_graphs and self.device.type == "cuda" and model.is_capturable()
     self.check_graphs = True      # replay every captured step against its eager result before it is used
-    self._staging: Optional[torch.Tensor] = None
+    # two pinned staging buffers for eager steps, used in turn, each with the event of the copy that last read it:
+    # a step's copy may still be queued on the stream while the host lays out the next step
+    self._staging: List[Optional[torch.Tensor]] = [None, None]
+    self._staging_done: List[Optional[torch.cuda.Event]] = [None, None]
+    self._staging_turn = 0
     self._allow_future = False
     self._graphs: Dict[tuple, _DecodeGraph] = {}
     # Tokens of the last step's sampling output, by row.  A token id -(r + 1) in a step's entries stands for
@@ -257,10 +277,17 @@ class ModelRunner:
 
   # ------------------------------------------------------------------ host side of a step
   def _stage(self, n: int) -> torch.Tensor:
-    if self._staging is None or self._staging.numel() < n:
+    """The pinned buffer to lay the next eager step out in: the one of the two that was not used last, once the
+    copy that last read it is done (that copy was queued two steps back, so the host practically never waits)."""
+    self._staging_turn ^= 1
+    t = self._staging_turn
+    if self._staging_done[t] is not None:
+      self._staging_done[t].synchronize()
+      self._staging_done[t] = None
+    if self._staging[t] is None or self._staging[t].numel() < n:
       cap = max(4096, 1 << (n - 1).bit_length())
-      self._staging = torch.empty(cap, dtype=torch.int32, pin_memory=(self.device.type == "cuda"))
-    return self._staging
+      self._staging[t] = torch.empty(cap, dtype=torch.int32, pin_memory=(self.device.type == "cuda"))
+    return self._staging[t]
 
   def _plan(self, entries: Sequence[StepEntry]):
     """Checks the entries, grows the requests' page tables (all or nothing), and orders the entries: those
@@ -334,17 +361,23 @@ class ModelRunner:
     rows = [first_row[i] + w for i, e in enumerate(entries) for w in e.want]
     W = max(1, max(-(-kv // cache.page_size) for kv in kv_lens))
     lay = _Layout(T=T, B=B, R=len(rows), G=len(cache.paged), W=W)
-    stage = self._stage(lay.total)
+    spare = 2 * (T // 4 + B + 1)           # room for a list of (entry, block of >= 4 query tokens)
+    stage = self._stage(lay.total + spare)
     host = lay.views(stage.numpy())
     self._fill(host, lay, entries, order, q_lens, starts, kv_lens)
     host["logit_rows"][:] = rows
     dev = torch.empty(lay.total, dtype=torch.int32, device=self.device)
-    dev.copy_(stage[:lay.total], non_blocking=False)
+    dev.copy_(stage[:lay.total], non_blocking=True)
+    if self.device.type == "cuda":
+      self._staging_done[self._staging_turn] = torch.cuda.Event()
+      self._staging_done[self._staging_turn].record()
     ctx = lay.context(dev, cache, self.device)
     ctx.q_lens, ctx.kv_lens = q_lens, kv_lens
     ctx.num_multi = sum(1 for n in q_lens if n > 1)
     ctx.max_q_len, ctx.max_kv_len = max(q_lens), max(kv_lens)
     ctx.future_tokens = self.future_tokens
+    if self.device.type == "cuda":
+      ctx._spare_host = stage[lay.total:lay.total + spare]
     return ctx, order, kv_lens
 
   # ------------------------------------------------------------------ the step
@@ -388,6 +421,8 @@ class ModelRunner:
   def _step_eager(self, entries: Sequence[StepEntry]) -> torch.Tensor:
     ctx, order, kv_lens = self.build_context(entries)
     logits = self.model.forward(ctx)
+    if ctx._spare_used:                     # further copies out of the staging buffer were queued by the layers
+      self._staging_done[self._staging_turn].record()
     for i, kv in zip(order, kv_lens):
       self.cache.commit(entries[i].req, kv)
     return logits

@@ -27,7 +27,7 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, Dict, List, Optional, Sequence
+from typing import Deque, Dict, Iterable, List, Optional, Sequence, Union
 
 from ..sampling.params import SamplingParams
 
@@ -109,7 +109,7 @@ class ScheduledStep:
 
 class Scheduler:
   def __init__(self, cache, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
-               enable_chunked_prefill: bool = True, eos_token_id: Optional[int] = None):
+               enable_chunked_prefill: bool = True, eos_token_id: Union[int, Iterable[int], None] = None):
     self.cache = cache
     self.max_num_seqs = max_num_seqs
     self.max_num_batched_tokens = max_num_batched_tokens
@@ -118,11 +118,28 @@ class Scheduler:
     self.eos_token_id = eos_token_id
     self.waiting: Deque[Request] = deque()
     self.running: List[Request] = []      # in order of admission
-    self.finished: List[Request] = []
+    self.finished: Deque[Request] = deque(maxlen=1024)   # the last requests that finished (a log, not a queue)
+    self.num_finished = 0
     self.num_preemptions = 0
     self.num_unresolved = 0               # sampled tokens launched and not yet written in
     self._draining: List[Request] = []    # finished, pages still held until their last token is written in
     self._retired_unadmitted: List[Request] = []
+
+  @property
+  def eos_token_id(self):
+    """One id, several, or None; any of them ends a request that does not ignore it (a generation_config.json
+    may list more than one)."""
+    return self._eos
+
+  @eos_token_id.setter
+  def eos_token_id(self, eos) -> None:
+    self._eos = eos
+    if eos is None:
+      self.eos_token_ids = frozenset()
+    elif isinstance(eos, int):
+      self.eos_token_ids = frozenset([eos])
+    else:
+      self.eos_token_ids = frozenset(int(t) for t in eos)
 
   # ------------------------------------------------------------------ requests in
   def add(self, req: Request) -> None:
@@ -170,6 +187,19 @@ class Scheduler:
     while True:
       need = sum(self._pages_for(r, r.num_tokens) for r in decoding)
       if need <= free or not decoding:
+        break
+      if self._draining:
+        # Finished requests hold pages until their last token is written in, one call from now.  The decodes
+        # that need a new page sit this step out (the most recently admitted first) rather than cost a running
+        # request its whole cache.
+        short = need - free
+        for r in reversed(list(decoding)):
+          if short <= 0:
+            break
+          n = self._pages_for(r, r.num_tokens)
+          if n > 0:
+            decoding.remove(r)
+            short -= n
         break
       victim = self.running[-1]
       self._preempt(victim)
@@ -277,8 +307,9 @@ class Scheduler:
       if e.output_index < len(r.outputs):          # else: dropped after an earlier end-of-sequence token
         tok = int(sampled[r.number])
         r.set_output(e.output_index, tok)
-        if not r.params.ignore_eos and self.eos_token_id is not None and tok == self.eos_token_id:
-          r.finish_reason = "eos"
+        is_eos = not r.params.ignore_eos and tok in self.eos_token_ids
+        if is_eos or tok in r.params.stop_token_ids:
+          r.finish_reason = "eos" if is_eos else "stop"
           r.truncate_outputs(e.output_index + 1)
           if r in self.running:
             self.running.remove(r)
@@ -295,6 +326,7 @@ class Scheduler:
         else:
           continue
         self.finished.append(r)
+        self.num_finished += 1
         done.append(r)
     return done
 

@@ -76,24 +76,51 @@ def build_dirs() -> List[str]:
   return dirs
 
 
+def _private_temp_dir(d: str) -> bool:
+  """The per-user folder under the temp dir is only used when it belongs to this user and nobody else can write to
+  it: a library is loaded from it, and another user of the machine could have made the folder first."""
+  uid = os.getuid() if hasattr(os, "getuid") else None
+  try:
+    os.makedirs(d, mode=0o700, exist_ok=True)
+    st = os.lstat(d)
+  except OSError:
+    return False
+  import stat
+  if not stat.S_ISDIR(st.st_mode) or (uid is not None and st.st_uid != uid) or (st.st_mode & 0o022):
+    return False
+  return True
+
+
+def _usable(d: str) -> bool:
+  """Whether built objects may be looked for in `d`: the in-tree folder and an explicitly named one always, the
+  shared temp dir's folder only when it is this user's own."""
+  return not d.startswith(tempfile.gettempdir() + os.sep) or d == os.environ.get("MINIINFER_AMD_BUILD_DIR") \
+      or (os.path.isdir(d) and _private_temp_dir(d))
+
+
 def _writable_dir() -> str:
   for d in build_dirs():
     try:
-      os.makedirs(d, exist_ok=True)
+      if d.startswith(tempfile.gettempdir() + os.sep) and d != os.environ.get("MINIINFER_AMD_BUILD_DIR"):
+        if not _private_temp_dir(d):
+          continue
+      else:
+        os.makedirs(d, exist_ok=True)
       fd, probe = tempfile.mkstemp(prefix=".probe-", dir=d)
       os.close(fd)
       os.unlink(probe)
       return d
     except OSError:
       continue
-  raise BuildError(f"no writable folder for built kernels among {build_dirs()}")
+  raise BuildError(f"no writable folder for built kernels among {build_dirs()} (a folder under the temp dir is "
+                   "used only if it belongs to this user and no one else can write to it)")
 
 
 def find_built(name: str, defines: Sequence[Tuple[str, object]] = ()) -> Optional[str]:
   fn = _tag(name, defines) + ".so"
   for d in build_dirs():
     p = os.path.join(d, fn)
-    if os.path.isfile(p):
+    if os.path.isfile(p) and _usable(d):
       return p
   return None
 

@@ -71,7 +71,9 @@ def _f32(name, t, n=None):
 
 _SIGS = {
   "elementwise": {
-    "mi_embed": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
+    "mi_embed": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p,
+                 c_void_p, c_int, c_void_p],
+    "mi_logit_transform": [c_void_p, c_int64, c_int, c_int, c_float, c_float, c_void_p],
     "mi_add_rmsnorm": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                        c_void_p],
     "mi_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -158,21 +160,44 @@ def _check_pages(what, k_pages, v_pages, nkv, d, dtype):
 
 # ----------------------------------------------------------------------------- embedding
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor,
-          future: Optional[torch.Tensor] = None) -> torch.Tensor:
-  """out[t, :] = float32(table[ids[t], :]).  An id outside the table gives a row of NaN.  With `future` (int32),
-  an id -(r + 1) is replaced by future[r] as it stands when the kernel runs."""
-  _dev(table, ids, out, future)
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, future: Optional[torch.Tensor] = None,
+          scale: float = 1.0, pos_table: Optional[torch.Tensor] = None,
+          positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+  """out[t, :] = float32(table[ids[t], :]) * scale (+ pos_table[positions[t], :]).  An id or a position outside
+  its table gives a row of NaN.  With `future` (int32), an id -(r + 1) is replaced by future[r] as it stands when
+  the kernel runs."""
+  _dev(table, ids, out, future, pos_table, positions)
   _i32("future", future)
   V, H = table.shape
   T = ids.numel()
   _contig("table", table)
   _i32("ids", ids)
   _f32("out", out, T * H)
+  max_pos = 0
+  if pos_table is not None:
+    _contig("pos_table", pos_table)
+    if pos_table.dtype != table.dtype or pos_table.dim() != 2 or pos_table.shape[1] != H:
+      raise KernelError(f"embed: the position table {tuple(pos_table.shape)} {pos_table.dtype} does not fit rows "
+                        f"of {H} {table.dtype}")
+    _i32("positions", positions, T)
+    max_pos = pos_table.shape[0]
   lib = _lib("elementwise")
   _check(lib, lib.mi_embed(dtype_code(table.dtype), _ptr(table), _ptr(ids), _ptr(out), T, H, V, _ptr(future),
-                           0 if future is None else future.numel(), _stream()))
+                           0 if future is None else future.numel(), float(scale), _ptr(pos_table),
+                           _ptr(positions) if pos_table is not None else None, max_pos, _stream()))
   return out
+
+
+def logit_transform(logits: torch.Tensor, scale: float = 1.0, softcap: float = 0.0) -> torch.Tensor:
+  """In place on float32 logits [R, V]: x = x * scale, then (softcap > 0) x = softcap * tanh(x / softcap)."""
+  _dev(logits)
+  if logits.dtype != torch.float32 or logits.dim() != 2 or (logits.shape[1] > 1 and logits.stride(1) != 1):
+    raise KernelError("logit_transform: logits must be float32 [R, V] with dense rows")
+  R, V = logits.shape
+  lib = _lib("elementwise")
+  _check(lib, lib.mi_logit_transform(_ptr(logits), logits.stride(0) if R > 1 else V, R, V, float(scale),
+                                     float(softcap), _stream()))
+  return logits
 
 
 # ----------------------------------------------------------------------------- norms

@@ -20,6 +20,8 @@ Mixer           `cache_requirement()` -> PagedKV | FixedState | None;
                 `forward(x [T, hidden], ctx: StepContext, cache: LayerCache) -> [T, hidden]`.
 FeedForward     `forward(x [T, hidden], ctx) -> [T, hidden]`.
 Block           `forward(h, residual, ctx, cache) -> (h, residual)`.
+Frame           the whole model around the blocks (`ModelSpec.kind`): `forward(ctx) -> float32 logits
+                [wanted rows, vocab]`, `cache_needs()`, `cache_index(run)`, `spec`, `ctx`.
 """
 
 from __future__ import annotations
@@ -94,6 +96,15 @@ class BuildContext:
 class Part:
   """Base of every part: owns tensors, may have children."""
 
+  # Whether the part's forward pass can be recorded into a HIP graph: everything it does is queued on the current
+  # stream from values the host already has.  A part that reads device values on the host (`.tolist()`, `.item()`),
+  # or launches a number of kernels that depends on them, sets this to False; steps of a model that holds such a
+  # part are never captured.
+  capturable = True
+
+  def is_capturable(self) -> bool:
+    return bool(self.capturable) and all(child.is_capturable() for _, child in self.children())
+
   def param_specs(self) -> List[ParamSpec]:
     return []
 
@@ -149,6 +160,7 @@ POSITIONS = Registry("position encoding")
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 BLOCKS = Registry("block")
+FRAMES = Registry("model frame")
 
 
 def register_norm(kind, cls): NORMS.register(kind, cls)
@@ -156,3 +168,4 @@ def register_position(kind, cls): POSITIONS.register(kind, cls)
 def register_mixer(kind, cls): MIXERS.register(kind, cls)
 def register_feed_forward(kind, cls): FEED_FORWARDS.register(kind, cls)
 def register_block(kind, cls): BLOCKS.register(kind, cls)
+def register_frame(kind, cls): FRAMES.register(kind, cls)

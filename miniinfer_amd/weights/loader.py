@@ -22,7 +22,7 @@ import torch
 
 from ..config import load_model_config, model_spec_of
 from ..config.spec import ModelSpec
-from ..parts import BuildContext, DecoderModel, ParamSpec, Part
+from ..parts import FRAMES, BuildContext, DecoderModel, ParamSpec, Part
 from .safetensors_io import SafetensorsFile, list_safetensors
 
 
@@ -77,7 +77,8 @@ def expected_tensors(model: DecoderModel) -> Dict[str, _Target]:
 
 
 def build_model(spec: ModelSpec, dtype: torch.dtype, device) -> DecoderModel:
-  return DecoderModel(spec, BuildContext(device=torch.device(device), dtype=dtype))
+  """The model frame that `spec.kind` names, with its blocks and parts, without tensors."""
+  return FRAMES.build(spec, BuildContext(device=torch.device(device), dtype=dtype))
 
 
 def load_weights(model: DecoderModel, model_dir: str) -> None:

@@ -16,7 +16,7 @@ from typing import Dict, List, Tuple
 import torch
 
 from ..config import model_spec_of
-from ..parts import BuildContext, DecoderModel
+from ..parts import FRAMES, BuildContext, DecoderModel
 from .loader import storage_dtype
 from .safetensors_io import write_safetensors
 
@@ -35,7 +35,7 @@ def _draw(shape, init: str, std: float, gen: torch.Generator, device) -> torch.T
 def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16) -> List[Tuple[str, torch.Tensor]]:
   """(checkpoint name, tensor) for every tensor of the architecture, drawn on the CPU."""
   spec = model_spec_of(config)
-  model = DecoderModel(spec, BuildContext(device=torch.device("cpu"), dtype=dtype))
+  model = FRAMES.build(spec, BuildContext(device=torch.device("cpu"), dtype=dtype))
   gen = torch.Generator(device="cpu")
   gen.manual_seed(seed)
   out = []

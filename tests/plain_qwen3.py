@@ -88,14 +88,30 @@ def apply_rope_neox(x: torch.Tensor, ang: torch.Tensor) -> torch.Tensor:
   return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), dim=-1)
 
 
-def causal_mask(L: int, S: int, dtype=torch.float32) -> torch.Tensor:
+def causal_mask(L: int, S: int, dtype=torch.float32, window: Optional[int] = None) -> torch.Tensor:
   """Additive mask [L, S], bottom-right aligned: query i sees keys j <= i + (S - L).
-  miniinfer/layers/attention.py:112-128."""
+  miniinfer/layers/attention.py:112-128.  With `window` (no counterpart in the reference, which reads no
+  sliding-window key of config.json) the query at position p = i + (S - L) sees the `window` keys
+  p - window < j <= p, itself included."""
   i = torch.arange(L)[:, None]
   j = torch.arange(S)[None, :]
   m = torch.zeros(L, S, dtype=dtype)
   m[j > i + (S - L)] = -math.inf
+  if window is not None:
+    m[j <= i + (S - L) - window] = -math.inf
   return m
+
+
+def layer_window(cfg: dict, i: int) -> Optional[int]:
+  """The window of layer i from the config.json keys `layer_types` ("full_attention" | "sliding_attention") and
+  `sliding_window`, or from `use_sliding_window` + `max_window_layers` (layers from that index on slide).
+  The reference ignores these keys (miniinfer/config/model/qwen3.py:16-63 reads none of them)."""
+  types = cfg.get("layer_types")
+  if types is not None:
+    return int(cfg["sliding_window"]) if types[i] == "sliding_attention" else None
+  if cfg.get("use_sliding_window") and cfg.get("sliding_window") is not None:
+    return int(cfg["sliding_window"]) if i >= int(cfg.get("max_window_layers", cfg["num_hidden_layers"])) else None
+  return None
 
 
 def grouped_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
@@ -127,7 +143,7 @@ def swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: to
 
 
 def attention_block(x: torch.Tensor, positions: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str,
-                    cfg: dict) -> torch.Tensor:
+                    cfg: dict, window: Optional[int] = None) -> torch.Tensor:
   """QKV projection (no bias), per-head RMSNorm of q and k before the rotation, rotation
   of q and k, causal grouped attention with scale d^-1/2, output projection.
   miniinfer/models/fused_qwen3.py:46-58,95-107."""
@@ -142,7 +158,7 @@ def attention_block(x: torch.Tensor, positions: torch.Tensor, w: Dict[str, torch
   ang = rope_angles(positions, d, cfg["rope_theta"], x.dtype)
   q = apply_rope_neox(q, ang)
   k = apply_rope_neox(k, ang)
-  o = grouped_attention(q, k, v, d ** -0.5, causal_mask(T, T, x.dtype))
+  o = grouped_attention(q, k, v, d ** -0.5, causal_mask(T, T, x.dtype, window))
   return o.reshape(T, nq * d) @ w[prefix + "o_proj.weight"].T
 
 
@@ -154,7 +170,8 @@ def decoder_block(h: torch.Tensor, positions: torch.Tensor, w: Dict[str, torch.T
   summed up that is this."""
   pre = f"{p}layers.{i}."
   eps = cfg["rms_norm_eps"]
-  a = attention_block(rms_norm(h, w[pre + "input_layernorm.weight"], eps), positions, w, pre + "self_attn.", cfg)
+  a = attention_block(rms_norm(h, w[pre + "input_layernorm.weight"], eps), positions, w, pre + "self_attn.", cfg,
+                      layer_window(cfg, i))
   h = h + a
   m = swiglu(rms_norm(h, w[pre + "post_attention_layernorm.weight"], eps),
              w[pre + "mlp.gate_proj.weight"], w[pre + "mlp.up_proj.weight"], w[pre + "mlp.down_proj.weight"])

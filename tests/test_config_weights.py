@@ -183,3 +183,69 @@ def test_safetensors_reader_refuses_broken_files(tmp_path):
   (tmp_path / "tiny.safetensors").write_bytes(b"abc")
   with pytest.raises(ValueError, match="not a safetensors"):
     SafetensorsFile(str(tmp_path / "tiny.safetensors"))
+
+
+def test_eos_of_generation_config(tmp_path):
+  """generation_config.json names the end-of-sequence id (one or several); without the file there is none."""
+  from miniinfer_amd.engine.llm_engine import LLMEngine
+  d = tmp_path / "m"
+  d.mkdir()
+  assert LLMEngine._eos_of_folder(str(d)) is None
+  (d / "generation_config.json").write_text(json.dumps({"eos_token_id": [7, 9], "temperature": 0.6}))
+  assert LLMEngine._eos_of_folder(str(d)) == [7, 9]
+  (d / "generation_config.json").write_text(json.dumps({"eos_token_id": 11}))
+  assert LLMEngine._eos_of_folder(str(d)) == 11
+  (d / "generation_config.json").write_text(json.dumps({"do_sample": True}))
+  assert LLMEngine._eos_of_folder(str(d)) is None
+
+
+def test_sampling_params_checks():
+  from miniinfer_amd import SamplingParams
+  sp = SamplingParams(stop_token_ids=(3, 5))
+  assert sp.stop_token_ids == [3, 5] and SamplingParams().stop_token_ids == []
+  for bad in (dict(temperature=-1), dict(max_tokens=0), dict(top_k=-1), dict(top_p=0.0), dict(stop_token_ids=[-2])):
+    with pytest.raises(ValueError):
+      SamplingParams(**bad)
+
+
+def test_built_kernels_are_not_loaded_from_a_folder_others_can_write(tmp_path, monkeypatch):
+  """The fallback folder for built kernels lies under the shared temp dir: it is used only when it belongs to
+  this user and nobody else may write to it."""
+  import tempfile
+  from miniinfer_amd.kernels import jit
+  monkeypatch.setattr(tempfile, "tempdir", str(tmp_path))
+  shared = tmp_path / "shared"
+  shared.mkdir()
+  os.chmod(shared, 0o777)
+  assert not jit._private_temp_dir(str(shared))
+  mine = tmp_path / "mine"
+  assert jit._private_temp_dir(str(mine)) and (os.stat(mine).st_mode & 0o777) == 0o700
+  link = tmp_path / "link"
+  os.symlink(shared, link)
+  assert not jit._private_temp_dir(str(link))
+  # the fallback of build_dirs() is refused as a place to write when someone else prepared it
+  monkeypatch.delenv("MINIINFER_AMD_BUILD_DIR", raising=False)
+  fallback = jit.build_dirs()[-1]
+  assert fallback.startswith(str(tmp_path))
+  os.makedirs(fallback)
+  os.chmod(fallback, 0o777)
+  assert not jit._usable(fallback)
+
+
+def test_model_frame_options_are_data_of_the_spec():
+  """The frame around the blocks (embedding factor, learned positions, logit factor and cap) is chosen by fields of
+  the spec, and another frame class by its kind."""
+  import dataclasses
+  from miniinfer_amd.parts import FRAMES, BuildContext
+  spec = model_spec_of(Qwen3Config.from_dict(tm.TINY_A))
+  assert spec.kind == "decoder" and spec.embedding_scale == 1.0 and spec.logit_softcap is None
+  spec2 = dataclasses.replace(spec, position_table_name="model.positions.weight", embedding_scale=8.0,
+                              logit_softcap=30.0)
+  model = FRAMES.build(spec2, BuildContext(device=torch.device("cpu"), dtype=torch.float32))
+  names = {prefix + src.name for prefix, _, ps in model.named_params() for src in ps.sources}
+  assert "model.positions.weight" in names
+  with pytest.raises(KeyError, match="model frame"):
+    FRAMES.build(dataclasses.replace(spec, kind="no_such_frame"), BuildContext(torch.device("cpu"), torch.float32))
+  with pytest.raises(ValueError, match="logit_softcap"):
+    FRAMES.build(dataclasses.replace(spec, logit_softcap=0.0), BuildContext(torch.device("cpu"), torch.float32))
+  assert model.is_capturable()

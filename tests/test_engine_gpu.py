@@ -94,7 +94,14 @@ def test_eos_and_seeded_sampling(tmp_path):
                          [SamplingParams(temperature=1.0, max_tokens=5, ignore_eos=True), sp,
                           SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True)], use_tqdm=False)
     assert mixed[1]["token_ids"] == alone
-    assert alone != first[:3] + alone[3:] or True
+    # the seed is what the draw depends on: the same seed repeats, another seed gives other tokens
+    assert eng.generate([p0], sp, use_tqdm=False)[0]["token_ids"] == alone
+    other = SamplingParams(temperature=0.8, max_tokens=12, ignore_eos=True, seed=4321)
+    assert eng.generate([p0], other, use_tqdm=False)[0]["token_ids"] != alone
+    # a request's own stop ids end it like the end-of-sequence id does, and are kept as its last token
+    out = eng.generate([p0], SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True, stop_token_ids=[first[1]]),
+                       use_tqdm=False)[0]
+    assert out["token_ids"] == first[:first.index(first[1]) + 1] and out["finish_reason"] == "stop"
 
 
 def test_unknown_option_is_an_error(tmp_path):
@@ -179,3 +186,110 @@ def test_stream_generate_yields_every_token_once_and_in_order(tmp_path):
       assert [seen[r] for r in sorted(seen, key=lambda r: int(r.split("-")[1]))] == [o["token_ids"] for o in whole]
       assert list(ended.values()) == ["max_tokens"] * 3 and eng.is_finished()
       assert eng.cache.num_free_pages() == eng.cache.num_pages
+
+
+def test_eos_comes_from_generation_config_json(tmp_path):
+  import json
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "A")
+  p0 = tm.random_tokens(cfg, 9, seed=1)
+  first = plain.greedy_generate(p0, 4, w, dict(cfg))
+  with open(tmp_path / "m" / "generation_config.json", "w") as f:
+    json.dump({"eos_token_id": [first[3], 255]}, f)
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", num_pages=32, max_num_seqs=4) as eng:
+    assert eng.eos_token_id == [first[3], 255]
+    out = eng.generate([p0], SamplingParams(temperature=0.0, max_tokens=10), use_tqdm=False)[0]
+  assert out["token_ids"] == first[:first.index(first[3]) + 1] and out["finish_reason"] == "eos"
+
+
+def test_text_prompts_go_through_the_folder_s_tokenizer(tmp_path):
+  """A tokenizer.json in the model folder (a word-level one, built here) turns text prompts into ids and the
+  generated ids back into text; without one, a text prompt is an error that says what to do."""
+  from tokenizers import Tokenizer
+  from tokenizers.models import WordLevel
+  from tokenizers.pre_tokenizers import Whitespace
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "A")
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", num_pages=32, max_num_seqs=4) as eng:
+    with pytest.raises(ValueError, match="tokenizer.json"):
+      eng.generate(["some words"], SamplingParams(max_tokens=2), use_tqdm=False)
+  vocab = {f"w{i}": i for i in range(cfg["vocab_size"])}
+  tok = Tokenizer(WordLevel(vocab, unk_token="w0"))
+  tok.pre_tokenizer = Whitespace()
+  tok.save(str(tmp_path / "m" / "tokenizer.json"))
+  ids = tm.random_tokens(cfg, 11, seed=5)
+  text = " ".join(f"w{i}" for i in ids)
+  want = plain.greedy_generate(ids, 6, w, dict(cfg))
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", num_pages=32, max_num_seqs=4) as eng:
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    outs = eng.generate([text, ids], sp, use_tqdm=False)
+    assert outs[0]["token_ids"] == want and outs[1]["token_ids"] == want
+    assert outs[0]["text"].split() == [f"w{i}" for i in want]
+    streamed = [o for o in eng.stream_generate(text, sp)]
+    assert [o.token_id for o in streamed] == want and streamed[-1].full_text.split() == [f"w{i}" for i in want]
+    assert "".join(o.delta_text for o in streamed) == streamed[-1].full_text
+
+
+def test_cache_is_sized_from_device_memory_when_no_page_count_is_given(tmp_path):
+  """Without `num_pages` the pool is what the device has left: bounded by the requests the engine may hold when
+  memory is plenty, by memory when it is not; a step of the full token budget still runs beside it."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  from miniinfer_amd.cache import CacheManager
+  cfg, w = _model(tmp_path, "B")
+  prompts = [tm.random_tokens(cfg, n, seed=80 + n) for n in (100, 9, 64)]
+  want = [plain.greedy_generate(p, 6, w, dict(cfg)) for p in prompts]
+  sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+  # plenty of memory: as many pages as max_num_seqs requests of max_model_len tokens can use
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, max_num_seqs=4, max_model_len=128) as eng:
+    assert eng.num_pages == 4 * (128 // 8) == eng.cache.num_pages
+    assert [o["token_ids"] for o in eng.generate(prompts, sp, use_tqdm=False)] == want
+  del eng
+  torch.cuda.empty_cache()
+  # memory binds: leave the engine 64 MiB beyond what the largest step needs
+  free, total = torch.cuda.mem_get_info()
+  probe = LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, max_num_seqs=256, num_pages=4)
+  act = probe.activation_bytes()
+  per_page = CacheManager.bytes_per_page(probe.model.cache_needs(), 8, torch.float32)
+  del probe
+  torch.cuda.empty_cache()
+  free, total = torch.cuda.mem_get_info()
+  room = 64 << 20
+  util = 1.0 - (free - act - room) / total
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, max_num_seqs=256,
+                 gpu_memory_utilization=util) as eng:
+    pages = eng.num_pages
+    assert pages < 256 * (256 // 8), "the test is meant to be bound by memory, not by the request limit"
+    assert 0.8 * room <= (pages + 1) * per_page <= room, (pages, per_page, room)
+    assert [o["token_ids"] for o in eng.generate(prompts, sp, use_tqdm=False)] == want
+  with pytest.raises(RuntimeError, match="not enough device memory"):
+    LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, gpu_memory_utilization=1e-3)
+
+
+@pytest.mark.parametrize("products", ["own", "library"])
+def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, products):
+  """The engine's choice between its own weight-streaming product and the library's is a matter of speed: with
+  every small product forced to either, each generated token is one the plain implementation all but ties for."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  from miniinfer_amd.kernels import ops
+  cfg, w = _model(tmp_path, "B", dtype=torch.bfloat16)
+  prompts = [tm.random_tokens(cfg, n, seed=90 + n) for n in (7, 60, 33)]
+  with LLMEngine(model=str(tmp_path / "m"), dtype="bfloat16", page_size=8, num_pages=64, max_num_seqs=4,
+                 tune_products=False, max_num_batched_tokens=48) as eng:
+    before = ops.library_products_run()[0]
+    if products == "own":
+      with ops.own_products_only():
+        outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
+    else:
+      for rows in ops.TUNE_ROWS:
+        for m in eng.model.products():
+          ops.set_product_choice(rows, m[0].shape[0], m[0].shape[1], m[1], own=False)
+      outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
+      ops.clear_product_choices()
+    ran_library = ops.library_products_run()[0] - before
+    assert (ran_library > 0) == (products == "library")
+  for p, o in zip(prompts, outs):
+    hist = list(p)
+    for tok in o["token_ids"]:
+      lg = plain.qwen3_logits(hist, w, dict(cfg))[-1]
+      assert lg[tok] >= lg.max() - 0.03 * lg.abs().max(), f"token {tok} is not near the plain top"
+      hist.append(tok)

@@ -160,3 +160,32 @@ def test_sampling_distribution():
   assert (p > 0).tolist() == [True, True, False, False]
   p = plain.sampling_distribution(lg, 0.01)
   assert p[0] > 0.999999
+
+
+def test_window_mask_reduces_to_the_causal_mask_and_to_one_key():
+  """A window at least as long as the sequence changes nothing; a window of one key leaves each query its own
+  key, so attention returns that key's value; in between, query p sees exactly keys p - window + 1 .. p."""
+  L, S = 5, 9
+  assert torch.equal(plain.causal_mask(L, S, window=S), plain.causal_mask(L, S))
+  m = plain.causal_mask(L, S, window=3)
+  for i in range(L):
+    p = i + S - L
+    assert [j for j in range(S) if m[i, j] == 0] == [j for j in range(p - 2, p + 1) if j >= 0]
+  g = torch.Generator().manual_seed(3)
+  q, k, v = (torch.randn(6, 2, 8, generator=g) for _ in range(3))
+  out = plain.grouped_attention(q, k, v, 0.3, plain.causal_mask(6, 6, window=1))
+  assert torch.allclose(out, v, atol=1e-6)
+
+
+def test_layer_windows_follow_the_config_keys():
+  cfg = dict(tm.TINY_D)
+  assert [plain.layer_window(cfg, i) for i in range(4)] == [None, 40, 40, None]
+  old = dict(tm.TINY_A, use_sliding_window=True, sliding_window=7, max_window_layers=1)
+  assert [plain.layer_window(old, i) for i in range(2)] == [None, 7]
+  assert plain.layer_window(dict(tm.TINY_A), 0) is None
+  # a sliding layer changes the logits only from the first position that has more keys than the window
+  w = tm.random_weights(cfg, 1, std=0.05)
+  toks = tm.random_tokens(cfg, 60, 2)
+  a = plain.qwen3_logits(toks, w, cfg)
+  b = plain.qwen3_logits(toks, w, dict(cfg, layer_types=["full_attention"] * 4))
+  assert torch.allclose(a[:40], b[:40], atol=1e-5) and (a[40:] - b[40:]).abs().max() > 1e-3

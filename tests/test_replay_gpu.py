@@ -16,7 +16,12 @@ import trace_tools as tt
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [5, 17, 33, 100, 128, 64], "B": [1, 9, 40, 64, 100, 200, 33], "C": [300, 77, 513, 2, 150]}
+LENGTHS = {"A": [5, 17, 33, 100, 128, 64], "B": [1, 9, 40, 64, 100, 200, 33], "C": [300, 77, 513, 2, 150],
+           "D": [130, 45, 300, 7, 81]}
+# The configuration with sliding windows, in 32-bit: attention that picks few keys shows a window's edge.  (In
+# bfloat16 the rounding of queries and keys grows with the scores too, 17% of the largest logit at this factor;
+# there the plain weights stand, with which a window that is off by one key still moves the logits by 9%.)
+SHARPEN = {("D", "float32"): 2.5}
 FP32_TOL = 1e-4
 
 
@@ -42,11 +47,18 @@ def _replay(folder, dtype, steps, requests, page_size, max_tokens):
   return outs
 
 
+_SEEN = {"max": 0.0, "mean": 0.0}
+
+
 def _bf16_check(got, want, what):
   scale = np.abs(want).max()
   err = np.abs(got - want)
-  assert err.max() <= 0.04 * scale, f"{what}: max err {err.max():.4g} vs scale {scale:.4g}"
-  assert err.mean() <= 0.006 * scale, f"{what}: mean err {err.mean():.4g} vs scale {scale:.4g}"
+  _SEEN["max"], _SEEN["mean"] = max(_SEEN["max"], err.max() / scale), max(_SEEN["mean"], err.mean() / scale)
+  print(f"bf16 {what}: max {err.max() / scale:.5f} mean {err.mean() / scale:.5f} of the largest logit; "
+        f"worst so far {_SEEN['max']:.5f} / {_SEEN['mean']:.5f}", flush=True)
+  # seen on an MI355X over all configurations and regimes: at most 0.8% (max) and 0.13% (mean) of the largest logit
+  assert err.max() <= 0.015 * scale, f"{what}: max err {err.max():.4g} vs scale {scale:.4g}"
+  assert err.mean() <= 0.0025 * scale, f"{what}: mean err {err.mean():.4g} vs scale {scale:.4g}"
   # the top token agrees wherever the plain margin is clear
   top = want.argmax(-1)
   srt = np.sort(want, -1)
@@ -63,11 +75,11 @@ REGIMES = {
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("regime", list(REGIMES))
 def test_regime(tmp_path, name, dtype, regime):
   file_dtype = torch.float32 if dtype == "float32" else torch.bfloat16
-  cfg, w = tm.make_model(str(tmp_path / "m"), name, seed=7, dtype=file_dtype, std=0.05)
+  cfg, w = tm.make_model(str(tmp_path / "m"), name, seed=7, dtype=file_dtype, std=0.05, sharpen=SHARPEN.get((name, dtype), 1.0))
   requests = _requests(name, cfg)
   want = _plain_logits(cfg, w, requests)
   steps = REGIMES[regime](requests)

@@ -238,3 +238,77 @@ def test_an_end_of_sequence_token_found_late_drops_the_token_launched_after_it()
   assert other.outputs == expected(other.prompt, 9)
   assert cache.num_free_pages() == 100 and cache.num_free_slots() == 4
   assert [q.number for q in sched.finished].count(0) == 1
+
+
+def test_a_decode_short_of_a_page_waits_for_a_finished_request_instead_of_preempting():
+  """Results arrive one step late.  Request a reaches max_tokens while its last token is still outstanding, so its
+  pages come back one call later; request b needs a new page for its next decoded token and none is free.  b must
+  sit the step out, not be preempted and recomputed."""
+  P = 8
+  cache, sched = make(pages=4, P=P, max_seqs=2, budget=64)
+  a = _req(0, 8, 2)           # one page; its 2nd token (the 9th) opens a second one
+  b = _req(1, 15, 4)          # two pages; its 2nd decoded token (the 17th) needs a third
+  sched.add(a)
+  sched.add(b)
+
+  def launch():
+    plan = sched.schedule()
+    if plan is None:
+      return None
+    for e in plan.entries:
+      cache.grow(e.request.number, e.start + e.num_tokens)
+      cache.commit(e.request.number, e.start + e.num_tokens)
+    sched.advance(plan)
+    return plan
+
+  def settle(plan):
+    # by now every earlier placeholder of the request has been written in
+    sched.resolve(plan, {e.request.number: fake_next(e.request.tokens[:e.start + e.num_tokens])
+                         for e in plan.entries if e.samples})
+    cache.check()
+
+  p0 = launch()
+  assert sorted((e.request.number, e.num_tokens) for e in p0.entries) == [(0, 8), (1, 15)]
+  assert cache.num_free_pages() == 1
+  p1 = launch()               # launched against placeholders: a's 9th token takes the last page, b's 16th fits
+  assert cache.num_free_pages() == 0 and a.finish_reason == "max_tokens" and a not in sched.running
+  settle(p0)
+  p2 = launch()               # b's 17th token needs a page; the only pages to come are a's, one call from now
+  assert p2 is None and sched.num_preemptions == 0 and b in sched.running and b.num_computed == 16
+  settle(p1)                  # a's last token is in: its two pages are free
+  assert cache.num_free_pages() == 2
+  p3 = launch()
+  assert [(e.request.number, e.start, e.num_tokens) for e in p3.entries] == [(1, 16, 1)]
+  settle(p3)
+  while sched.has_unfinished():
+    settle(launch())
+  assert sched.num_preemptions == 0 and b.num_preemptions == 0
+  assert a.outputs == expected(a.prompt, 2) and b.outputs == expected(b.prompt, 4)
+  assert cache.num_free_pages() == 4 and cache.num_free_slots() == 2
+
+
+def test_stop_token_ids_end_a_request_and_several_eos_ids_are_honoured():
+  prompt = [2, 7, 1, 8]
+  want = expected(prompt, 8)
+  cache, sched = make(pages=50, eos=[want[5], 999999])
+  r = Request(number=0, request_id="r0", prompt=list(prompt),
+              params=SamplingParams(temperature=0.0, max_tokens=8, stop_token_ids=[want[3]]))
+  run(cache, sched, [r])
+  assert r.outputs == want[:want.index(want[3]) + 1] and r.finish_reason == "stop"
+  r = Request(number=1, request_id="r1", prompt=list(prompt), params=SamplingParams(temperature=0.0, max_tokens=8))
+  run(cache, sched, [r])
+  assert r.outputs == want[:want.index(want[5]) + 1] and r.finish_reason == "eos"
+  # ignore_eos switches the end-of-sequence ids off, not the request's own stop ids
+  r = Request(number=2, request_id="r2", prompt=list(prompt),
+              params=SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True, stop_token_ids=[want[6]]))
+  run(cache, sched, [r])
+  assert r.outputs == want[:want.index(want[6]) + 1] and r.finish_reason == "stop"
+  assert sched.num_finished == 3 and cache.num_free_pages() == 50
+
+
+def test_the_log_of_finished_requests_is_bounded():
+  cache, sched = make(pages=50)
+  n = sched.finished.maxlen + 10
+  for i in range(0, n, 4):
+    run(cache, sched, [_req(j, 3, 1) for j in range(i, min(n, i + 4))])
+  assert sched.num_finished == n and len(sched.finished) == sched.finished.maxlen

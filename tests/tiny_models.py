@@ -22,8 +22,14 @@ TINY_C = dict(  # no size a power of two: 3 kv heads, head 48, vocab 500, long p
   num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=3, head_dim=48, hidden_act="silu",
   max_position_embeddings=2048, rms_norm_eps=3e-6, rope_theta=500000.0, tie_word_embeddings=False,
   attention_bias=False, rope_scaling=None)
-PAGE_SIZE = {"A": 16, "B": 8, "C": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+TINY_D = dict(  # sliding windows in the two middle layers, one kv head, head 64, tied head
+  architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=320, hidden_size=128, intermediate_size=96,
+  num_hidden_layers=4, num_attention_heads=4, num_key_value_heads=1, head_dim=64, hidden_act="silu",
+  max_position_embeddings=512, rms_norm_eps=1e-6, rope_theta=50000.0, tie_word_embeddings=True,
+  attention_bias=False, rope_scaling=None, sliding_window=40, use_sliding_window=True,
+  layer_types=["full_attention", "sliding_attention", "sliding_attention", "full_attention"])
+PAGE_SIZE = {"A": 16, "B": 8, "C": 16, "D": 8}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def random_weights(cfg: dict, seed: int, dtype=torch.float32, std=0.02, norm_std=0.1):
@@ -66,9 +72,15 @@ def write_model(folder: str, cfg: dict, weights: dict) -> str:
   return folder
 
 
-def make_model(folder: str, name: str, seed: int = 0, dtype=torch.float32, std=0.02):
+def make_model(folder: str, name: str, seed: int = 0, dtype=torch.float32, std=0.02, sharpen: float = 1.0):
+  """sharpen: factor on the per-head norm weights of q and k; scores grow with its square, so attention picks
+  few keys and a key wrongly seen or missed (a window's edge, a page) moves the logits."""
   cfg = CONFIGS[name]
   w = random_weights(cfg, seed, dtype=dtype, std=std)
+  if sharpen != 1.0:
+    for k in w:
+      if k.endswith("q_norm.weight") or k.endswith("k_norm.weight"):
+        w[k] = (w[k].float() * sharpen).to(dtype)
   write_model(folder, cfg, w)
   return cfg, w
 
