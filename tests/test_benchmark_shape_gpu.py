@@ -61,8 +61,9 @@ REGIMES = {
 }
 
 # largest errors seen on an MI355X against the plain logits (scale = the largest plain logit of the request):
-# bfloat16 max 1.1% of the scale (over 151,936 logits a position); the bounds are about twice what was seen
-BF16_MAX, BF16_MEAN = 0.025, 0.004
+# bfloat16 max 1.1% and mean 0.15% of the scale (the max is over 151,936 logits a position); the bounds are about
+# twice what was seen
+BF16_MAX, BF16_MEAN = 0.025, 0.003
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
