@@ -22,6 +22,9 @@
 // accumulators, and that only when some column's maximum moved), in base 2: scores are scaled by
 // scale * log2(e), so a probability is one v_exp_f32.
 #include "common.h"
+#include "attention_mfma.h"
+
+#include <mutex>
 
 #ifndef HEAD_DIM
 #error "compile with -DHEAD_DIM=<head size>"
@@ -1047,4 +1050,53 @@ MI_EXPORT int mi_attn_decode_front(const void* qkv, int64_t qkv_row_stride, void
     MI_CHECK_LAUNCH("attn_decode_front merge");
   }
   return 0;
+}
+
+// ---------------------------------------------------------------- decode without a workspace argument
+// The partials of the key splits in a device array of the shared object itself (see attention_mfma.h).
+static __device__ __align__(256) float scratch[MI_ATTN_STATIC_SCRATCH_FLOATS];
+
+// In host code `scratch` is only a handle of the symbol, never an address a kernel may use: each device has its own
+// copy of the array at its own address, asked for once per device with that device current.
+constexpr int STATIC_MAX_DEVICES = 64;
+static float* g_scratch_ptr[STATIC_MAX_DEVICES] = {nullptr};
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  MI_REQUIRE(e == hipSuccess, "attn_decode_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  MI_REQUIRE(dev >= 0 && dev < STATIC_MAX_DEVICES, "attn_decode_static: device %d; at most %d are served", dev,
+             STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    MI_REQUIRE(e == hipSuccess && p != nullptr, "attn_decode_static: hipGetSymbolAddress failed on device %d: %s", dev,
+               hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+MI_EXPORT int mi_attn_static_scratch_floats() { return MI_ATTN_STATIC_SCRATCH_FLOATS; }
+
+MI_EXPORT int mi_attn_decode_static(const void* q, int64_t q_row_stride, void* out, int64_t out_row_stride,
+                                    const void* k_pages, const void* v_pages, const int* block_table, int table_width,
+                                    const int* cu_q, const int* kv_len, int first_entry, int num_entries,
+                                    int num_splits, int nq, int nkv, int page_size, float scale, int window,
+                                    hipStream_t stream) {
+  MI_REQUIRE(num_entries >= 0 && num_splits >= 1 && nq > 0, "attn_decode_static: bad entry range or splits");
+  const int64_t need = (int64_t)num_entries * nq * num_splits;        // partials: D floats of output, 2 of (max, sum)
+  MI_REQUIRE(num_splits == 1 || need * (D + 2) <= (int64_t)MI_ATTN_STATIC_SCRATCH_FLOATS,
+             "attn_decode_static: %d entries x %d heads x %d splits need %lld floats of partial results; the static "
+             "scratch holds %d (use fewer splits, or mi_attn_decode with a workspace of your own)",
+             num_entries, nq, num_splits, (long long)(need * (D + 2)), MI_ATTN_STATIC_SCRATCH_FLOATS);
+  float* base = nullptr;
+  if (static_scratch(&base)) return 1;
+  // part_o first (need * D floats: a multiple of 16 floats, so part_ml behind it stays 64-byte aligned)
+  return mi_attn_decode(q, q_row_stride, out, out_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len,
+                        first_entry, num_entries, num_splits, base, base + need * D, nq, nkv, page_size, scale, window,
+                        stream);
 }

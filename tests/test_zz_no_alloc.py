@@ -1,0 +1,101 @@
+"""The decode attention entry point that allocates nothing (`mi_attn_decode_static`), called through ctypes.
+
+It runs the kernels of `mi_attn_decode` with the key splits' partial results in a device array of the shared
+object instead of a workspace the caller brings.  Its output must equal `mi_attn_decode`'s on two calls in a row,
+the second with a smaller input (the array then still holds the first call's partials), and a launch whose
+partials do not fit the array must be refused with a message.
+"""
+
+import ctypes
+from ctypes import c_float, c_int, c_int64, c_void_p
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+D = 64
+
+
+def _load():
+  from miniinfer_amd.kernels import jit
+  lib = ctypes.CDLL(jit.compile_module("attention_mfma", (("HEAD_DIM", D),)))
+  common = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int,
+            c_int, c_int]
+  tail = [c_int, c_int, c_int, c_float, c_int, c_void_p]
+  lib.mi_attn_decode.argtypes = common + [c_void_p, c_void_p] + tail
+  lib.mi_attn_decode_static.argtypes = common + tail
+  for f in (lib.mi_attn_decode, lib.mi_attn_decode_static, lib.mi_attn_static_scratch_floats):
+    f.restype = c_int
+  lib.mi_last_error.restype = ctypes.c_char_p
+  return lib
+
+
+def _case(entries, nq, nkv, P, kv_lens, seed):
+  """Random queries and paged keys and values for `entries` requests of one new token each."""
+  dev = torch.device("cuda:0")
+  g = torch.Generator().manual_seed(seed)
+  W = max(-(-n // P) for n in kv_lens)
+  pages = 1 + entries * W
+  k = (torch.randn(pages, nkv, P, D, generator=g) * 0.5).bfloat16().to(dev)
+  v = (torch.randn(pages, nkv, D, P, generator=g) * 0.5).bfloat16().to(dev)
+  perm = (torch.randperm(pages - 1, generator=g) + 1).to(torch.int32)
+  table = torch.zeros(entries, W, dtype=torch.int32)
+  for b in range(entries):
+    n = -(-kv_lens[b] // P)
+    table[b, :n] = perm[b * W:b * W + n]
+  q = (torch.randn(entries, nq * D, generator=g)).bfloat16().to(dev)
+  cu = torch.arange(entries + 1, dtype=torch.int32, device=dev)
+  kv = torch.tensor(kv_lens, dtype=torch.int32, device=dev)
+  return dict(q=q, k=k, v=v, table=table.to(dev), cu=cu, kv=kv, W=W)
+
+
+def _run(lib, c, entries, nq, nkv, P, splits, static):
+  out = torch.full((entries, nq * D), float("nan"), dtype=torch.bfloat16, device=c["q"].device)
+  stream = torch.cuda.current_stream().cuda_stream
+  args = [c["q"].data_ptr(), c["q"].stride(0), out.data_ptr(), out.stride(0), c["k"].data_ptr(), c["v"].data_ptr(),
+          c["table"].data_ptr(), c["W"], c["cu"].data_ptr(), c["kv"].data_ptr(), 0, entries, splits]
+  tail = [nq, nkv, P, D ** -0.5, 0, stream]
+  if static:
+    rc = lib.mi_attn_decode_static(*args, *tail)
+  else:
+    need = entries * nq * splits
+    part_o = torch.empty(need * D, dtype=torch.float32, device=out.device)
+    part_ml = torch.empty(need * 2, dtype=torch.float32, device=out.device)
+    rc = lib.mi_attn_decode(*args, part_o.data_ptr(), part_ml.data_ptr(), *tail)
+  assert rc == 0, lib.mi_last_error().decode()
+  torch.cuda.synchronize()
+  return out
+
+
+def test_decode_attention_from_the_static_scratch_equals_the_workspace_form():
+  lib = _load()
+  assert lib.mi_attn_static_scratch_floats() == 1 << 20
+  nq, nkv, P = 8, 2, 16
+  # first a larger launch (6 requests, 8 key splits), then a smaller one (2 requests, 3 splits, shorter contexts)
+  for entries, splits, kv_lens, seed in ((6, 8, [700, 1500, 64, 1, 333, 2048], 1), (2, 3, [200, 517], 2)):
+    c = _case(entries, nq, nkv, P, kv_lens, seed)
+    print(f"static decode attention: {entries} entries, {splits} splits", flush=True)
+    want = _run(lib, c, entries, nq, nkv, P, splits, static=False)
+    got = _run(lib, c, entries, nq, nkv, P, splits, static=True)
+    assert not torch.isnan(got.float()).any()
+    assert torch.equal(got, want)
+  # one split needs no partials at all
+  c = _case(3, nq, nkv, P, [90, 30, 55], 3)
+  assert torch.equal(_run(lib, c, 3, nq, nkv, P, 1, static=True), _run(lib, c, 3, nq, nkv, P, 1, static=False))
+
+
+def test_a_launch_beyond_the_static_scratch_is_refused():
+  lib = _load()
+  nq, nkv, P = 16, 2, 16
+  entries, splits = 64, 32                     # 64 * 16 * 32 * (64 + 2) floats = 2.1 M > 1 M
+  c = _case(entries, nq, nkv, P, [40] * entries, 4)
+  out = torch.zeros((entries, nq * D), dtype=torch.bfloat16, device=c["q"].device)
+  rc = lib.mi_attn_decode_static(c["q"].data_ptr(), c["q"].stride(0), out.data_ptr(), out.stride(0), c["k"].data_ptr(),
+                                 c["v"].data_ptr(), c["table"].data_ptr(), c["W"], c["cu"].data_ptr(),
+                                 c["kv"].data_ptr(), 0, entries, splits, nq, nkv, P, D ** -0.5, 0,
+                                 torch.cuda.current_stream().cuda_stream)
+  assert rc != 0
+  msg = lib.mi_last_error().decode()
+  assert "static scratch" in msg and "2162688" in msg, msg
+  torch.cuda.synchronize()
+  assert float(out.float().abs().max()) == 0.0     # nothing was launched
