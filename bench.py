@@ -2,10 +2,18 @@
 """Decode and prefill throughput of the engine on one MI355X, Qwen3-0.6B shape, random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--preset qwen3-0.6b]
+    python bench.py --mixed [--preset qwen3-8b] [--num-seqs 64] [--min-input 128] [--max-input 2048] [--output-len 256]
 
 A step is one decode step of the whole engine (schedule, batch building, model, sampling) with `batch`
 requests that each hold `context` tokens in the cache.  Prints ONE JSON line: decoded tokens a second, the
-2,048-token prefill, the decode step's HBM roofline, and decode at batch 1 and 64.
+2,048-token prefill, the decode step's HBM roofline, and decode at batch 1 and 64.  Fractions are given against
+the data sheet's peaks and against what two bare kernels measure on this device when the run starts (one that only
+reads memory, one that only feeds the matrix cores).
+
+`--mixed` runs the serving workload instead: `num-seqs` requests with random prompts of `min-input` to `max-input`
+tokens (uniform) and exactly `output-len` sampled tokens each, all added at once, so that the steps mix prompt
+portions (token budget 8,192) with decoded tokens (the reference's benchmark/bench_miniinfer.py:28-58 with its
+workload's numbers).  Prints one JSON line with output and input tokens a second, steps and preemptions.
 """
 
 from __future__ import annotations
@@ -94,6 +102,65 @@ def time_prefill(engine, T, reps, seed):
   return min(times)
 
 
+def run_mixed(args) -> int:
+  import torch
+  from random import Random
+  from miniinfer_amd import LLMEngine, SamplingParams
+  from miniinfer_amd.kernels import ops
+  from miniinfer_amd.presets import preset
+
+  full = preset(args.preset)
+  cfg = preset(args.preset, args.layers) if args.layers else full
+  page_size = 16
+  max_len = args.max_input + args.output_len + 16
+  pages = args.mixed_pages or args.num_seqs * (-(-max_len // page_size)) + 16
+  hbm_gbs, mfma_tflops = ops.measured_peaks()
+  engine = LLMEngine(model="", model_config=cfg, random_weights_seed=0, dtype=args.dtype, page_size=page_size,
+                     num_pages=pages, max_num_seqs=args.num_seqs, max_model_len=max_len, max_num_batched_tokens=8192,
+                     enforce_eager=args.eager, tune_products=not args.no_tune)
+  rnd = Random(0)
+  V = cfg.vocab_size
+  prompts = [[rnd.randrange(V) for _ in range(rnd.randint(args.min_input, args.max_input))] for _ in range(args.num_seqs)]
+  sp = SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=args.output_len)
+  engine.generate([prompts[0][:8]], SamplingParams(temperature=0.6, max_tokens=2, ignore_eos=True), use_tqdm=False)
+  engine.warm_up(args.num_seqs, max_len)
+  torch.cuda.synchronize()
+  steps0, pre0 = engine.num_steps, engine.scheduler.num_preemptions
+  t0 = time.perf_counter()
+  outs = engine.generate(prompts, sp, use_tqdm=False)
+  torch.cuda.synchronize()
+  dt = time.perf_counter() - t0
+  n_out = sum(len(o["token_ids"]) for o in outs)
+  n_in = sum(len(p) for p in prompts)
+  assert n_out == args.num_seqs * args.output_len
+  esize = 2 if args.dtype == "bfloat16" else 4
+  n = model_numbers(cfg, cfg.num_hidden_layers)
+  shape_name = {"qwen3-0.6b": "Qwen3-0.6B", "qwen3-8b": "Qwen3-8B", "qwen3-32b": "Qwen3-32B"}.get(args.preset, args.preset)
+  steps = engine.num_steps - steps0
+  # what the run must at least do: every weight once per step, and 2 flops per weight and token
+  flops = 2.0 * (n_in + n_out) * n["linear_params"] + 2.0 * n_out * n["head_params"]
+  rec = {
+    "metric": f"output tok/s, {args.num_seqs} requests, prompts {args.min_input}-{args.max_input}, "
+              f"{args.output_len} outputs each, mixed chunked-prefill/decode steps, {shape_name} shape",
+    "value": round(n_out / dt, 1), "unit": "tok/s", "n_gpus": 1, "higher_is_better": True,
+    "input_tok_s": round(n_in / dt, 1), "total_tok_s": round((n_in + n_out) / dt, 1), "seconds": round(dt, 3),
+    "engine_steps": steps, "ms_per_step": round(dt / steps * 1e3, 3),
+    "preemptions": engine.scheduler.num_preemptions - pre0, "input_tokens": n_in, "output_tokens": n_out,
+    "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (seeded random token ids, random weights)",
+    "config": {"model": args.preset, "layers": cfg.num_hidden_layers, "layers_full": full.num_hidden_layers,
+               "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+               "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+               "num_seqs": args.num_seqs, "min_input": args.min_input, "max_input": args.max_input,
+               "output_len": args.output_len, "token_budget": 8192, "page_size": page_size, "pages": pages,
+               "graphs": not args.eager, "overlap": True, "temperature": 0.6},
+    "weights_gbs": round(steps * (n["linear_params"] + n["head_params"]) * esize / dt / 1e9, 1),
+    "frac_flops": round(flops / dt / PEAK_FLOPS[args.dtype], 4),
+    "measured": {"hbm_gbs": round(hbm_gbs, 1), "mfma_bf16_tflops": round(mfma_tflops, 1)},
+  }
+  print(json.dumps(rec))
+  return 0
+
+
 def main() -> int:
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -108,18 +175,31 @@ def main() -> int:
   ap.add_argument("--no-tune", action="store_true", help="choose product kernels by rule instead of timing them at start")
   ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
   ap.add_argument("--only-prefill", action="store_true", help="run only the 2,048-token prefill (for profiling)")
+  ap.add_argument("--mixed", action="store_true", help="the serving workload: many requests, prompts and decodes mixed")
+  ap.add_argument("--num-seqs", type=int, default=64)
+  ap.add_argument("--min-input", type=int, default=128)
+  ap.add_argument("--max-input", type=int, default=2048)
+  ap.add_argument("--output-len", type=int, default=256)
+  ap.add_argument("--mixed-pages", type=int, default=0, help="pages of the cache for --mixed (default: room for all)")
   args = ap.parse_args()
   if args.gpus != 1:
     print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
     return 2
+  if args.mixed:
+    if args.preset == "qwen3-0.6b" and "--preset" not in sys.argv:
+      args.preset = "qwen3-8b"
+    return run_mixed(args)
 
   import torch
   from miniinfer_amd import LLMEngine
+  from miniinfer_amd.kernels import ops
   from miniinfer_amd.presets import preset
 
   full = preset(args.preset)
   cfg = preset(args.preset, args.layers) if args.layers else full
   layers = cfg.num_hidden_layers
+  hbm_gbs, mfma_tflops = ops.measured_peaks()     # what a bare read loop and a bare matrix-core loop reach here
+  mfma_flops = mfma_tflops * 1e12 if args.dtype == "bfloat16" else None
   max_batch = max(args.batch, 1 if args.no_points else 64)
   page_size = 16
   room = args.context + args.steps + args.warmup + (-(-max_batch * args.context // 8192)) + 16
@@ -131,8 +211,10 @@ def main() -> int:
   esize = 2 if args.dtype == "bfloat16" else 4
   if args.only_prefill:
     psec = time_prefill(engine, 2048, reps=max(1, args.steps), seed=2)
+    fl = prefill_flops(cfg, layers, 2048)
     print(json.dumps({"prefill": {"value": round(2048 / psec, 1), "tokens": 2048, "ms": round(psec * 1e3, 3),
-                                  "frac": round(prefill_flops(cfg, layers, 2048) / psec / PEAK_FLOPS[args.dtype], 4)}}))
+                                  "frac": round(fl / psec / PEAK_FLOPS[args.dtype], 4),
+                                  "frac_measured": round(fl / psec / mfma_flops, 4) if mfma_flops else None}}))
     return 0
 
   sec = time_decode(engine, args.batch, args.context, args.steps, args.warmup, seed=1)
@@ -155,14 +237,17 @@ def main() -> int:
       "parallelism": "1 GPU", "graphs": not args.eager, "prefill_tokens": 2048,
     },
     "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                 "frac": round(achieved / PEAK_HBM_GBS, 4)},
+                 "frac": round(achieved / PEAK_HBM_GBS, 4), "peak_measured": round(hbm_gbs, 1),
+                 "frac_measured": round(achieved / hbm_gbs, 4)},
+    "measured": {"hbm_gbs": round(hbm_gbs, 1), "mfma_bf16_tflops": round(mfma_tflops, 1)},
   }
   if not args.no_points:
     T = 2048
     psec = time_prefill(engine, T, reps=3, seed=2)
     fl = prefill_flops(cfg, layers, T)
     rec["prefill"] = {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
-                      "frac": round(fl / psec / PEAK_FLOPS[args.dtype], 4)}
+                      "frac": round(fl / psec / PEAK_FLOPS[args.dtype], 4),
+                      "frac_measured": round(fl / psec / mfma_flops, 4) if mfma_flops else None}
     points = {}
     for b in (1, 64):
       s = time_decode(engine, b, args.context, max(8, args.steps // 2), max(2, args.warmup // 2), seed=10 + b)

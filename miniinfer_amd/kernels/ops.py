@@ -122,6 +122,11 @@ _SIGS["sampling"] = {
   "mi_sample_parts_count": [c_int],
 }
 
+_SIGS["probes"] = {
+  "mi_probe_stream_read": [c_void_p, c_int64, c_void_p, c_void_p],
+  "mi_probe_mfma": [c_int, c_int, c_void_p, c_void_p, c_void_p],
+}
+
 _libs = {}
 
 
@@ -700,3 +705,50 @@ def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.T
     block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry, num_entries, num_splits, _ptr(part_o), _ptr(part_ml),
     nq, nkv, k_pages.shape[2], float(scale), int(window), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin),
     rotary_dim, max_pos, _ptr(positions), _ptr(slots), _stream()))
+
+
+# ----------------------------------------------------------------------------- what the device delivers
+
+_MEASURED_PEAKS: Dict[int, Tuple[float, float]] = {}
+
+
+def measured_peaks(device=None, stream_bytes: int = 1 << 31) -> Tuple[float, float]:
+  """(GB/s of a kernel that only reads `stream_bytes` of device memory, TFLOP/s of a kernel that only runs dense
+  bfloat16 matrix instructions on registers) on this device: the best of a few runs each, measured once per process
+  and device (about 50 ms)."""
+  index = torch.device(device).index if device is not None else None
+  if index is None:
+    index = torch.cuda.current_device()
+  if index in _MEASURED_PEAKS:
+    return _MEASURED_PEAKS[index]
+  lib = _lib("probes")
+  dev = torch.device("cuda", index)
+  free, _ = torch.cuda.mem_get_info(dev)
+  nbytes = max(1 << 24, min(stream_bytes, free // 4) // 16 * 16)
+  buf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+  buf.random_(0, 255)
+  sink = torch.zeros(4, dtype=torch.float32, device=dev)
+  start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  flops = ctypes.c_double(0.0)
+  cus = torch.cuda.get_device_properties(dev).multi_processor_count
+
+  def best_ms(launch, reps):
+    launch()
+    torch.cuda.synchronize(dev)
+    best = float("inf")
+    for _ in range(reps):
+      start.record()
+      launch()
+      end.record()
+      torch.cuda.synchronize(dev)
+      best = min(best, start.elapsed_time(end))
+    return best
+
+  with torch.cuda.device(dev):
+    ms = best_ms(lambda: _check(lib, lib.mi_probe_stream_read(_ptr(buf), nbytes, _ptr(sink), _stream())), 5)
+    gbs = nbytes / ms / 1e6
+    ms = best_ms(lambda: _check(lib, lib.mi_probe_mfma(cus * 8, 4096, _ptr(sink), ctypes.byref(flops), _stream())), 3)
+    tflops = flops.value / ms / 1e9
+  del buf
+  _MEASURED_PEAKS[index] = (gbs, tflops)
+  return _MEASURED_PEAKS[index]
