@@ -312,7 +312,8 @@ __device__ __forceinline__ void prefill_body(
   const int kgroup = (threadIdx.x >> 6) >> 2;            // which macro tile of a step this wave multiplies
   const int wave = (threadIdx.x >> 6) & 3;               // its query block within the workgroup
   const int tid = threadIdx.x & 255;                     // the thread's place among those that stage one macro tile
-  const int stage = threadIdx.x >> 8;                    // and which macro tile of a step they stage
+  // and which macro tile of a step they stage (the same for a whole wave: said so, for the scalar page lookups)
+  const int stage = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
   uint16_t* Ks = Ks_all + kgroup * KS_TILE;
   uint16_t* Vs = Vs_all + kgroup * VS_TILE;
   uint16_t* Ks_stage = Ks_all + stage * KS_TILE;
@@ -391,15 +392,22 @@ __device__ __forceinline__ void prefill_body(
   const uint16_t* kbase = k_pages + (int64_t)g * P * D;     // + page * page_stride + (slot in page) * D + element
   const uint16_t* vbase = v_pages + (int64_t)g * D * P;     // + page * page_stride + dim * P + slot in page
   const int page_stride = nkv * P * D;                      // elements; a page of one layer is far below 2^31
+  // For head sizes that are multiples of 64 (pages hold 8 tokens or more) the 64 chunks of a wave lie in one page,
+  // keys and values alike: the page number is then looked up once per wave with scalar instructions (from the
+  // first lane's key), and the page's base address is scalar arithmetic instead of 64-bit vector arithmetic
+  // (a third of the vector instructions that fetching a macro tile took).
+  constexpr bool PAGE_PER_WAVE = (D % 64) == 0;
 #define PREFILL_PAGES(J0)                                                                                            \
   {                                                                                                                  \
     _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
-      const int key = min((J0) + k_key[it], last); /* masked keys read valid memory of the request */               \
+      int key = min((J0) + k_key[it], last); /* masked keys read valid memory of the request */                     \
+      if (PAGE_PER_WAVE) key = __builtin_amdgcn_readfirstlane(key);                                                  \
       kpage[it] = bt[key >> page_shift];                                                                             \
     }                                                                                                                \
     _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
       int key = (J0) + v_key[it];                                                                                    \
       key = key > last ? (last & ~7) : key; /* a run of 8 keys lies in one page */                                  \
+      if (PAGE_PER_WAVE) key = __builtin_amdgcn_readfirstlane(key);                                                  \
       vpage[it] = bt[key >> page_shift];                                                                             \
     }                                                                                                                \
   }
@@ -407,14 +415,14 @@ __device__ __forceinline__ void prefill_body(
   {                                                                                                                  \
     _Pragma("unroll") for (int it = 0; it < LDS_KITER; ++it) {                                                       \
       const int key = min((J0) + k_key[it], last);                                                                   \
-      pk[it] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kpage[it] * page_stride +                            \
-                                               ((key & (P - 1)) * D + k_col[it]));                                   \
+      const uint16_t* page = kbase + (int64_t)kpage[it] * page_stride;                                               \
+      pk[it] = *reinterpret_cast<const u32x4*>(page + ((key & (P - 1)) * D + k_col[it]));                            \
     }                                                                                                                \
     _Pragma("unroll") for (int it = 0; it < LDS_VITER; ++it) {                                                       \
       int key = (J0) + v_key[it];                                                                                    \
       key = key > last ? (last & ~7) : key;                                                                          \
-      pv[it] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)vpage[it] * page_stride +                            \
-                                               (v_dim[it] * P + (key & (P - 1))));                                   \
+      const uint16_t* page = vbase + (int64_t)vpage[it] * page_stride;                                               \
+      pv[it] = *reinterpret_cast<const u32x4*>(page + (v_dim[it] * P + (key & (P - 1))));                            \
     }                                                                                                                \
   }
 #define PREFILL_STASH()                                                                                              \

@@ -401,18 +401,19 @@ __global__ void qk_norm_rope_cache_kernel(T* __restrict__ qkv, int64_t row_strid
 // pairs (j .. j + 3, each with its partner d/2 further on) in 64-bit or 128-bit accesses, so a wave holds 64 / LPH
 // heads of one token at a time, and two such sets in flight.  LPH is the power of two >= d / 8.
 template <typename T, int LPH>
-__global__ void qk_norm_rope_many_kernel(T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
-                                         const float* __restrict__ qw, const float* __restrict__ kw, float eps,
-                                         const float* __restrict__ cos_sin, int max_pos,
-                                         const int* __restrict__ positions, T* __restrict__ k_pages,
-                                         const int* __restrict__ slots, int page_shift, int num_tokens) {
+__device__ __forceinline__ void qk_norm_rope_many_body(int block, T* __restrict__ qkv, int64_t row_stride, int nq,
+                                                       int nkv, int d, const float* __restrict__ qw,
+                                                       const float* __restrict__ kw, float eps,
+                                                       const float* __restrict__ cos_sin, int max_pos,
+                                                       const int* __restrict__ positions, T* __restrict__ k_pages,
+                                                       const int* __restrict__ slots, int page_shift, int num_tokens) {
   constexpr int HPS = MI_WAVE / LPH;     // heads per set
   constexpr int SETS = 2;
   const int lane = threadIdx.x & (MI_WAVE - 1);
   const int sub = lane / LPH, ln = lane % LPH;
   const int heads = nq + nkv;
   const int groups = (heads + HPS * SETS - 1) / (HPS * SETS);
-  const int64_t wid = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + threadIdx.x / MI_WAVE;
+  const int64_t wid = (int64_t)block * (blockDim.x / MI_WAVE) + threadIdx.x / MI_WAVE;
   if (wid >= (int64_t)num_tokens * groups) return;
   const int t = (int)(wid / groups);
   const int h0 = (int)(wid - (int64_t)t * groups) * HPS * SETS;
@@ -489,13 +490,13 @@ __global__ void qk_norm_rope_many_kernel(T* __restrict__ qkv, int64_t row_stride
 // of 8 tokens whose slots are consecutive and start at a multiple of 8 is written as one run of 8 per dim (16 bytes
 // in bfloat16) instead of 8 scattered elements; any other half falls back to single elements.
 template <typename T>
-__global__ void value_cache_write_kernel(const T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
-                                         T* __restrict__ v_pages, const int* __restrict__ slots, int page_shift,
-                                         int num_tokens) {
-  const int g = blockIdx.y;
+__device__ __forceinline__ void value_cache_write_body(int block_x, int g, const T* __restrict__ qkv,
+                                                       int64_t row_stride, int nq, int nkv, int d,
+                                                       T* __restrict__ v_pages, const int* __restrict__ slots,
+                                                       int page_shift, int num_tokens) {
   const int P = 1 << page_shift;
   for (int hf = 0; hf < 2; ++hf) {
-    const int t0 = blockIdx.x * 16 + 8 * hf;
+    const int t0 = block_x * 16 + 8 * hf;
     const int n = min(8, num_tokens - t0);
     if (n <= 0) break;
     const int slot0 = slots[t0];
@@ -527,6 +528,45 @@ __global__ void value_cache_write_kernel(const T* __restrict__ qkv, int64_t row_
       }
     }
   }
+}
+
+template <typename T, int LPH>
+__global__ void qk_norm_rope_many_kernel(T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
+                                         const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+                                         const float* __restrict__ cos_sin, int max_pos,
+                                         const int* __restrict__ positions, T* __restrict__ k_pages,
+                                         const int* __restrict__ slots, int page_shift, int num_tokens) {
+  qk_norm_rope_many_body<T, LPH>(blockIdx.x, qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, max_pos, positions,
+                                 k_pages, slots, page_shift, num_tokens);
+}
+
+// Both at once, for many tokens: the first `norm_blocks` workgroups norm and rotate the q and k heads (and write the
+// keys), the others copy the values (workgroup norm_blocks + x + value_blocks_x * g takes tokens 16 x .. of kv head
+// g).  The two halves read different columns of qkv and depend on nothing of each other, so one launch does for
+// what two launches in a row would wait for each other.
+template <typename T, int LPH>
+__global__ void qk_norm_rope_values_kernel(T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
+                                           const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+                                           const float* __restrict__ cos_sin, int max_pos,
+                                           const int* __restrict__ positions, T* __restrict__ k_pages,
+                                           T* __restrict__ v_pages, const int* __restrict__ slots, int page_shift,
+                                           int num_tokens, int norm_blocks, int value_blocks_x) {
+  if ((int)blockIdx.x < norm_blocks) {
+    qk_norm_rope_many_body<T, LPH>(blockIdx.x, qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, max_pos, positions,
+                                   k_pages, slots, page_shift, num_tokens);
+  } else {
+    const int b = blockIdx.x - norm_blocks;
+    value_cache_write_body<T>(b % value_blocks_x, b / value_blocks_x, qkv, row_stride, nq, nkv, d, v_pages, slots,
+                              page_shift, num_tokens);
+  }
+}
+
+template <typename T>
+__global__ void value_cache_write_kernel(const T* __restrict__ qkv, int64_t row_stride, int nq, int nkv, int d,
+                                         T* __restrict__ v_pages, const int* __restrict__ slots, int page_shift,
+                                         int num_tokens) {
+  value_cache_write_body<T>(blockIdx.x, blockIdx.y, qkv, row_stride, nq, nkv, d, v_pages, slots, page_shift,
+                            num_tokens);
 }
 
 MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, int num_tokens, int nq, int nkv, int d,
@@ -564,9 +604,19 @@ MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, in
   const int heads_per_wave = 2 * (MI_WAVE / lph);
   const int64_t many_waves = (int64_t)num_tokens * ((nq + nkv + heads_per_wave - 1) / heads_per_wave);
   const int many_blocks = (int)((many_waves + waves_per_block - 1) / waves_per_block);
+  // many tokens with their values: one launch for both halves
+  const bool both = many && split_values;
+  const int64_t all_blocks = (int64_t)many_blocks + (int64_t)vgrid.x * vgrid.y;
+  MI_REQUIRE(!both || all_blocks < (1ll << 31), "qk_norm_rope_cache: too many workgroups");
 #define MI_LAUNCH_MANY(T, LPH)                                                                                      \
-  qk_norm_rope_many_kernel<T, LPH><<<many_blocks, waves_per_block * MI_WAVE, 0, stream>>>(                          \
-      (T*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, max_pos, positions, (T*)k_pages, slots, shift, num_tokens)
+  if (both)                                                                                                         \
+    qk_norm_rope_values_kernel<T, LPH><<<(unsigned)all_blocks, waves_per_block * MI_WAVE, 0, stream>>>(             \
+        (T*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, max_pos, positions, (T*)k_pages, (T*)v_pages, slots, \
+        shift, num_tokens, many_blocks, (int)vgrid.x);                                                              \
+  else                                                                                                              \
+    qk_norm_rope_many_kernel<T, LPH><<<many_blocks, waves_per_block * MI_WAVE, 0, stream>>>(                        \
+        (T*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, max_pos, positions, (T*)k_pages, slots, shift,       \
+        num_tokens)
 #define MI_LAUNCH_MANY_ANY(T)                                                                                       \
   switch (lph) {                                                                                                    \
     case 1: case 2: MI_LAUNCH_MANY(T, 2); break;                                                                    \
@@ -583,7 +633,7 @@ MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, in
           (float*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (float*)k_pages,
           (float*)v_pages, slots, shift, num_tokens, heads);
     }
-    if (split_values)
+    if (split_values && !both)
       value_cache_write_kernel<float><<<vgrid, vthreads, 0, stream>>>((const float*)qkv, row_stride, nq, nkv, d,
                                                                       (float*)v_pages, slots, shift, num_tokens);
   } else if (dtype == MI_DTYPE_BF16) {
@@ -594,7 +644,7 @@ MI_EXPORT int mi_qk_norm_rope_cache(int dtype, void* qkv, int64_t row_stride, in
           (bf16*)qkv, row_stride, nq, nkv, d, qw, kw, eps, cos_sin, rotary_dim, max_pos, positions, (bf16*)k_pages,
           (bf16*)v_pages, slots, shift, num_tokens, heads);
     }
-    if (split_values)
+    if (split_values && !both)
       value_cache_write_kernel<bf16><<<vgrid, vthreads, 0, stream>>>((const bf16*)qkv, row_stride, nq, nkv, d,
                                                                      (bf16*)v_pages, slots, shift, num_tokens);
   } else {
