@@ -52,6 +52,8 @@ class AttentionSpec:
                                      # named by LayerSpec.cache_of
   # checkpoint names of the q, k, v and output projections and of the q and k norms
   tensor_names: Tuple[str, ...] = ("q_proj", "k_proj", "v_proj", "o_proj", "q_norm", "k_norm")
+  qkv_bias: bool = False             # "<name>.bias" tensors beside the q, k, v projections' weights
+  o_bias: bool = False               # and beside the output projection's
   kind: str = "paged_attention"
 
 
@@ -62,6 +64,7 @@ class GatedMLPSpec:
   intermediate_size: int
   activation: str = "silu"
   tensor_names: Tuple[str, ...] = ("gate_proj", "up_proj", "down_proj")
+  bias: bool = False                 # "<name>.bias" tensors beside the three weights
   kind: str = "gated_mlp"
 
 

@@ -202,6 +202,34 @@ MI_EXPORT int mi_add_rmsnorm(int x_dtype, int y_dtype, const void* x, float* res
   return 0;
 }
 
+// ---------------------------------------------------------------- bias of a projection
+// y[m][n] += b[n], in 32-bit, for projections that carry a bias (the products themselves have none).
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, int64_t ld, const T* __restrict__ b, int M, int N) {
+  const int64_t total = (int64_t)M * N;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = idx / N;
+    const int n = (int)(idx - m * N);
+    y[m * ld + n] = from_float<T>(to_float(y[m * ld + n]) + to_float(b[n]));
+  }
+}
+
+MI_EXPORT int mi_add_bias(int dtype, void* y, int64_t ld, const void* b, int M, int N, hipStream_t stream) {
+  MI_REQUIRE(M >= 0 && N > 0 && ld >= N, "add_bias: bad sizes M=%d N=%d ld=%lld", M, N, (long long)ld);
+  if (M == 0) return 0;
+  int64_t blocks = ((int64_t)M * N + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == MI_DTYPE_F32)
+    add_bias_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)y, ld, (const float*)b, M, N);
+  else if (dtype == MI_DTYPE_BF16)
+    add_bias_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((bf16*)y, ld, (const bf16*)b, M, N);
+  else
+    MI_FAIL("add_bias: unknown dtype %d", dtype);
+  MI_CHECK_LAUNCH("add_bias");
+  return 0;
+}
+
 // ---------------------------------------------------------------- SiLU(gate) * up
 // gu [M, 2I]: gate = first I columns, up = last I.  out [M, I].
 template <typename T>

@@ -31,7 +31,7 @@ DEV = "cuda:0"
 def cmd_product(args) -> int:
   rows_w = 2 * args.n if args.gate_up else args.n
   nbytes = rows_w * args.k * 2
-  copies = max(2, min(8, (1536 << 20) // nbytes))
+  copies = args.copies or max(2, min(8, (1536 << 20) // nbytes))
   ws = [(torch.randn(rows_w, args.k, device=DEV) * 0.02).bfloat16() for _ in range(copies)]
   a = torch.randn(args.rows, args.k, device=DEV).bfloat16()
   out = torch.empty(args.rows, args.n, dtype=torch.bfloat16, device=DEV)
@@ -146,6 +146,9 @@ def main(argv=None) -> int:
   p.add_argument("--k", type=int, required=True)
   p.add_argument("--gate-up", action="store_true", help="a fused gate|up matrix [2 n, k] with the activation in the epilogue")
   p.add_argument("--calls", type=int, default=24)
+  p.add_argument("--copies", type=int, default=0,
+                 help="matrices the calls cycle through (default: up to 8, 1.5 GB at most); with many, the weights "
+                      "come from memory and not from a cache that holds the few")
   p.set_defaults(fn=cmd_product)
   a = sub.add_parser("prefill-attention", help="the MFMA prefill attention for one prompt")
   a.add_argument("--tokens", type=int, default=2048)

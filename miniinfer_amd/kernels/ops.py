@@ -77,6 +77,7 @@ _SIGS = {
     "mi_add_rmsnorm": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                        c_void_p],
     "mi_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "mi_add_bias": [c_int, c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p],
     "mi_qk_norm_rope_cache": [c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
                               c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
   },
@@ -241,6 +242,20 @@ def add_rmsnorm(x: Optional[torch.Tensor], residual: Optional[torch.Tensor], wei
                                  _ptr(residual), _ptr(weight), _ptr(out), _ptr(rows), M, N, float(eps),
                                  1 if write_back else 0, _stream()))
   return out
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+  """y[m, :] += bias, in place; y [M, N] with dense rows, bias [N] of y's dtype (bfloat16 or float32)."""
+  _dev(y, bias)
+  if y.dim() != 2 or (y.shape[1] > 1 and y.stride(1) != 1) or bias.dim() != 1 or bias.numel() != y.shape[1]:
+    raise KernelError(f"add_bias: y {tuple(y.shape)} and bias {tuple(bias.shape)} do not fit")
+  if bias.dtype != y.dtype:
+    raise KernelError(f"add_bias: y is {y.dtype}, the bias {bias.dtype}")
+  _contig("bias", bias)
+  M, N = y.shape
+  lib = _lib("elementwise")
+  _check(lib, lib.mi_add_bias(dtype_code(y.dtype), _ptr(y), y.stride(0) if M > 1 else N, _ptr(bias), M, N, _stream()))
+  return y
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -37,6 +37,8 @@ class PagedAttention(Part):
     self.shares_kv = bool(getattr(spec, "shares_kv", False))
     self.qkv_weight: Optional[torch.Tensor] = None   # q rows only when the keys and values are borrowed
     self.o_weight: Optional[torch.Tensor] = None
+    self.qkv_bias: Optional[torch.Tensor] = None     # only when the spec asks for them
+    self.o_bias: Optional[torch.Tensor] = None
 
   # ------------------------------------------------------------------ tensors
   def param_specs(self) -> List[ParamSpec]:
@@ -47,7 +49,14 @@ class PagedAttention(Part):
     else:
       qkv = ParamSpec("qkv_weight", ((nq + 2 * nkv) * d, H),
                       (Source(qn + ".weight", nq * d), Source(kn + ".weight", nkv * d), Source(vn + ".weight", nkv * d)))
-    return [qkv, ParamSpec("o_weight", (H, nq * d), (Source(on + ".weight", H),))]
+    out = [qkv, ParamSpec("o_weight", (H, nq * d), (Source(on + ".weight", H),))]
+    if getattr(self.spec, "qkv_bias", False):
+      srcs = (Source(qn + ".bias", nq * d),) if self.shares_kv else \
+          (Source(qn + ".bias", nq * d), Source(kn + ".bias", nkv * d), Source(vn + ".bias", nkv * d))
+      out.append(ParamSpec("qkv_bias", (sum(s.rows for s in srcs),), srcs, init="normal"))
+    if getattr(self.spec, "o_bias", False):
+      out.append(ParamSpec("o_bias", (H,), (Source(on + ".bias", H),), init="normal"))
+    return out
 
   def children(self) -> List[Tuple[str, Part]]:
     if self.q_norm is None:
@@ -71,7 +80,7 @@ class PagedAttention(Part):
     """The same with the output projection left pending, so that the block can fold the add and the next norm
     into it."""
     T = x.shape[0]
-    qkv = linear(x, self.qkv_weight)
+    qkv = linear(x, self.qkv_weight, bias=self.qkv_bias)
     table = self.position.rotary_table()
     eps = self.q_norm.eps if self.q_norm is not None else 0.0
     if ctx.num_multi == 0 and not self.shares_kv and (table is None or table.shape[1] == self.d) and \
@@ -79,7 +88,7 @@ class PagedAttention(Part):
       # a step of decoded tokens only: the attention kernel norms, rotates and caches by itself
       out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
       self._attend_decode(qkv, out, ctx, cache, 0, ctx.num_requests, front=(table, eps))
-      return PendingLinear(out, self.o_weight)
+      return PendingLinear(out, self.o_weight, self.o_bias)
     if self.shares_kv:
       # only queries of its own: they are normed and rotated; the borrowed pages are read, never written
       ops.qk_norm_rope_cache(qkv, self.nq, 0, self.d, self.q_norm.weight if self.q_norm is not None else None, None,
@@ -92,7 +101,7 @@ class PagedAttention(Part):
         eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
     out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
     self._attend(qkv, out, ctx, cache)
-    return PendingLinear(out, self.o_weight)
+    return PendingLinear(out, self.o_weight, self.o_bias)
 
   def _attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx, cache) -> None:
     nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0

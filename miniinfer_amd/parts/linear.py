@@ -22,9 +22,10 @@ class PendingLinear:
   split between the two products' kernels (`_fuse_norm`) and need none of their own; anyone else calls
   `materialize()`."""
 
-  def __init__(self, a: torch.Tensor, weight: torch.Tensor):
+  def __init__(self, a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
     self.a = a
     self.weight = weight
+    self.bias = bias
     self.value: Optional[torch.Tensor] = None
 
   @property
@@ -41,7 +42,7 @@ class PendingLinear:
 
   def materialize(self) -> torch.Tensor:
     if self.value is None:
-      self.value = linear(self.a, self.weight)
+      self.value = linear(self.a, self.weight, bias=self.bias)
     return self.value
 
 
@@ -58,6 +59,8 @@ def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]
   if not ops.skinny_preferred(M, weight.shape[0], weight.shape[1], gate_up):
     return None
   N = weight.shape[0] // 2 if gate_up else weight.shape[0]
+  if isinstance(d.x, PendingLinear) and d.x.value is None and d.x.bias is not None:
+    d.x = d.x.materialize()              # a product with a bias is finished by its own kernels
   if isinstance(d.x, PendingLinear) and d.x.value is None:
     # The branch's last product is still pending: its kernel adds to the residual stream in place and leaves
     # bfloat16(residual * norm weight) and partial sums of squares; this product's kernel scales its rows by them.
@@ -85,9 +88,13 @@ def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]
 _MM_TAKES_OUT_DTYPE = [True]     # torch.mm(..., out_dtype=) exists in this torch (found out at the first call)
 
 
-def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
   """x: a tensor [M, K], a pending product, or a DeferredNorm (the add and the norm are then fused into the product
-  if possible)."""
+  if possible).  bias [N] (of the result's dtype) is added by a kernel of its own: the architecture this engine
+  serves has none, so the products' kernels carry no bias path."""
+  if bias is not None:
+    return ops.add_bias(linear(x, weight, out_dtype), bias)
   x = as_tensor(x)
   if hasattr(x, "materialize"):
     if out_dtype in (None, torch.bfloat16):
@@ -129,9 +136,15 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> 
   return torch.matmul(x, weight.t())
 
 
-def gate_up_activation(x: torch.Tensor, gate_up_weight: torch.Tensor) -> torch.Tensor:
+def gate_up_activation(x: torch.Tensor, gate_up_weight: torch.Tensor,
+                       bias: Optional[torch.Tensor] = None) -> torch.Tensor:
   """silu(x Wg^T) * (x Wu^T) for a fused gate|up matrix [2 I, K]: one kernel for few rows (the activation is made
-  from the 32-bit sums in the product's epilogue), product and activation kernels otherwise."""
+  from the 32-bit sums in the product's epilogue), product and activation kernels otherwise.  With a bias [2 I]
+  (gate | up) the product, the bias and the activation are separate kernels."""
+  if bias is not None:
+    gu = linear(x, gate_up_weight, bias=bias)
+    act = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype, device=gu.device)
+    return ops.silu_mul(gu, act)
   x = as_tensor(x)
   if hasattr(x, "materialize"):
     y = _fuse_norm(x, gate_up_weight, gate_up=True)

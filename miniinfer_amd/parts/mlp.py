@@ -22,14 +22,21 @@ class GatedMLP(Part):
     self.inter = spec.intermediate_size
     self.gate_up_weight: Optional[torch.Tensor] = None
     self.down_weight: Optional[torch.Tensor] = None
+    self.gate_up_bias: Optional[torch.Tensor] = None     # only when the spec asks for them
+    self.down_bias: Optional[torch.Tensor] = None
 
   def param_specs(self) -> List[ParamSpec]:
     g, u, d = self.spec.tensor_names
-    return [
+    out = [
       ParamSpec("gate_up_weight", (2 * self.inter, self.hidden),
                 (Source(g + ".weight", self.inter), Source(u + ".weight", self.inter))),
       ParamSpec("down_weight", (self.hidden, self.inter), (Source(d + ".weight", self.hidden),)),
     ]
+    if getattr(self.spec, "bias", False):
+      out.append(ParamSpec("gate_up_bias", (2 * self.inter,),
+                           (Source(g + ".bias", self.inter), Source(u + ".bias", self.inter))))
+      out.append(ParamSpec("down_bias", (self.hidden,), (Source(d + ".bias", self.hidden),)))
+    return out
 
   def products(self):
     return [(self.gate_up_weight, True), (self.down_weight, False)]
@@ -39,7 +46,7 @@ class GatedMLP(Part):
 
   def forward_lazy(self, x, ctx) -> PendingLinear:
     """The same with the down projection left pending, so that the block can fold the add and the next norm into it."""
-    return PendingLinear(gate_up_activation(x, self.gate_up_weight), self.down_weight)
+    return PendingLinear(gate_up_activation(x, self.gate_up_weight, self.gate_up_bias), self.down_weight, self.down_bias)
 
 
 register_feed_forward("gated_mlp", GatedMLP)

@@ -494,3 +494,37 @@ def test_norm_split_between_two_products(M, N, K, N2, gate_up):
                              rtol=3e-2, atol=3e-2 * float(y.abs().max()))
   want = torch.nn.functional.silu(y[:, :N2]) * y[:, N2:] if gate_up else y
   torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N", [(7, 136), (1, 5), (130, 1000)])
+def test_add_bias(dtype, M, N):
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(M + N)
+  y = torch.randn(M, N, generator=g).to(dtype)
+  b = torch.randn(N, generator=g).to(dtype)
+  want = (y.float() + b.float()).to(dtype)
+  got = ops.add_bias(y.clone().to(DEV), b.to(DEV))
+  assert torch.equal(got.cpu(), want)
+  with pytest.raises(ops.KernelError):
+    ops.add_bias(y.to(DEV), b[:-1].to(DEV))
+
+
+def test_microbench_commands_run_at_small_sizes(capsys):
+  """The measuring tool that the profile summaries cite: each command runs and prints its line."""
+  from miniinfer_amd.kernels import microbench
+  assert microbench.main(["product", "--rows", "4", "--n", "256", "--k", "128", "--calls", "4", "--copies", "2"]) == 0
+  assert microbench.main(["product", "--rows", "20", "--n", "64", "--k", "256", "--gate-up", "--calls", "4"]) == 0
+  assert microbench.main(["prefill-attention", "--tokens", "200", "--heads", "4", "--kv-heads", "2", "--head-dim", "64",
+                          "--calls", "2"]) == 0
+  assert microbench.main(["decode-attention", "--batch", "3", "--context", "300", "--heads", "4", "--kv-heads", "2",
+                          "--head-dim", "64", "--calls", "4"]) == 0
+  out = capsys.readouterr().out
+  assert out.count("gemm_skinny:") == 2 and "attn_prefill dense" in out and "attn_decode_front" in out
+
+
+def test_measured_peaks_are_plausible():
+  from miniinfer_amd.kernels import ops
+  gbs, tflops = ops.measured_peaks(stream_bytes=1 << 28)
+  assert 500 < gbs < 8000 and 100 < tflops < 2500, (gbs, tflops)
+  assert ops.measured_peaks() == (gbs, tflops)      # measured once per process and device

@@ -4,7 +4,8 @@ the framework:
     weights renormalised),
   * another position encoding (rotation of half of each head only, by angles of an interpolated position, from a
     table the part builds itself),
-  * a layer whose attention has no position encoding at all, beside a layer with the ordinary one.
+  * a layer whose attention has no position encoding at all, beside a layer with the ordinary one,
+  * a layer whose projections (q, k, v, output, gate, up, down) carry biases.
 A second toy architecture made of them is built from a config.json, loaded by tensor name and stepped whole, in
 portions and in mixed batches; its logits must equal a plain whole-sequence statement of the same model."""
 
@@ -115,12 +116,12 @@ def _register():
       positions = (SlowPartialRotarySpec(d // 2, self.theta, self.factor, self.max_positions), NoPositionSpec(),
                    RotarySpec(rotary_dim=d, theta=self.theta, max_positions=self.max_positions))
       routed = RoutedSpec(H, self.expert_size, E, TOPK)
-      dense = GatedMLPSpec(hidden_size=H, intermediate_size=self.intermediate_size)
+      dense = GatedMLPSpec(hidden_size=H, intermediate_size=self.intermediate_size, bias=True)
       layers = tuple(
         LayerSpec(prefix=f"toy2.layers.{i}.",
                   mixer=AttentionSpec(hidden_size=H, num_heads=self.num_heads, num_kv_heads=self.num_kv_heads,
                                       head_dim=d, scale=d ** -0.5, position=positions[i],
-                                      qk_norm=NormSpec(d, self.eps)),
+                                      qk_norm=NormSpec(d, self.eps), qkv_bias=(i == 1), o_bias=(i == 1)),
                   feed_forward=dense if i == 1 else routed, mixer_norm=norm, feed_forward_norm=norm)
         for i in range(3))
       return ModelSpec(architecture="Toy2ForCausalLM", vocab_size=self.vocab_size, hidden_size=H, layers=layers,
@@ -154,6 +155,9 @@ def _weights(seed=0, std=0.08):
     if i == 1:
       for n, shape in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
         w[p + f"mlp.{n}.weight"] = mat(*shape)
+        w[p + f"mlp.{n}.bias"] = mat(shape[0]) * 3
+      for n, rows in (("q_proj", nq * d), ("k_proj", nkv * d), ("v_proj", nkv * d), ("o_proj", H)):
+        w[p + f"self_attn.{n}.bias"] = mat(rows) * 3
     else:
       w[p + "mlp.router.weight"] = mat(E, H) * 40         # decided choices: a third expert is seldom close to the second
       w[p + "mlp.gate_up"] = mat(E, 2 * Ie, H)
@@ -179,9 +183,12 @@ def _plain_toy2(tokens: List[int], w, round_act, close_calls=None) -> torch.Tens
   for i in range(3):
     p = f"toy2.layers.{i}."
     x = plain.rms_norm(h, w[p + "input_layernorm.weight"], c["eps"])
-    q = plain.rms_norm((x @ w[p + "self_attn.q_proj.weight"].T).reshape(T, nq, d), w[p + "self_attn.q_norm.weight"], c["eps"])
-    k = plain.rms_norm((x @ w[p + "self_attn.k_proj.weight"].T).reshape(T, nkv, d), w[p + "self_attn.k_norm.weight"], c["eps"])
-    v = (x @ w[p + "self_attn.v_proj.weight"].T).reshape(T, nkv, d)
+    bias = lambda name: w.get(p + name + ".bias", 0.0)      # only layer 1 has biases
+    q = plain.rms_norm((x @ w[p + "self_attn.q_proj.weight"].T + bias("self_attn.q_proj")).reshape(T, nq, d),
+                       w[p + "self_attn.q_norm.weight"], c["eps"])
+    k = plain.rms_norm((x @ w[p + "self_attn.k_proj.weight"].T + bias("self_attn.k_proj")).reshape(T, nkv, d),
+                       w[p + "self_attn.k_norm.weight"], c["eps"])
+    v = (x @ w[p + "self_attn.v_proj.weight"].T + bias("self_attn.v_proj")).reshape(T, nkv, d)
     if i == 0:
       ang = plain.rope_angles(pos.double() / c["factor"], d // 2, c["theta"], torch.float64)
       q, k = _rotate_part(q, ang, d // 2), _rotate_part(k, ang, d // 2)
@@ -189,10 +196,12 @@ def _plain_toy2(tokens: List[int], w, round_act, close_calls=None) -> torch.Tens
       ang = plain.rope_angles(pos, d, c["theta"], torch.float64)
       q, k = plain.apply_rope_neox(q, ang), plain.apply_rope_neox(k, ang)
     o = plain.grouped_attention(q, k, v, d ** -0.5, plain.causal_mask(T, T, torch.float64))
-    h = h + o.reshape(T, nq * d) @ w[p + "self_attn.o_proj.weight"].T
+    h = h + o.reshape(T, nq * d) @ w[p + "self_attn.o_proj.weight"].T + bias("self_attn.o_proj")
     x = plain.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["eps"])
     if i == 1:
-      h = h + plain.swiglu(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+      gate = x @ w[p + "mlp.gate_proj.weight"].T + bias("mlp.gate_proj")
+      up = x @ w[p + "mlp.up_proj.weight"].T + bias("mlp.up_proj")
+      h = h + (torch.nn.functional.silu(gate) * up) @ w[p + "mlp.down_proj.weight"].T + bias("mlp.down_proj")
       continue
     logits = x @ w[p + "mlp.router.weight"].T
     probs = torch.softmax(logits, dim=-1)
