@@ -117,7 +117,7 @@ def run_mixed(args) -> int:
   hbm_gbs, mfma_tflops = ops.measured_peaks()
   engine = LLMEngine(model="", model_config=cfg, random_weights_seed=0, dtype=args.dtype, page_size=page_size,
                      num_pages=pages, max_num_seqs=args.num_seqs, max_model_len=max_len, max_num_batched_tokens=8192,
-                     enforce_eager=args.eager, tune_products=not args.no_tune)
+                     enforce_eager=args.eager, tune_products=not args.no_tune, enable_overlap=not args.no_overlap)
   rnd = Random(0)
   V = cfg.vocab_size
   prompts = [[rnd.randrange(V) for _ in range(rnd.randint(args.min_input, args.max_input))] for _ in range(args.num_seqs)]
@@ -152,7 +152,7 @@ def run_mixed(args) -> int:
                "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                "num_seqs": args.num_seqs, "min_input": args.min_input, "max_input": args.max_input,
                "output_len": args.output_len, "token_budget": 8192, "page_size": page_size, "pages": pages,
-               "graphs": not args.eager, "overlap": True, "temperature": 0.6},
+               "graphs": not args.eager, "overlap": not args.no_overlap, "temperature": 0.6},
     "weights_gbs": round(steps * (n["linear_params"] + n["head_params"]) * esize / dt / 1e9, 1),
     "frac_flops": round(flops / dt / PEAK_FLOPS[args.dtype], 4),
     "measured": {"hbm_gbs": round(hbm_gbs, 1), "mfma_bf16_tflops": round(mfma_tflops, 1)},
@@ -175,6 +175,7 @@ def main() -> int:
   ap.add_argument("--no-tune", action="store_true", help="choose product kernels by rule instead of timing them at start")
   ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
   ap.add_argument("--only-prefill", action="store_true", help="run only the 2,048-token prefill (for profiling)")
+  ap.add_argument("--no-overlap", action="store_true", help="read every step's tokens back before the next step is launched")
   ap.add_argument("--mixed", action="store_true", help="the serving workload: many requests, prompts and decodes mixed")
   ap.add_argument("--num-seqs", type=int, default=64)
   ap.add_argument("--min-input", type=int, default=128)
@@ -207,7 +208,7 @@ def main() -> int:
   pages = max_batch * (-(-room // page_size)) + 16
   engine = LLMEngine(model="", model_config=cfg, random_weights_seed=0, dtype=args.dtype, page_size=page_size,
                      num_pages=pages, max_num_seqs=max_batch, max_model_len=max_len, max_num_batched_tokens=8192,
-                     enforce_eager=args.eager, tune_products=not args.no_tune)
+                     enforce_eager=args.eager, tune_products=not args.no_tune, enable_overlap=not args.no_overlap)
   esize = 2 if args.dtype == "bfloat16" else 4
   if args.only_prefill:
     psec = time_prefill(engine, 2048, reps=max(1, args.steps), seed=2)
