@@ -395,7 +395,7 @@ __device__ __forceinline__ void prefill_body(
   // For head sizes that are multiples of 64 (pages hold 8 tokens or more) the 64 chunks of a wave lie in one page,
   // keys and values alike: the page number is then looked up once per wave with scalar instructions (from the
   // first lane's key), and the page's base address is scalar arithmetic instead of 64-bit vector arithmetic
-  // (a third of the vector instructions that fetching a macro tile took).
+  // (about a quarter of the vector instructions that fetching a macro tile took).
   constexpr bool PAGE_PER_WAVE = (D % 64) == 0;
 #define PREFILL_PAGES(J0)                                                                                            \
   {                                                                                                                  \
