@@ -168,7 +168,7 @@ def main() -> int:
   ap.add_argument("--warmup", type=int, default=8)
   ap.add_argument("--batch", type=int, default=8)
   ap.add_argument("--context", type=int, default=2048)
-  ap.add_argument("--preset", default="qwen3-0.6b")
+  ap.add_argument("--preset", default=None, help="default: qwen3-0.6b, and qwen3-8b for --mixed")
   ap.add_argument("--layers", type=int, default=None, help="fewer layers than the preset (named in the record)")
   ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
   ap.add_argument("--eager", action="store_true")
@@ -186,9 +186,9 @@ def main() -> int:
   if args.gpus != 1:
     print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
     return 2
+  if args.preset is None:
+    args.preset = "qwen3-8b" if args.mixed else "qwen3-0.6b"
   if args.mixed:
-    if args.preset == "qwen3-0.6b" and "--preset" not in sys.argv:
-      args.preset = "qwen3-8b"
     return run_mixed(args)
 
   import torch
