@@ -88,7 +88,7 @@ _SIGS = {
   "attention": {
     "mi_paged_attention": [c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                           c_void_p],
+                           c_int, c_void_p, c_void_p, c_void_p],
   },
 }
 
@@ -537,14 +537,24 @@ def norm_gemm_skinny(residual: torch.Tensor, x: Optional[torch.Tensor], norm_wei
 
 def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
                     v_pages: torch.Tensor, block_table: torch.Tensor, token_req: torch.Tensor, cu_q: torch.Tensor,
-                    kv_len: torch.Tensor, scale: float, window: int = 0) -> torch.Tensor:
+                    kv_len: torch.Tensor, scale: float, window: int = 0, num_splits: int = 1,
+                    part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None) -> torch.Tensor:
   """Causal attention of new tokens over their requests' paged keys and values.
 
   q: [T, >= nq*d] rows (the q part of a fused qkv buffer is fine), out [T, nq*d];
   key pages [num_pages, nkv, P, d], value pages [num_pages, nkv, d, P]; block_table [B, W] int32; token_req [T] = request of each token;
-  cu_q [B+1] = first token of each request; kv_len [B] = keys per request including the new tokens."""
+  cu_q [B+1] = first token of each request; kv_len [B] = keys per request including the new tokens.
+  num_splits > 1 cuts every token's keys into that many parts that run side by side (for few tokens over many
+  keys); then part_o float32 [>= T * nq * num_splits * d] and part_ml float32 [>= T * nq * num_splits * 2] are
+  scratch."""
   _dev(q, out, k_pages, v_pages, block_table, token_req, cu_q, kv_len)
   T = q.shape[0]
+  if num_splits > 1:
+    need = T * nq * num_splits
+    if part_o is None or part_ml is None or part_o.dtype != torch.float32 or part_ml.dtype != torch.float32 or \
+        part_o.numel() < need * d or part_ml.numel() < need * 2:
+      raise KernelError("paged_attention: partial buffers are missing, too small or not float32")
+    _dev(part_o, part_ml)
   B = kv_len.numel()
   if q.stride(1) != 1 or q.shape[1] < nq * d or out.stride(1) != 1 or out.shape != (T, nq * d):
     raise KernelError(f"paged_attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not hold {nq} heads of {d}")
@@ -561,7 +571,9 @@ def paged_attention(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tenso
   _check(lib, lib.mi_paged_attention(dtype_code(q.dtype), _ptr(q), q.stride(0), _ptr(out), out.stride(0),
                                      _ptr(k_pages), _ptr(v_pages), _ptr(block_table), block_table.shape[1],
                                      _ptr(token_req), _ptr(cu_q), _ptr(kv_len), T, B, nq, nkv, d,
-                                     k_pages.shape[2], float(scale), int(window), _stream()))
+                                     k_pages.shape[2], float(scale), int(window), int(num_splits),
+                                     _ptr(part_o) if num_splits > 1 else None,
+                                     _ptr(part_ml) if num_splits > 1 else None, _stream()))
   return out
 
 

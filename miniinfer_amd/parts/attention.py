@@ -107,8 +107,14 @@ class PagedAttention(Part):
     nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0
     table = ctx.block_tables[cache.group]
     if not ops.mfma_attention_supported(qkv.dtype, nq, nkv, d, cache.page_size):
+      T = qkv.shape[0]
+      splits = plain_splits(T * nq, min(ctx.max_kv_len, window) if window else ctx.max_kv_len)
+      part_o = part_ml = None
+      if splits > 1:
+        part_o = ctx.scratch("attn_part_o", T * nq * splits * d, torch.float32)
+        part_ml = ctx.scratch("attn_part_ml", T * nq * splits * 2, torch.float32)
       ops.paged_attention(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.token_req, ctx.cu_q, ctx.kv_len,
-                          self.scale, window)
+                          self.scale, window, splits, part_o, part_ml)
       return
     # entries with several tokens come first, single tokens last
     if ctx.num_multi > 0:
@@ -154,6 +160,15 @@ def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, wav
   if want == 1 and n < resident_workgroups and 5 * n <= 4 * resident_workgroups:
     want = 2
   return int(max(1, min(want, max(1, tiles // waves), 32)))
+
+
+def plain_splits(num_head_tokens: int, max_keys: int, resident_waves: int = 4096) -> int:
+  """Into how many key ranges the one-wave-per-(token, head) kernel cuts each token's keys: as many as fill the
+  chip's wave slots (16 on each of 256 compute units) once, each range at least two tiles of 64 keys, at most 64
+  ranges.  Prompt portions have waves enough and stay whole."""
+  want = resident_waves // max(1, num_head_tokens)
+  tiles = -(-max_keys // 64)
+  return int(max(1, min(want, tiles // 2, 64)))
 
 
 register_mixer("paged_attention", PagedAttention)

@@ -173,13 +173,15 @@ def _attention_ref(q, k, v, scale, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("splits", [1, 2, 3, 7])
 @pytest.mark.parametrize("nq,nkv,d,P,window", [(6, 3, 48, 16, 0), (8, 2, 128, 8, 0), (4, 4, 16, 4, 0), (5, 1, 80, 32, 0),
-                                               (4, 2, 64, 16, 37), (16, 8, 256, 16, 0)])
-def test_paged_attention(dtype, nq, nkv, d, P, window):
+                                               (4, 2, 64, 16, 37), (16, 8, 256, 16, 0), (4, 2, 64, 16, 150)])
+def test_paged_attention(dtype, nq, nkv, d, P, window, splits):
+  """Key ranges cut into parts (some of them empty for the short requests) give the same result as whole ones."""
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(5)
   # requests: (keys already cached, new tokens)
-  reqs = [(0, 70), (129, 1), (40, 3), (0, 1), (63, 2), (200, 1)]
+  reqs = [(0, 70), (129, 1), (40, 3), (0, 1), (63, 2), (200, 1), (447, 2)]
   B = len(reqs)
   kv_lens = [a + n for a, n in reqs]
   T = sum(n for _, n in reqs)
@@ -206,8 +208,10 @@ def test_paged_attention(dtype, nq, nkv, d, P, window):
   want = torch.cat(want, 0)
   out = torch.empty(T, nq * d, dtype=dtype, device=DEV)
   i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+  part_o = torch.full((T * nq * splits * d,), float("nan"), device=DEV) if splits > 1 else None
+  part_ml = torch.full((T * nq * splits * 2,), float("nan"), device=DEV) if splits > 1 else None
   ops.paged_attention(q.to(DEV), nq, nkv, d, out, kp.to(DEV), vp.transpose(2, 3).contiguous().to(DEV), table.to(DEV),
-                      i32(token_req), i32(cu), i32(kv_lens), d ** -0.5, window)
+                      i32(token_req), i32(cu), i32(kv_lens), d ** -0.5, window, splits, part_o, part_ml)
   torch.testing.assert_close(out.double().cpu(), want, **(_tol(dtype) if dtype == torch.bfloat16
                                                            else dict(rtol=1e-5, atol=1e-5)))
 

@@ -189,3 +189,15 @@ def test_layer_windows_follow_the_config_keys():
   a = plain.qwen3_logits(toks, w, cfg)
   b = plain.qwen3_logits(toks, w, dict(cfg, layer_types=["full_attention"] * 4))
   assert torch.allclose(a[:40], b[:40], atol=1e-5) and (a[40:] - b[40:]).abs().max() > 1e-3
+
+
+def test_plain_attention_key_ranges():
+  """The one-wave-per-head kernel's key ranges: whole for prompt portions and short contexts, cut for few tokens
+  over many keys, never shorter than two tiles, never more than 64."""
+  from miniinfer_amd.parts.attention import plain_splits
+  assert plain_splits(2048 * 16, 2048) == 1
+  assert plain_splits(8 * 16, 100) == 1
+  assert plain_splits(8 * 16, 2048) == 16
+  assert plain_splits(1, 700) == 5
+  assert plain_splits(1, 1 << 20) == 64
+  assert plain_splits(4096, 1 << 20) == 1
