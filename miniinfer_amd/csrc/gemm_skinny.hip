@@ -494,3 +494,332 @@ MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t ld
   return mi_gemm_skinny_ex(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, nullptr, 0, 0.f, nullptr, nullptr,
                            nullptr, nullptr, stream);
 }
+
+// ================================================================ the same product with k split across workgroups
+// For more than 16 rows of A the kernel above pays for its left operand: every workgroup owns whole rows of the
+// result, so it reads all of A, and what a compute unit draws from L2 between its weight loads is what the time
+// grows with.  Here a workgroup owns SK_WN blocks of 16 weight rows and only a range of k: grid (row groups,
+// splits).  The A columns of a chunk of SK_KC k's are read once per workgroup, coalesced, into LDS (two buffers: the
+// next chunk's loads and the next chunk's weights are in flight while the current chunk is multiplied), every wave
+// takes its operands from there, and a wave's weights come straight from global memory as above.  Each workgroup
+// leaves a 32-bit partial result P[split][m][n]; a second kernel adds the partials of a result element in the
+// order of the splits (so the sum does not depend on timing) and applies the same endings as the kernel above:
+// row scale from partial sums of squares, gate|up activation, or residual add + next operand + sums of squares.
+constexpr int SK_KC = 128;
+constexpr int SK_STEPS = SK_KC / 32;
+constexpr int SK_STRIDE = SK_KC + 8;      // LDS row stride in elements: 16 rows of an operand read spread over the banks
+constexpr int SK_MAX_CHUNKS = 32;         // chunks of one split at most: columns per split <= 4096
+
+// A wave owns RB blocks of 16 weight rows, a workgroup WN waves: 16 RB WN weight rows share every A chunk, and what
+// a compute unit fetches beside its weights (the A columns, from L2) shrinks with that number: the time of this
+// product follows the bytes a compute unit fetches, weights and A alike.
+// D chunks are on their way at any time: chunk c + D (its A columns into staging registers, its weights into
+// operand registers) is asked for when chunk c has been multiplied.  Loads come back in the order they were asked
+// for, so the A columns of a chunk are asked for together with its weights, D chunks ahead, and waiting for them
+// leaves the D - 1 later chunks in flight.
+template <int MB, int WN, int RB, int D>
+__global__ __launch_bounds__(64 * WN) void gemm_splitk_kernel(const uint16_t* __restrict__ A, int64_t lda,
+                                                              const uint16_t* __restrict__ W, int64_t ldw,
+                                                              float* __restrict__ P, int64_t ldp, void* __restrict__ C,
+                                                              int64_t ldc, int out_f32, int M, int N, int K, int kr) {
+  __shared__ __attribute__((aligned(16))) uint16_t a_lds[2][16 * MB * SK_STRIDE];
+  constexpr int THREADS = 64 * WN;
+  constexpr int ROWS_PER_PASS = THREADS / (SK_KC / 8);            // A rows that one load per thread covers
+  constexpr int A_LOADS = (16 * MB + ROWS_PER_PASS - 1) / ROWS_PER_PASS;
+  static_assert(THREADS % (SK_KC / 8) == 0, "a pass of the staging loads covers whole rows");
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.x * WN + wave) * 16 * RB;
+  const int split = blockIdx.y;
+  const int k_lo = split * kr;
+  const int k_hi = min(K, k_lo + kr);
+  const int nchunks = k_hi > k_lo ? (k_hi - k_lo + SK_KC - 1) / SK_KC : 0;
+
+  const uint16_t* wrow_base[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    int wr = n0 + 16 * rb + (lane & 15);
+    wr = wr < N ? wr : N - 1;                   // rows past the end read the last row; they are never stored
+    wrow_base[rb] = W + (int64_t)wr * ldw;
+  }
+
+  // this thread's pieces of an A chunk: 16 bytes of rows r0, r0 + ROWS_PER_PASS, ... at column 8 c16 of the chunk
+  const int r0 = threadIdx.x / (SK_KC / 8), c16 = threadIdx.x % (SK_KC / 8);
+  const int a_dst = r0 * SK_STRIDE + 8 * c16;
+
+  f32x4 acc[RB][MB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 a_st[D][A_LOADS];
+  bf16x8 w[D][RB][SK_STEPS];
+  // Loads are unconditional (a load inside a branch would end the straight-line code in which the compiler can
+  // count the loads on their way): a piece outside the range reads a valid address instead and is zeroed afterwards.
+  const int r_last = M - 1;
+#define SK_FETCH(CH, SLOT)                                                                                    \
+  {                                                                                                           \
+    const int k0_ = k_lo + (CH) * SK_KC;                                                                      \
+    const int ka = min(k0_ + 8 * c16, K - 8);                                                                 \
+    _Pragma("unroll") for (int i = 0; i < A_LOADS; ++i) {                                                     \
+      const int r = min(r0 + i * ROWS_PER_PASS, r_last);                                                      \
+      a_st[SLOT][i] = *reinterpret_cast<const u32x4*>(A + (int64_t)r * lda + ka);                             \
+    }                                                                                                         \
+    _Pragma("unroll") for (int s = 0; s < SK_STEPS; ++s) {                                                    \
+      const int k = min(k0_ + 32 * s + 8 * (lane >> 4), K - 8);                                               \
+      _Pragma("unroll") for (int rb = 0; rb < RB; ++rb)                                                       \
+        w[SLOT][rb][s] = *reinterpret_cast<const bf16x8*>(wrow_base[rb] + k);                                 \
+    }                                                                                                         \
+  }
+// zeroes what SK_FETCH read from outside the chunk's range (rows past M, columns past k_hi)
+#define SK_MASK(CH, SLOT)                                                                                     \
+  {                                                                                                           \
+    const int k0_ = k_lo + (CH) * SK_KC;                                                                      \
+    const bool col_ok = k0_ + 8 * c16 < k_hi;                                                                 \
+    _Pragma("unroll") for (int i = 0; i < A_LOADS; ++i)                                                       \
+      if (!(col_ok && r0 + i * ROWS_PER_PASS < M)) a_st[SLOT][i] = u32x4{0, 0, 0, 0};                         \
+    _Pragma("unroll") for (int s = 0; s < SK_STEPS; ++s)                                                      \
+      if (!(k0_ + 32 * s + 8 * (lane >> 4) < k_hi)) {                                                         \
+        _Pragma("unroll") for (int rb = 0; rb < RB; ++rb) w[SLOT][rb][s] = zero_bf16x8();                     \
+      }                                                                                                       \
+  }
+#pragma unroll
+  for (int j = 0; j < D; ++j) SK_FETCH(j, j)      // chunks past the range read clamped addresses and are never used
+  // The chunks are written out one after the other, with an exit after each: a loop would make the compiler wait
+  // for all loads but the newest at its head (it cannot count loads in flight around a back edge), and the D chunks
+  // on their way would shrink to one.  A split holds at most SK_MAX_CHUNKS chunks (the host cuts k accordingly).
+#define SK_CHUNK(CI)                                                                                          \
+  {                                                                                                           \
+    constexpr int j = (CI) % D;                                                                               \
+    uint16_t* buf = a_lds[(CI) & 1];                                                                          \
+    SK_MASK(CI, j)                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < A_LOADS; ++i)                                                       \
+      if (r0 + i * ROWS_PER_PASS < 16 * MB)                                                                   \
+        *reinterpret_cast<u32x4*>(buf + a_dst + i * ROWS_PER_PASS * SK_STRIDE) = a_st[j][i];                  \
+    __syncthreads(); /* the chunk is in LDS; every wave is past the chunk before last, whose buffer is next */ \
+    _Pragma("unroll") for (int s = 0; s < SK_STEPS; ++s) {                                                    \
+      _Pragma("unroll") for (int mb = 0; mb < MB; ++mb) {                                                     \
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(buf + (16 * mb + (lane & 15)) * SK_STRIDE + 32 * s + \
+                                                          8 * (lane >> 4));                                   \
+        _Pragma("unroll") for (int rb = 0; rb < RB; ++rb)                                                     \
+          acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j][rb][s], a, acc[rb][mb], 0, 0, 0);        \
+      }                                                                                                       \
+    }                                                                                                         \
+    if ((CI) + D < SK_MAX_CHUNKS) SK_FETCH((CI) + D, j)                                                       \
+    if (nchunks <= (CI) + 1) goto chunks_done;                                                                \
+  }
+  if (nchunks <= 0) goto chunks_done;
+  SK_CHUNK(0) SK_CHUNK(1) SK_CHUNK(2) SK_CHUNK(3) SK_CHUNK(4) SK_CHUNK(5) SK_CHUNK(6) SK_CHUNK(7)
+  SK_CHUNK(8) SK_CHUNK(9) SK_CHUNK(10) SK_CHUNK(11) SK_CHUNK(12) SK_CHUNK(13) SK_CHUNK(14) SK_CHUNK(15)
+  SK_CHUNK(16) SK_CHUNK(17) SK_CHUNK(18) SK_CHUNK(19) SK_CHUNK(20) SK_CHUNK(21) SK_CHUNK(22) SK_CHUNK(23)
+  SK_CHUNK(24) SK_CHUNK(25) SK_CHUNK(26) SK_CHUNK(27) SK_CHUNK(28) SK_CHUNK(29) SK_CHUNK(30) SK_CHUNK(31)
+  static_assert(SK_MAX_CHUNKS == 32, "one SK_CHUNK per chunk of a split");
+chunks_done:
+#undef SK_CHUNK
+#undef SK_MASK
+#undef SK_FETCH
+  // lane holds C^T[n0 + 16 rb + 4 (lane / 16) + i][16 mb + lane % 16]
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    if (n0 + 16 * rb >= N) break;   // a block past the last row (the row groups round N up) is not stored
+    const int n = n0 + 16 * rb + 4 * (lane >> 4);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = 16 * mb + (lane & 15);
+      if (m >= M) continue;
+      if (C) {            // one split: the result itself
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) {
+            if (out_f32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n + i] = acc[rb][mb][i];
+            else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n + i] = float_to_bf16_bits(acc[rb][mb][i]);
+          }
+      } else {            // ldp covers whole blocks of 16 columns: columns past N are written and never read
+        *reinterpret_cast<f32x4*>(P + ((int64_t)split * M + m) * ldp + n) = acc[rb][mb];
+      }
+    }
+  }
+}
+
+// Adds the partials and finishes the product.  Grid (ceil(N / 256), ceil(M / 4)), 4 waves: wave w takes row
+// 4 blockIdx.y + w, a lane 4 columns.  N counts result columns; with gate_up the partials hold 2 N (gate | up).
+struct SplitkEnd {
+  const float* row_ss;      // [ss_parts][ss_row]: scale row m by rsqrt(sum_p row_ss[p][m] / K + eps)
+  int ss_parts;
+  int ss_row;
+  float eps;
+  float* residual;          // [M, N]: residual += result; a_out = bf16(residual * norm_weight); ss_out[blockIdx.x][m]
+  const float* norm_weight;
+  uint16_t* a_out;
+  float* ss_out;            // [gridDim.x][ss_row]
+};
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ P, int64_t ldp, int S,
+                                                            void* __restrict__ C, int64_t ldc, int out_f32, int gate_up,
+                                                            int M, int N, int K, SplitkEnd e) {
+  const int lane = threadIdx.x & 63;
+  const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int n = blockIdx.x * 256 + 4 * lane;
+  if (m >= M) return;                         // whole waves leave: no barrier below
+  const bool live = n < N;                    // N is not a multiple of 4 in general: the last piece is partly live
+  float ssum = 0.f;
+  if (e.row_ss)
+    for (int p = lane; p < e.ss_parts; p += 64) ssum += e.row_ss[(int64_t)p * e.ss_row + m];
+  float r_old[4] = {0.f, 0.f, 0.f, 0.f}, nw[4] = {0.f, 0.f, 0.f, 0.f};
+  if (e.residual && live) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (n + i < N) {
+        r_old[i] = e.residual[(int64_t)m * N + n + i];
+        nw[i] = e.norm_weight[n + i];
+      }
+  }
+  f32x4 g = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      f32x4 pg[8], pu[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int s = s0 + j < S ? s0 + j : S - 1;        // a split again instead of a branch; it is not added
+        const float* row = P + ((int64_t)s * M + m) * ldp;
+        pg[j] = *reinterpret_cast<const f32x4*>(row + n);
+        if (gate_up) pu[j] = *reinterpret_cast<const f32x4*>(row + N + n);    // N % 4 == 0 is required for gate|up
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (s0 + j < S) {
+          g += pg[j];
+          if (gate_up) u += pu[j];
+        }
+    }
+  }
+  if (e.row_ss) {
+    const float rstd = rsqrtf(wave_sum(ssum) / (float)K + e.eps);
+    g *= rstd;
+    u *= rstd;
+  }
+  float v[4] = {g[0], g[1], g[2], g[3]};
+  if (gate_up) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = silu_f(v[i]) * u[i];
+  }
+  if (e.residual) {
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (live && n + i < N) {
+        const float rv = r_old[i] + v[i];
+        e.residual[(int64_t)m * N + n + i] = rv;
+        e.a_out[(int64_t)m * N + n + i] = float_to_bf16_bits(rv * nw[i]);
+        sq += rv * rv;
+      }
+    sq = wave_sum(sq);
+    if (lane == 0) e.ss_out[(int64_t)blockIdx.x * e.ss_row + m] = sq;
+    return;
+  }
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (n + i < N) {
+      if (out_f32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n + i] = v[i];
+      else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n + i] = float_to_bf16_bits(v[i]);
+    }
+}
+
+// How a product of M rows with a [rows, K] matrix (rows = 2 N for gate|up) is cut: waves per workgroup (blocks of 16
+// matrix rows), splits of k, columns per split, and the leading dimension of the partials.
+struct SplitkPlan {
+  int wn, rb, splits, kr, groups;
+  int64_t ldp;
+};
+
+static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
+  SplitkPlan p;
+  // weight rows per workgroup: 128 for matrices of many rows, 32 for those of few (which need the workgroups)
+  const bool wide = rows >= 2048;
+  p.wn = wide ? 4 : 2;
+  p.rb = wide ? 2 : 1;
+  const int tn = 16 * p.wn * p.rb;
+  p.groups = (rows + tn - 1) / tn;
+  const int target = 2 * compute_units();
+  int s = want_splits > 0 ? want_splits : (target + p.groups / 2) / p.groups;
+  if (s < 1) s = 1;
+  if (s > 32) s = 32;
+  int kr = ((K + s - 1) / s + 31) / 32 * 32;
+  if (kr < 256) kr = 256;
+  if (kr > SK_MAX_CHUNKS * SK_KC) kr = SK_MAX_CHUNKS * SK_KC;
+  p.kr = kr;
+  p.splits = (K + kr - 1) / kr;
+  p.ldp = (int64_t)(rows + 15) / 16 * 16;
+  return p;
+}
+
+// What a caller needs before a call of mi_gemm_skinny_v: rows of ss_out / row_ss that this product leaves when it
+// is the first half of a norm (`ss_parts`), and the floats of scratch it needs (0 for variant 0).
+MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K, int* ss_parts, int64_t* scratch_floats) {
+  MI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_plan: M=%d N=%d K=%d", M, N, K);
+  MI_REQUIRE(variant == 0 || variant == 1, "gemm_skinny_plan: variant %d", variant);
+  if (variant == 0) {
+    if (ss_parts) *ss_parts = skinny_grid(gate_up != 0, N, M).groups;
+    if (scratch_floats) *scratch_floats = 0;
+    return 0;
+  }
+  const SplitkPlan p = splitk_plan(M, gate_up ? 2 * N : N, K, 0);
+  if (ss_parts) *ss_parts = (N + 255) / 256;
+  if (scratch_floats) *scratch_floats = (int64_t)p.splits * M * p.ldp;
+  return 0;
+}
+
+// mi_gemm_skinny_ex with a choice of kernel: variant 0 = every workgroup owns whole rows of the result (above),
+// variant 1 = k split across workgroups, partial results in `scratch` (float, at least the plan's scratch_floats),
+// added in the order of the splits by a second kernel that also does the endings.
+MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void* A, int64_t lda, const void* W,
+                               int64_t ldw, void* C, int64_t ldc, int M, int N, int K, const float* row_ss,
+                               int ss_parts, float eps, float* residual, const float* norm_weight, void* a_out,
+                               float* ss_out, float* scratch, int64_t scratch_floats, hipStream_t stream) {
+  if (variant == 0)
+    return mi_gemm_skinny_ex(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual,
+                             norm_weight, a_out, ss_out, stream);
+  MI_REQUIRE(variant == 1, "gemm_skinny: variant %d", variant);
+  MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
+  MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);
+  MI_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K, "gemm_skinny: row strides (%lld, %lld)",
+             (long long)lda, (long long)ldw);
+  MI_REQUIRE(!gate_up || N % 4 == 0, "gemm_skinny: a gate|up product with k split needs a multiple of 4 columns, got %d",
+             N);
+  MI_REQUIRE(residual || (C && ldc >= N), "gemm_skinny: no result buffer");
+  MI_REQUIRE(!residual || (norm_weight && a_out && ss_out && !gate_up),
+             "gemm_skinny: the residual form needs norm_weight, a_out and ss_out, and no gate|up");
+  MI_REQUIRE(!row_ss || ss_parts > 0, "gemm_skinny: row_ss without parts");
+  if (M == 0) return 0;
+  const int rows = gate_up ? 2 * N : N;
+  const SplitkPlan p = splitk_plan(M, rows, K, 0);
+  MI_REQUIRE(scratch && scratch_floats >= (int64_t)p.splits * M * p.ldp,
+             "gemm_skinny: %lld floats of scratch, %lld are needed", (long long)scratch_floats,
+             (long long)p.splits * M * p.ldp);
+  const int MB = (M + 15) / 16;
+  const dim3 grid(p.groups, p.splits);
+#define GO(mb, wn, rb, d)                                                                                       \
+  gemm_splitk_kernel<mb, wn, rb, d><<<grid, 64 * wn, 0, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W,   \
+                                                                  ldw, scratch, p.ldp, nullptr, ldc, out_f32, M, \
+                                                                  rows, K, p.kr)
+  if (p.wn == 4) {
+    if (MB == 1) GO(1, 4, 2, 4);
+    else if (MB == 2) GO(2, 4, 2, 3);
+    else if (MB == 3) GO(3, 4, 2, 3);
+    else GO(4, 4, 2, 3);
+  } else {
+    if (MB == 1) GO(1, 2, 1, 4);
+    else if (MB == 2) GO(2, 2, 1, 4);
+    else if (MB == 3) GO(3, 2, 1, 3);
+    else GO(4, 2, 1, 3);
+  }
+#undef GO
+  MI_CHECK_LAUNCH("gemm_skinny (k split)");
+  const SplitkEnd e{row_ss, ss_parts, SS_ROW(M), eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
+  splitk_reduce_kernel<<<dim3((N + 255) / 256, (M + 3) / 4), 256, 0, stream>>>(scratch, p.ldp, p.splits, C, ldc, out_f32,
+                                                                              gate_up, M, N, K, e);
+  MI_CHECK_LAUNCH("gemm_skinny (k split, sum)");
+  return 0;
+}

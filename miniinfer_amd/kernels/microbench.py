@@ -38,7 +38,11 @@ def cmd_product(args) -> int:
   turn = [0]
 
   def ours():
-    ops.gemm_skinny(a, ws[turn[0] % copies], out, gate_up=args.gate_up)
+    ops.gemm_skinny(a, ws[turn[0] % copies], out, gate_up=args.gate_up, variant=0)
+    turn[0] += 1
+
+  def ours_ksplit():
+    ops.gemm_skinny(a, ws[turn[0] % copies], out, gate_up=args.gate_up, variant=1)
     turn[0] += 1
 
   def library():
@@ -46,7 +50,7 @@ def cmd_product(args) -> int:
     turn[0] += 1
 
   calls = copies * max(1, args.calls // copies)
-  for name, fn in (("gemm_skinny", ours), ("library", library)):
+  for name, fn in (("gemm_skinny", ours), ("gemm_skinny with k split", ours_ksplit), ("library", library)):
     t = graph_time_us(fn, calls)
     print(f"{name}: rows {args.rows}, weights [{rows_w}, {args.k}] {nbytes / 1e6:.1f} MB: {t:.1f} us, "
           f"{nbytes / t / 1e6:.2f} TB/s" + (" (without the activation)" if name == "library" and args.gate_up else ""))
@@ -87,7 +91,7 @@ def cmd_decode_attention(args) -> int:
   per_req = -(-L // P)
   pages = B * per_req
   cache_bytes = 2 * pages * nkv * P * d * 2
-  copies = max(2, min(8, (1536 << 20) // cache_bytes))
+  copies = args.copies or max(2, min(8, (1536 << 20) // cache_bytes))
   g = torch.Generator(device=DEV).manual_seed(0)
   caches = [(torch.randn(pages + 1, nkv, P, d, device=DEV, generator=g).bfloat16(),
              torch.randn(pages + 1, nkv, d, P, device=DEV, generator=g).bfloat16()) for _ in range(copies)]
@@ -167,6 +171,8 @@ def main(argv=None) -> int:
   d.add_argument("--page-size", type=int, default=16)
   d.add_argument("--splits", type=int, default=0, help="key ranges per request (default: the engine's choice)")
   d.add_argument("--calls", type=int, default=24)
+  d.add_argument("--copies", type=int, default=0,
+                 help="caches the calls cycle through, as a model's layers do (default: 2 to 8, 1.5 GB at most)")
   d.set_defaults(fn=cmd_decode_attention)
   c = sub.add_parser("choices", help="own against library kernel for each product of a preset's model")
   c.add_argument("--preset", default="qwen3-0.6b")

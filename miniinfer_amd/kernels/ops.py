@@ -112,6 +112,10 @@ _SIGS["gemm_skinny"]["mi_gemm_skinny_ex"] = [c_int, c_int, c_void_p, c_int64, c_
                                              c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p,
                                              c_void_p, c_void_p]
 _SIGS["gemm_skinny"]["mi_gemm_skinny_groups"] = [c_int, c_int, c_int]
+_SIGS["gemm_skinny"]["mi_gemm_skinny_v"] = [c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
+                                            c_int, c_int, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_int64, c_void_p]
+_SIGS["gemm_skinny"]["mi_gemm_skinny_plan"] = [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]
 _SIGS["gemm_skinny"]["mi_gemm_skinny_ss_row"] = [c_int]
 _SIGS["gemm_skinny"]["mi_norm_gemm_skinny"] = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                                c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]
@@ -330,11 +334,17 @@ SKINNY_MAX_ROWS = 64
 SKINNY_OWN_ROWS = 16                 # without a measurement: up to here the weight-streaming kernel for every matrix,
 SKINNY_OWN_ELEMENTS = 8 << 20        # and for more rows (up to SKINNY_MAX_ROWS) while the matrix is smaller than this
 TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_products` times the two candidates
-_PRODUCT_CHOICE: Dict[tuple, bool] = {}  # (rows point, matrix rows, k, gate|up) -> the weight-streaming kernel is quicker
+# (rows point, matrix rows, k, gate|up) -> the quickest: LIBRARY, or this library's kernel in which every workgroup
+# owns whole rows of the result (OWN_ROWS), or the one that splits k across workgroups (OWN_KSPLIT)
+LIBRARY, OWN_ROWS, OWN_KSPLIT = 0, 1, 2
+_PRODUCT_CHOICE: Dict[tuple, int] = {}
+KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
+KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)
 
 
-def set_product_choice(rows_point: int, matrix_rows: int, k: int, gate_up: bool, own: bool) -> None:
-  _PRODUCT_CHOICE[(rows_point, matrix_rows, k, bool(gate_up))] = bool(own)
+def set_product_choice(rows_point: int, matrix_rows: int, k: int, gate_up: bool, choice) -> None:
+  """choice: LIBRARY / OWN_ROWS / OWN_KSPLIT (False and True stand for the first two)."""
+  _PRODUCT_CHOICE[(rows_point, matrix_rows, k, bool(gate_up))] = int(choice)
 
 
 def product_choice_known(matrix_rows: int, k: int, gate_up: bool) -> bool:
@@ -399,14 +409,55 @@ def skinny_preferred(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fa
     return False
   if _OWN_ONLY[0]:
     return True
+  c = _measured_choice(num_rows, matrix_rows, k, gate_up)
+  if c is not None:
+    return c != LIBRARY
+  return num_rows <= SKINNY_OWN_ROWS or matrix_rows * k < SKINNY_OWN_ELEMENTS
+
+
+def _measured_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> Optional[int]:
   if _PRODUCT_CHOICE:
     for p in TUNE_ROWS:
       if p >= num_rows:
-        c = _PRODUCT_CHOICE.get((p, matrix_rows, k, bool(gate_up)))
-        if c is not None:
-          return c
-        break
-  return num_rows <= SKINNY_OWN_ROWS or matrix_rows * k < SKINNY_OWN_ELEMENTS
+        return _PRODUCT_CHOICE.get((p, matrix_rows, k, bool(gate_up)))
+  return None
+
+
+def skinny_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> int:
+  """Which of this library's two kernels runs a product that `skinny_preferred` keeps: 0 = every workgroup owns whole
+  rows of the result and reads the whole left operand (which is what its time grows with beyond 16 rows); 1 = k is
+  split across workgroups, which read a slice of the left operand each and leave 32-bit partial results that a
+  second kernel adds in a fixed order.  Measured where `tuning.tune_products` has been; else by the rule above."""
+  if gate_up and (matrix_rows // 2) % 4:
+    return 0
+  c = _measured_choice(num_rows, matrix_rows, k, gate_up)
+  if c == OWN_ROWS:
+    return 0
+  if c == OWN_KSPLIT:
+    return 1
+  return 1 if num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K else 0
+
+
+_KSPLIT_SCRATCH: Dict[tuple, torch.Tensor] = {}
+
+
+def _ksplit_scratch(device, floats: int) -> torch.Tensor:
+  """Partial results of the k-split kernel.  Buffers are kept for good, one per device and size class: a captured
+  step holds the address of the one it was recorded with."""
+  size = max(1 << 16, 1 << (int(floats) - 1).bit_length())
+  key = (torch.device(device).index, size)
+  t = _KSPLIT_SCRATCH.get(key)
+  if t is None:
+    t = torch.empty(size, dtype=torch.float32, device=device)
+    _KSPLIT_SCRATCH[key] = t
+  return t
+
+
+def _skinny_plan(lib, variant: int, gate_up: bool, M: int, N: int, K: int) -> Tuple[int, int]:
+  """(rows of the table of partial sums of squares, floats of scratch) of a launch of the chosen kernel."""
+  parts, floats = ctypes.c_int(0), ctypes.c_int64(0)
+  _check(lib, lib.mi_gemm_skinny_plan(variant, 1 if gate_up else 0, M, N, K, ctypes.byref(parts), ctypes.byref(floats)))
+  return parts.value, floats.value
 
 
 def gemm_skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -417,10 +468,25 @@ def gemm_skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
           and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bool = False) -> torch.Tensor:
+def _skinny_call(lib, variant: int, out_f32: bool, gate_up: bool, a, w, c_ptr, ldc: int, M: int, N: int, K: int,
+                 row_ss=None, eps: float = 0.0, residual=None, norm_weight=None, a_out=None, ss_out=None) -> None:
+  scratch, floats = None, 0
+  if variant == 1:
+    _, floats = _skinny_plan(lib, 1, gate_up, M, N, K)
+    scratch = _ksplit_scratch(a.device, floats)
+  _check(lib, lib.mi_gemm_skinny_v(variant, 1 if out_f32 else 0, 1 if gate_up else 0, _ptr(a),
+                                   a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), c_ptr, ldc, M, N, K,
+                                   _ptr(row_ss), row_ss.shape[0] if row_ss is not None else 0, float(eps),
+                                   _ptr(residual), _ptr(norm_weight), _ptr(a_out), _ptr(ss_out), _ptr(scratch),
+                                   scratch.numel() if scratch is not None else 0, _stream()))
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bool = False,
+                variant: Optional[int] = None) -> torch.Tensor:
   """out[M, N] = a[M, K] @ w[N, K]^T on the matrix cores for M <= 64 rows, bfloat16 operands, bfloat16 or float32
   result.  With `gate_up`, w is a fused gate|up matrix [2 N, K] (gate rows first) and
-  out = silu(a @ w_gate^T) * (a @ w_up^T), made from the 32-bit sums."""
+  out = silu(a @ w_gate^T) * (a @ w_up^T), made from the 32-bit sums.  variant: see `skinny_variant` (default: its
+  answer for this shape)."""
   _dev(a, w, out)
   if not gemm_skinny_supported(a, w):
     raise KernelError(f"gemm_skinny does not take a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}")
@@ -433,14 +499,15 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bo
   if tuple(out.shape) != (M, N) or out.stride(1) != 1 or out.dtype not in (torch.bfloat16, torch.float32):
     raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit [{M}, {N}]")
   lib = _lib("gemm_skinny")
-  _check(lib, lib.mi_gemm_skinny(1 if out.dtype == torch.float32 else 0, 1 if gate_up else 0, _ptr(a),
-                                 a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), _ptr(out),
-                                 out.stride(0) if M > 1 else N, M, N, K, _stream()))
+  if variant is None:
+    variant = skinny_variant(M, w.shape[0], K, gate_up)
+  _skinny_call(lib, variant, out.dtype == torch.float32, gate_up, a, w, _ptr(out), out.stride(0) if M > 1 else N,
+               M, N, K)
   return out
 
 
 def gemm_skinny_scaled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_ss: torch.Tensor, eps: float,
-                       gate_up: bool = False) -> torch.Tensor:
+                       gate_up: bool = False, variant: Optional[int] = None) -> torch.Tensor:
   """`gemm_skinny` whose rows are scaled by rsqrt(sum_p row_ss[p, m] / K + eps) before they are stored (and, with
   `gate_up`, before the activation): the second half of an RMS norm whose first half `gemm_skinny_into_norm` did.
   row_ss float32 [parts, 16] for up to 16 rows, [parts, 64] for more."""
@@ -459,10 +526,10 @@ def gemm_skinny_scaled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_
   ss_row = lib.mi_gemm_skinny_ss_row(M)
   if row_ss.dtype != torch.float32 or row_ss.dim() != 2 or row_ss.shape[1] != ss_row or not row_ss.is_contiguous():
     raise KernelError(f"gemm_skinny_scaled: row_ss must be a contiguous float32 [parts, {ss_row}] for {M} rows")
-  _check(lib, lib.mi_gemm_skinny_ex(1 if out.dtype == torch.float32 else 0, 1 if gate_up else 0, _ptr(a),
-                                    a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), _ptr(out),
-                                    out.stride(0) if M > 1 else N, M, N, K, _ptr(row_ss), row_ss.shape[0], float(eps),
-                                    None, None, None, None, _stream()))
+  if variant is None:
+    variant = skinny_variant(M, w.shape[0], K, gate_up)
+  _skinny_call(lib, variant, out.dtype == torch.float32, gate_up, a, w, _ptr(out), out.stride(0) if M > 1 else N,
+               M, N, K, row_ss=row_ss, eps=eps)
   return out
 
 
@@ -474,7 +541,8 @@ def gemm_skinny_into_norm_supported(a: torch.Tensor, w: torch.Tensor, residual: 
           and norm_weight.numel() == N and norm_weight.is_contiguous())
 
 
-def gemm_skinny_into_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor):
+def gemm_skinny_into_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor,
+                          variant: Optional[int] = None):
   """residual += a @ w^T (in place, 32-bit), and the first half of the RMS norm of the new residual: returns
   (operand, row_ss) with operand[m, n] = bfloat16(residual[m, n] * norm_weight[n]) and row_ss float32 [parts, 16 or 64],
   the sum of squares of row m over each workgroup's columns.  `gemm_skinny_scaled` finishes the norm."""
@@ -484,12 +552,13 @@ def gemm_skinny_into_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tens
   M = a.shape[0]
   N, K = w.shape
   lib = _lib("gemm_skinny")
-  parts = lib.mi_gemm_skinny_groups(0, N, M)
+  if variant is None:
+    variant = skinny_variant(M, N, K)
+  parts, _ = _skinny_plan(lib, variant, False, M, N, K)
   operand = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
   row_ss = torch.empty((parts, lib.mi_gemm_skinny_ss_row(M)), dtype=torch.float32, device=a.device)
-  _check(lib, lib.mi_gemm_skinny_ex(0, 0, _ptr(a), a.stride(0) if M > 1 else a.shape[1], _ptr(w), w.stride(0), None,
-                                    N, M, N, K, None, 0, 0.0, _ptr(residual), _ptr(norm_weight), _ptr(operand),
-                                    _ptr(row_ss), _stream()))
+  _skinny_call(lib, variant, False, False, a, w, None, N, M, N, K, residual=residual, norm_weight=norm_weight,
+               a_out=operand, ss_out=row_ss)
   return operand, row_ss
 
 

@@ -1,10 +1,12 @@
 """Which kernel runs a product of few rows is measured, not guessed.
 
-For a matrix of tens of MB and a handful of rows there are two candidates: this library's weight-streaming kernel
-(`ops.gemm_skinny`, whose epilogue can take a norm's halves or the gated activation) and the library product
+For a matrix of tens of MB and a handful of rows there are three candidates: this library's weight-streaming kernel
+(`ops.gemm_skinny`, whose epilogue can take a norm's halves or the gated activation) in its two forms (every
+workgroup owns whole rows of the result, or k is split across workgroups and a second kernel adds the partial
+results), and the library product
 (hipBLASLt through `torch.matmul`, which splits k across workgroups and so reads the left operand less often, but
 needs the norm and the activation as kernels of their own).  Which is quicker depends on the shape and the number
-of rows in ways no short rule covers, so `tune_products` times both on the model's own matrices once, when an
+of rows in ways no short rule covers, so `tune_products` times them on the model's own matrices once, when an
 engine is built, and `ops.skinny_preferred` then answers from the table.  Matrices below `MIN_ELEMENTS` are not
 timed: there the weight-streaming kernel and its fusions win by the kernels they save.
 """
@@ -19,6 +21,7 @@ from . import ops
 
 MIN_ELEMENTS = 2 << 20
 UNFUSED_US = 3.0          # what a norm or activation kernel of its own costs inside a decode step
+KSPLIT_MARGIN = 0.9       # the k-split kernel replaces the library's product only if it takes at most this much of its time
 
 
 def graph_time_us(fn: Callable[[], None], calls: int, flush: Optional[torch.Tensor] = None) -> float:
@@ -78,20 +81,34 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
       out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
       turn = [0]
 
-      def own():
-        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up)
+      def own_rows():
+        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=0)
+        turn[0] += 1
+
+      def own_ksplit():
+        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=1)
         turn[0] += 1
 
       def library():
         torch.matmul(a, ws[turn[0] % len(ws)].t())
         turn[0] += 1
 
-      t_own = graph_time_us(own, calls, flush)
+      t_rows = graph_time_us(own_rows, calls, flush)
+      # k is split for more than 16 rows only: below, the left operand is too small for its re-reads to matter, and
+      # the second kernel costs more than they do
+      t_split = graph_time_us(own_ksplit, calls, flush) if M > 16 and not (gate_up and N % 4) else float("inf")
       t_lib = graph_time_us(library, calls, flush) + (2 if gate_up else 1) * UNFUSED_US
-      ops.set_product_choice(M, rows_w, K, gate_up, t_own <= t_lib)
+      # The two own kernels end alike, so they are compared as timed.  Against the library the k-split kernel must
+      # win by a tenth: inside a step of the 8B shape at 64 rows it lost 4 us a layer to the library's product for
+      # the down projection although it had won this timing by 3 us (its partial results are 17 MB there).
+      if t_split < t_rows:
+        choice = ops.OWN_KSPLIT if t_split <= KSPLIT_MARGIN * t_lib else ops.LIBRARY
+      else:
+        choice = ops.OWN_ROWS if t_rows <= t_lib else ops.LIBRARY
+      ops.set_product_choice(M, rows_w, K, gate_up, choice)
       if log is not None:
-        log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: own {t_own:.1f} us, "
-            f"library {t_lib:.1f} us with its extra kernels")
+        log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: own {t_rows:.1f} us, "
+            f"own with k split {t_split:.1f} us, library {t_lib:.1f} us with its extra kernels")
     timed += 1
   if timed:
     # give the timing's buffers back to the driver: what is allocated next (the cache pools) then lies as it would

@@ -265,10 +265,11 @@ def test_cache_is_sized_from_device_memory_when_no_page_count_is_given(tmp_path)
     LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, gpu_memory_utilization=1e-3)
 
 
-@pytest.mark.parametrize("products", ["own", "library"])
+@pytest.mark.parametrize("products", ["own", "own_ksplit", "library"])
 def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, products):
-  """The engine's choice between its own weight-streaming product and the library's is a matter of speed: with
-  every small product forced to either, each generated token is one the plain implementation all but ties for."""
+  """The engine's choice between its own weight-streaming products (whole rows per workgroup, or k split across
+  workgroups) and the library's is a matter of speed: with every small product forced to one of them, each generated
+  token is one the plain implementation all but ties for."""
   from miniinfer_amd import LLMEngine, SamplingParams
   from miniinfer_amd.kernels import ops
   cfg, w = _model(tmp_path, "B", dtype=torch.bfloat16)
@@ -280,11 +281,14 @@ def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, produ
       with ops.own_products_only():
         outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
     else:
+      choice = ops.OWN_KSPLIT if products == "own_ksplit" else ops.LIBRARY
       for rows in ops.TUNE_ROWS:
         for m in eng.model.products():
-          ops.set_product_choice(rows, m[0].shape[0], m[0].shape[1], m[1], own=False)
-      outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
-      ops.clear_product_choices()
+          ops.set_product_choice(rows, m[0].shape[0], m[0].shape[1], m[1], choice)
+      try:
+        outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
+      finally:
+        ops.clear_product_choices()
     ran_library = ops.library_products_run()[0] - before
     assert (ran_library > 0) == (products == "library")
   for p, o in zip(prompts, outs):

@@ -338,17 +338,18 @@ def test_mfma_attention_finds_a_far_key_and_respects_the_window_edge():
   torch.testing.assert_close(out[0, :d].float(), vp[page, 0, :, off].float(), rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("variant", [0, 1])      # whole rows of the result per workgroup / k split across workgroups
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (8, 4096, 1024), (16, 1024, 3072), (17, 500, 80), (64, 6144, 1024),
                                    (3, 151936, 256), (33, 48, 2048), (5, 130, 88), (64, 1000, 40), (7, 2050, 64),
-                                   (16, 1001, 512)])
-def test_gemm_skinny(M, N, K, out_dtype):
+                                   (16, 1001, 512), (48, 1024, 4360), (64, 100, 12288), (20, 2064, 1000)])
+def test_gemm_skinny(M, N, K, out_dtype, variant):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(9)
   a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
   w = (torch.randn(N, K, generator=g) * 0.1).bfloat16().to(DEV)
-  out = torch.empty(M, N, dtype=out_dtype, device=DEV)
-  ops.gemm_skinny(a, w, out)
+  out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+  ops.gemm_skinny(a, w, out, variant=variant)
   want = a.double() @ w.double().T
   if out_dtype == torch.float32:
     torch.testing.assert_close(out.double(), want, rtol=1e-4, atol=1e-4 * K ** 0.5)
@@ -356,14 +357,15 @@ def test_gemm_skinny(M, N, K, out_dtype):
     torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 112, 80), (40, 160, 96), (64, 100, 256)])
-def test_gemm_skinny_gate_up_activation(M, I, K):
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 112, 80), (40, 160, 96), (64, 100, 256), (33, 1028, 2200)])
+def test_gemm_skinny_gate_up_activation(M, I, K, variant):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(10)
   x = torch.randn(M, K, generator=g).bfloat16().to(DEV)
   w = (torch.randn(2 * I, K, generator=g) * 0.1).bfloat16().to(DEV)
-  out = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
-  ops.gemm_skinny(x, w, out, gate_up=True)
+  out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+  ops.gemm_skinny(x, w, out, gate_up=True, variant=variant)
   gu = x.double() @ w.double().T
   want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
   torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
@@ -469,8 +471,10 @@ def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, win
 
 @pytest.mark.parametrize("M,N,K,N2,gate_up", [(8, 1024, 2048, 6144, True), (1, 80, 96, 112, False), (16, 1024, 3072, 4096, False),
                                                (40, 136, 264, 200, True), (64, 1024, 2048, 3072, False), (5, 88, 40, 24, False),
-                                               (12, 2056, 96, 160, True)])
-def test_norm_split_between_two_products(M, N, K, N2, gate_up):
+                                               (12, 2056, 96, 160, True), (64, 1024, 3072, 4096, False),
+                                               (33, 520, 2304, 132, True)])
+@pytest.mark.parametrize("variants", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_norm_split_between_two_products(M, N, K, N2, gate_up, variants):
   """residual += a W1^T; y = rmsnorm(residual) * w; out = y W2^T (or the gated activation of it), the add and the
   norm done half in the first product's kernel and half in the second's.  Against 64-bit arithmetic with the
   kernels' rounding points restated: the second product's left operand is bfloat16(residual * w), and the row's
@@ -485,12 +489,12 @@ def test_norm_split_between_two_products(M, N, K, N2, gate_up):
   w2 = (torch.randn(2 * N2 if gate_up else N2, N, generator=g) * 0.1).bfloat16().to(DEV)
   want_r = r.double() + a.double() @ w1.double().T
   r_dev = r.clone()
-  operand, row_ss = ops.gemm_skinny_into_norm(a, w1, r_dev, nw)
+  operand, row_ss = ops.gemm_skinny_into_norm(a, w1, r_dev, nw, variant=variants[0])
   torch.testing.assert_close(r_dev.double(), want_r, rtol=1e-5, atol=1e-4)
   torch.testing.assert_close(operand.double(), (r_dev.double() * nw.double()).bfloat16().double(), rtol=1e-2, atol=1e-6)
   torch.testing.assert_close(row_ss[:, :M].sum(0).double(), r_dev.double().pow(2).sum(-1), rtol=1e-5, atol=1e-5)
   out = torch.empty(M, N2, dtype=torch.bfloat16, device=DEV)
-  ops.gemm_skinny_scaled(operand, w2, out, row_ss, eps, gate_up=gate_up)
+  ops.gemm_skinny_scaled(operand, w2, out, row_ss, eps, gate_up=gate_up, variant=variants[1])
   rstd = torch.rsqrt(r_dev.double().pow(2).mean(-1, keepdim=True) + eps)
   y = (operand.double() @ w2.double().T) * rstd
   # ... which is the norm followed by the product, up to the operand's rounding
@@ -524,7 +528,7 @@ def test_microbench_commands_run_at_small_sizes(capsys):
   assert microbench.main(["decode-attention", "--batch", "3", "--context", "300", "--heads", "4", "--kv-heads", "2",
                           "--head-dim", "64", "--calls", "4"]) == 0
   out = capsys.readouterr().out
-  assert out.count("gemm_skinny:") == 2 and "attn_prefill dense" in out and "attn_decode_front" in out
+  assert out.count("gemm_skinny:") == 2 and out.count("gemm_skinny with k split:") == 2 and "attn_prefill dense" in out and "attn_decode_front" in out
 
 
 def test_measured_peaks_are_plausible():

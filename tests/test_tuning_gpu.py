@@ -35,10 +35,11 @@ def test_products_are_timed_once_per_shape_and_small_ones_are_left_alone(clean_c
   assert not ops.skinny_preferred(65, 2048, 1024)
 
 
-@pytest.mark.parametrize("own", [True, False])
+@pytest.mark.parametrize("choice", [0, 1, 2])     # the library / whole rows per workgroup / k split across workgroups
 @pytest.mark.parametrize("M", [3, 16, 40])
-def test_either_choice_gives_the_product(clean_choices, own, M):
+def test_either_choice_gives_the_product(clean_choices, choice, M):
   ops = clean_choices
+  own = choice != ops.LIBRARY
   from miniinfer_amd.parts.linear import gate_up_activation, linear
   g = torch.Generator().manual_seed(M)
   N, K, inter = 192, 160, 112
@@ -46,9 +47,10 @@ def test_either_choice_gives_the_product(clean_choices, own, M):
   wgu = (torch.randn(2 * inter, K, generator=g) * 0.1).bfloat16()
   x = torch.randn(M, K, generator=g).bfloat16()
   for p in ops.TUNE_ROWS:
-    ops.set_product_choice(p, N, K, False, own)
-    ops.set_product_choice(p, 2 * inter, K, True, own)
+    ops.set_product_choice(p, N, K, False, choice)
+    ops.set_product_choice(p, 2 * inter, K, True, choice)
   assert ops.skinny_preferred(M, N, K) == own and ops.skinny_preferred(M, 2 * inter, K, True) == own
+  assert ops.skinny_variant(M, N, K) == (1 if choice == ops.OWN_KSPLIT else 0)
   y = linear(x.to(DEV), w.to(DEV))
   torch.testing.assert_close(y.double().cpu(), x.double() @ w.double().T, rtol=2e-2, atol=2e-2)
   a = gate_up_activation(x.to(DEV), wgu.to(DEV))
