@@ -67,6 +67,50 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
   }
 }
 
+// The same product for up to 16 rows of A (a decode step of the 32-bit path), where the 64 x 64 tiles above would
+// leave the chip idle: a workgroup takes 16 rows of W and all rows of A, one result element per thread, chunks of
+// 64 k through LDS with the next chunk's loads in flight.  Every element is summed over k in the same order, with
+// the same fused multiply-adds, as in the kernel above: a row's result is bit for bit what it is there.
+#define FK 64
+template <typename TA, typename TC>
+__global__ __launch_bounds__(256) void gemm_nt_few_rows_kernel(const TA* __restrict__ A, int64_t lda,
+                                                               const TA* __restrict__ W, int64_t ldw,
+                                                               TC* __restrict__ C, int64_t ldc, int M, int N, int K) {
+  __shared__ float As[16][FK + 1];
+  __shared__ float Ws[16][FK + 1];
+  const int tid = threadIdx.x;
+  const int m = tid >> 4;          // the thread's row of A (and the row of A it loads)
+  const int nl = tid & 15;         // its row of W within the workgroup's 16
+  const int n0 = blockIdx.x * 16;
+  const int lk = (tid & 15) * 4;   // first k of the chunk that it loads: rows tid / 16 of A and of W
+  const bool a_ok = m < M, w_ok = n0 + m < N;
+  const TA* arow = A + (int64_t)(a_ok ? m : 0) * lda;
+  const TA* wrow = W + (int64_t)(w_ok ? n0 + m : 0) * ldw;
+  float ar[4], wr[4];
+#define FEW_FETCH(K0)                                                                          \
+  _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                              \
+    const int k = (K0) + lk + j;                                                               \
+    ar[j] = (a_ok && k < K) ? to_float(arow[k]) : 0.f;                                         \
+    wr[j] = (w_ok && k < K) ? to_float(wrow[k]) : 0.f;                                         \
+  }
+  FEW_FETCH(0)
+  float acc = 0.f;
+  for (int k0 = 0; k0 < K; k0 += FK) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      As[m][lk + j] = ar[j];
+      Ws[m][lk + j] = wr[j];
+    }
+    __syncthreads();
+    if (k0 + FK < K) FEW_FETCH(k0 + FK)
+#pragma unroll
+    for (int kk = 0; kk < FK; ++kk) acc = fmaf(As[m][kk], Ws[nl][kk], acc);
+    __syncthreads();
+  }
+#undef FEW_FETCH
+  if (m < M && n0 + nl < N) C[(int64_t)m * ldc + n0 + nl] = from_float<TC>(acc);
+}
+
 // in_dtype: dtype of A and W; out_dtype: dtype of C.
 MI_EXPORT int mi_gemm_nt(int in_dtype, int out_dtype, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                          int64_t ldc, int M, int N, int K, hipStream_t stream) {
@@ -74,14 +118,24 @@ MI_EXPORT int mi_gemm_nt(int in_dtype, int out_dtype, const void* A, int64_t lda
   MI_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_nt: leading dimensions (%lld, %lld, %lld) too small for K=%d N=%d",
              (long long)lda, (long long)ldw, (long long)ldc, K, N);
   if (M == 0) return 0;
-  dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
+  const bool few = M <= 16;
+  dim3 grid(few ? ceil_div(N, 16) : ceil_div(N, BN), few ? 1 : ceil_div(M, BM));
   MI_REQUIRE(grid.y <= 65535, "gemm_nt: M=%d too large for one launch", M);
-#define LAUNCH(TA, TC)                                                                                         \
-  gemm_nt_kernel<TA, TC><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TA*)W, ldw, (TC*)C, ldc, M, N, K)
-  if (in_dtype == MI_DTYPE_F32 && out_dtype == MI_DTYPE_F32) LAUNCH(float, float);
-  else if (in_dtype == MI_DTYPE_BF16 && out_dtype == MI_DTYPE_BF16) LAUNCH(bf16, bf16);
-  else if (in_dtype == MI_DTYPE_BF16 && out_dtype == MI_DTYPE_F32) LAUNCH(bf16, float);
-  else MI_FAIL("gemm_nt: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+#define LAUNCH(TA, TC)                                                                                              \
+  if (few)                                                                                                          \
+    gemm_nt_few_rows_kernel<TA, TC><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TA*)W, ldw, (TC*)C, ldc, M, \
+                                                              N, K);                                               \
+  else                                                                                                              \
+    gemm_nt_kernel<TA, TC><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TA*)W, ldw, (TC*)C, ldc, M, N, K)
+  if (in_dtype == MI_DTYPE_F32 && out_dtype == MI_DTYPE_F32) {
+    LAUNCH(float, float);
+  } else if (in_dtype == MI_DTYPE_BF16 && out_dtype == MI_DTYPE_BF16) {
+    LAUNCH(bf16, bf16);
+  } else if (in_dtype == MI_DTYPE_BF16 && out_dtype == MI_DTYPE_F32) {
+    LAUNCH(bf16, float);
+  } else {
+    MI_FAIL("gemm_nt: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+  }
 #undef LAUNCH
   MI_CHECK_LAUNCH("gemm_nt");
   return 0;

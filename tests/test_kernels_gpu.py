@@ -97,6 +97,21 @@ def test_gemm_nt(dtype, M, N, K):
                              atol=1e-4 if dtype == torch.float32 else 1e-1)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,K", [(130, 96), (1000, 1030), (48, 17)])
+def test_gemm_nt_rows_do_not_depend_on_the_batch(dtype, N, K):
+  """Few rows go to a kernel of their own (one result element per thread), many to the tiled one: both add a result
+  element's products in the same order, so a row's result is the same bits whichever kernel ran it."""
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(4)
+  a = torch.randn(40, K, generator=g).to(dtype).to(DEV)
+  w = torch.randn(N, K, generator=g).to(dtype).to(DEV)
+  many = ops.gemm_nt(a, w, torch.empty(40, N, dtype=torch.float32, device=DEV))
+  for rows in (1, 7, 16):
+    few = ops.gemm_nt(a[:rows], w, torch.full((rows, N), float("nan"), dtype=torch.float32, device=DEV))
+    assert torch.equal(few, many[:rows])
+
+
 def _rope_ref(x, pos, theta, rotary_dim):
   """Complex multiplication by e^{i pos theta^(-2j/rd)} on pairs (j, j + rd/2): the statement of the
   reference's test helper (tests/utils.py:12-17,65-116)."""
