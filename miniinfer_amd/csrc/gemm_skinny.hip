@@ -642,8 +642,8 @@ chunks_done:
   }
 }
 
-// Adds the partials and finishes the product.  Grid (ceil(N / 256), ceil(M / 4)), 4 waves: wave w takes row
-// 4 blockIdx.y + w, a lane 4 columns.  N counts result columns; with gate_up the partials hold 2 N (gate | up).
+// Adds the partials and finishes the product.  Grid (ceil(N / 256), ceil(M / waves)), 1 or 4 waves a workgroup (one
+// where that still leaves few workgroups): wave w takes row waves * blockIdx.y + w, a lane 4 columns.  N counts result columns; with gate_up the partials hold 2 N (gate | up).
 struct SplitkEnd {
   const float* row_ss;      // [ss_parts][ss_row]: scale row m by rsqrt(sum_p row_ss[p][m] / K + eps)
   int ss_parts;
@@ -659,7 +659,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
                                                             void* __restrict__ C, int64_t ldc, int out_f32, int gate_up,
                                                             int M, int N, int K, SplitkEnd e) {
   const int lane = threadIdx.x & 63;
-  const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int m = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int n = blockIdx.x * 256 + 4 * lane;
   if (m >= M) return;                         // whole waves leave: no barrier below
   const bool live = n < N;                    // N is not a multiple of 4 in general: the last piece is partly live
@@ -742,7 +742,9 @@ static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
   p.rb = wide ? 2 : 1;
   const int tn = 16 * p.wn * p.rb;
   p.groups = (rows + tn - 1) / tn;
-  const int target = 2 * compute_units();
+  // one workgroup for every compute unit: with twice as many (and half the k range each) every shape measured was
+  // slower, by 5 to 25%
+  const int target = compute_units();
   int s = want_splits > 0 ? want_splits : (target + p.groups / 2) / p.groups;
   if (s < 1) s = 1;
   if (s > 32) s = 32;
@@ -818,8 +820,9 @@ MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void
 #undef GO
   MI_CHECK_LAUNCH("gemm_skinny (k split)");
   const SplitkEnd e{row_ss, ss_parts, SS_ROW(M), eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
-  splitk_reduce_kernel<<<dim3((N + 255) / 256, (M + 3) / 4), 256, 0, stream>>>(scratch, p.ldp, p.splits, C, ldc, out_f32,
-                                                                              gate_up, M, N, K, e);
+  const int red_waves = (int64_t)((N + 255) / 256) * M <= 2048 ? 1 : 4;
+  splitk_reduce_kernel<<<dim3((N + 255) / 256, (M + red_waves - 1) / red_waves), 64 * red_waves, 0, stream>>>(
+      scratch, p.ldp, p.splits, C, ldc, out_f32, gate_up, M, N, K, e);
   MI_CHECK_LAUNCH("gemm_skinny (k split, sum)");
   return 0;
 }
