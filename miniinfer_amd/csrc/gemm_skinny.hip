@@ -6,6 +6,8 @@
 // from global memory into its operand slot (no LDS staging), and the few rows of A (which stay in L2)
 // fill the other operand.  A workgroup owns 16 * RB weight rows; its waves split K and add their partial
 // blocks through LDS.  32-bit accumulation; the result is stored as bfloat16 or float32.
+// A second form, further down, splits K across workgroups instead (for 17 to 64 rows of A, where reading all of A
+// in every workgroup is what the first form's time grows with); mi_gemm_skinny_v takes either.
 //
 // With GATE_UP, W is a fused gate|up matrix [2 N, K] (gate rows first) and the result is the feed-forward's
 // activation C[m, n] = silu(A W_gate^T)[m, n] * (A W_up^T)[m, n] (kernels/triton/silu_mul.py:33-37 of the
