@@ -55,12 +55,13 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   const int wave = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
   // GATE_UP: RB == 2, row block 0 = gate rows n0.., row block 1 = up rows N + n0..; N counts output columns
-  // rpg: rows of W per workgroup and row block when RB == 1 or GATE_UP: 16, or fewer so that the workgroups fill
-  // whole rounds of the compute units (the lanes of the other rows then load nothing and their results are dropped)
-  constexpr bool CUT = GATE_UP || RB == 1;
-  const int n0 = CUT ? blockIdx.x * rpg : blockIdx.x * 16 * RB;
-  const int n_end = min(N, n0 + (CUT ? rpg : 16 * RB));
-  const bool w_live = !CUT || (lane & 15) < rpg;
+  // rpg: rows of W per workgroup and row block: 16, or fewer so that the workgroups fill whole rounds of the
+  // compute units (the lanes of the other rows then load nothing and their results are dropped).  Row block rb
+  // starts at row n0 + rb * rpg (GATE_UP: at n0 of its half).
+  constexpr int BLOCKS = GATE_UP ? 1 : RB;        // row blocks side by side in the result
+  const int n0 = blockIdx.x * rpg * BLOCKS;
+  const int n_end = min(N, n0 + rpg * BLOCKS);
+  const bool w_live = (lane & 15) < rpg;
   const int steps = (K + 31) / 32;
   const int spw = (steps + nw - 1) / nw;
   const int s_begin = wave * spw;
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   const uint16_t* wrow[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    int row = GATE_UP ? n0 + (lane & 15) : n0 + 16 * rb + (lane & 15);
+    int row = GATE_UP ? n0 + (lane & 15) : n0 + rpg * rb + (lane & 15);
     row = row < N ? row : N - 1;            // rows past the end read the last row; they are never stored
     if (GATE_UP && rb == 1) row += N;
     wrow[rb] = W + (int64_t)row * ldw;
@@ -105,9 +106,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     for (int j = 0; j < 2; ++j) {
       const int e = threadIdx.x + j * blockDim.x;
       const int blk = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-      const int n = n0 + 16 * (blk / MB) + 4 * (ln >> 4) + i;
+      const int r = 4 * (ln >> 4) + i;            // row within its block
+      const int n = n0 + rpg * (blk / MB) + r;
       const int m = 16 * (blk % MB) + (ln & 15);
-      if (e < OBLK * 256 && n < n_end && m < M) {
+      if (e < OBLK * 256 && r < rpg && n < n_end && m < M) {
         r_pre[j] = nh.residual[(int64_t)m * N + n];
         w_pre[j] = nh.norm_weight[n];
       }
@@ -193,7 +195,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       if (GATE_UP) u += red[(w * RB * MB + MB + blk) * 256 + r];
     }
     const int ln = r >> 2, i = r & 3;
-    const int n = n0 + 16 * (GATE_UP ? 0 : blk / MB) + 4 * (ln >> 4) + i;
+    const int rr = 4 * (ln >> 4) + i;             // row within its block
+    const int n = n0 + rpg * (GATE_UP ? 0 : blk / MB) + rr;
     const int m = 16 * (blk % MB) + (ln & 15);
     if (nh.row_ss) {
       float total = 0.f;
@@ -203,7 +206,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       u *= rstd;
     }
     if (GATE_UP) v = silu_f(v) * u;
-    const bool live = n < n_end && m < M;
+    const bool live = rr < rpg && n < n_end && m < M;
     if (nh.residual) {
       float rv = 0.f;
       if (live) {
@@ -406,19 +409,40 @@ static int compute_units() {
 
 static SkinnyGrid skinny_grid(bool gate_up, int N, int M) {
   const int row_blocks = (N + 15) / 16;
+  const int cus = compute_units();
   SkinnyGrid g;
-  g.RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
   g.rpg = 16;
-  if ((gate_up || g.RB == 1) && M <= 16) {
+  if (gate_up) {
+    g.RB = 2;
+    if (M <= 16) {
+      const int rounds = (N + 16 * cus - 1) / (16 * cus);
+      const int rpg = (N + cus * rounds - 1) / (cus * rounds);
+      g.rpg = rpg < 4 ? 4 : (rpg > 16 ? 16 : rpg);
+    }
+    g.groups = (N + g.rpg - 1) / g.rpg;
+  } else if (M <= 16 && row_blocks < 1024) {
     // A workgroup of 16 waves has a compute unit to itself, so the launch runs in rounds of as many workgroups as
     // there are units, and 320 workgroups take as long as 512.  The rows are shared out so that the last round is
-    // as full as the others: 5,120 rows on 256 units go as 512 groups of 10, 1,024 rows as 256 groups of 4.
-    const int cus = compute_units();
-    const int rounds = (N + 16 * cus - 1) / (16 * cus);
-    const int rpg = (N + cus * rounds - 1) / (cus * rounds);
-    g.rpg = rpg < 4 ? 4 : (rpg > 16 ? 16 : rpg);
+    // as full as the others, up to 32 to a workgroup (two row blocks, which halves what the left operand's reads
+    // add to the weights'): 1,024 rows on 256 units go as 256 groups of 4, 5,120 rows as 256 groups of 2 x 10,
+    // 10,240 rows as 512 groups of 2 x 10.
+    // (With fewer than 4 rows the left operand is a small part of the bytes, and the finer cut's extra workgroups
+    // win: a row block each, then.)
+    const int most = M < 4 ? 16 : 32;
+    const int rounds = (N + most * cus - 1) / (most * cus);
+    const int per_group = (N + cus * rounds - 1) / (cus * rounds);      // at most `most`
+    if (per_group <= 16) {
+      g.RB = 1;
+      g.rpg = per_group < 4 ? 4 : per_group;
+    } else {
+      g.RB = 2;
+      g.rpg = (per_group + 1) / 2;
+    }
+    g.groups = (N + g.rpg * g.RB - 1) / (g.rpg * g.RB);
+  } else {
+    g.RB = row_blocks >= 1024 ? 2 : 1;
+    g.groups = (row_blocks + g.RB - 1) / g.RB;
   }
-  g.groups = (gate_up || g.RB == 1) ? (N + g.rpg - 1) / g.rpg : (row_blocks + g.RB - 1) / g.RB;
   return g;
 }
 
