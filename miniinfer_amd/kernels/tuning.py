@@ -94,9 +94,9 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
         turn[0] += 1
 
       t_rows = graph_time_us(own_rows, calls, flush)
-      # k is split for more than 16 rows only: below, the left operand is too small for its re-reads to matter, and
-      # the second kernel costs more than they do
-      t_split = graph_time_us(own_ksplit, calls, flush) if M > 16 and not (gate_up and N % 4) else float("inf")
+      # k is split from 16 rows up only: below, the left operand is too small for its re-reads to matter, and the
+      # second kernel costs more than they do (at 16 rows it wins where k is long: 68 against 76 us for [5120, 25600])
+      t_split = graph_time_us(own_ksplit, calls, flush) if M >= 16 and not (gate_up and N % 4) else float("inf")
       t_lib = graph_time_us(library, calls, flush) + (2 if gate_up else 1) * UNFUSED_US
       # The two own kernels end alike, so they are compared as timed.  Against the library the k-split kernel must
       # win by a tenth: inside a step of the 8B shape at 64 rows it lost 4 us a layer to the library's product for
