@@ -48,9 +48,11 @@ constexpr int D = HEAD_DIM;
 #if HEAD_DIM <= 128
 #define DECODE_OCCUPANCY __attribute__((amdgpu_waves_per_eu(2)))
 #define PREFILL_DENSE_OCCUPANCY __attribute__((amdgpu_waves_per_eu(3)))
+#define PREFILL_WIDE 1          // a third prefill instance: two blocks of query columns per wave, two waves per SIMD
 #else
 #define DECODE_OCCUPANCY
 #define PREFILL_DENSE_OCCUPANCY
+#define PREFILL_WIDE 0          // (its accumulators alone would fill the registers of head sizes above 128)
 #endif
 constexpr int KSTEPS = D / 32;          // 16x16x32 products over the head dim
 constexpr bool KREM = (D % 32) != 0;    // plus one more, half of it zeros
@@ -530,6 +532,17 @@ template <int NB>
 __global__ __launch_bounds__(256) PREFILL_DENSE_OCCUPANCY void prefill_dense_kernel(PREFILL_ARGS) {
   prefill_body<NB, 1>(PREFILL_PASS);
 }
+
+// Long prompts (many workgroups for every compute unit): every wave takes two blocks of 16 query columns, so a
+// tile's operands, read from LDS once per wave, serve twice the products (what the instances above wait for is
+// those LDS reads and the vector work of fetching a tile, the same per tile whatever a wave multiplies it with):
+// 246 registers at head size 128, two waves per SIMD, no spills.  32,768 tokens: 789 against 665 TFLOP/s; 8,192:
+// 672 against 619; for short prompts it has too few workgroups (2,048 tokens: 82 against 52 us).
+#if PREFILL_WIDE
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void prefill_wide_kernel(PREFILL_ARGS) {
+  prefill_body<2, 1>(PREFILL_PASS);
+}
+#endif
 #undef PREFILL_ARGS
 #undef PREFILL_PASS
 
@@ -959,13 +972,21 @@ MI_EXPORT int mi_attn_prefill_tokens_per_block(int nq, int nkv) {
   return gpad > 16 ? 0 : 4 * (16 * PREFILL_NB / gpad);
 }
 
+// The same for the instance with two column blocks per wave (variant 3 of mi_attn_prefill); 0 where there is none.
+MI_EXPORT int mi_attn_prefill_tokens_per_block_wide(int nq, int nkv) {
+  const int gpad = group_pad(nq, nkv);
+  return (gpad > 16 || !PREFILL_WIDE) ? 0 : 4 * (32 / gpad);
+}
+
 MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, int64_t out_row_stride, const void* k_pages,
                               const void* v_pages, const int* block_table, int table_width, const int* work,
                               int num_work, const int* cu_q, const int* kv_len, int nq, int nkv, int page_size,
                               float scale, int window, int variant, hipStream_t stream) {
-  // variant: 0 = chosen from the grid's size; 1 = 8 waves, two macro tiles a step; 2 = 4 waves, three waves a SIMD
+  // variant: 0 = chosen from the grid's size; 1 = 8 waves, two macro tiles a step; 2 = 4 waves, three waves a SIMD;
+  // 3 = 4 waves with two column blocks each (its work items count mi_attn_prefill_tokens_per_block_wide tokens)
   if (check_common("attn_prefill", nq, nkv, page_size, q_row_stride, out_row_stride, table_width)) return 1;
-  MI_REQUIRE(variant >= 0 && variant <= 2, "attn_prefill: variant %d", variant);
+  MI_REQUIRE(variant >= 0 && variant <= 3, "attn_prefill: variant %d", variant);
+  MI_REQUIRE(variant != 3 || PREFILL_WIDE, "attn_prefill: head size %d has no instance with two column blocks", D);
   if (check_scale("attn_prefill", scale)) return 1;
   MI_REQUIRE(num_work >= 0 && window >= 0, "attn_prefill: bad work count or window");
   MI_REQUIRE(num_work <= 65535, "attn_prefill: %d work items; the grid takes at most 65535", num_work);
@@ -979,6 +1000,16 @@ MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, in
         compute_units <= 0)
       compute_units = 256;
   }
+#if PREFILL_WIDE
+  if (variant == 3) {
+    prefill_wide_kernel<<<grid, 256, 0, stream>>>(
+        (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,
+        (const uint16_t*)v_pages, block_table, table_width, work, cu_q, kv_len, nq, nkv, group_pad(nq, nkv),
+        log2_of(page_size), scale, window);
+    MI_CHECK_LAUNCH("attn_prefill");
+    return 0;
+  }
+#endif
   if (variant == 2 || (variant == 0 && (int64_t)num_work * nkv > 2 * (int64_t)compute_units))
     prefill_dense_kernel<PREFILL_NB><<<grid, 256, 0, stream>>>(
         (const uint16_t*)q, q_row_stride, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages,

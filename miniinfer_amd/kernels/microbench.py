@@ -74,10 +74,14 @@ def cmd_prefill_attention(args) -> int:
   tpb = ops.attn_prefill_tokens_per_block(nq, nkv, d)
   work = torch.tensor([(0, i) for i in reversed(range(-(-L // tpb)))], dtype=torch.int32, device=DEV)
   flops = 4 * nq * d * L * (L + 1) / 2
-  for variant in ("two_tiles", "dense"):
-    t = graph_time_us(lambda: ops.attn_prefill(q, nq, nkv, d, out, kp, vp, table, work, cu, kv, d ** -0.5, 0,
+  tpb_wide = ops.attn_prefill_tokens_per_block(nq, nkv, d, wide=True)
+  work_wide = torch.tensor([(0, i) for i in reversed(range(-(-L // tpb_wide)))], dtype=torch.int32, device=DEV) \
+      if tpb_wide else None
+  for variant in ("two_tiles", "dense") + (("wide",) if tpb_wide else ()):
+    wk = work_wide if variant == "wide" else work
+    t = graph_time_us(lambda: ops.attn_prefill(q, nq, nkv, d, out, kp, vp, table, wk, cu, kv, d ** -0.5, 0,
                                                variant=variant), args.calls)
-    print(f"attn_prefill {variant}: {L} tokens, {nq}/{nkv} heads of {d}, {len(work) * nkv} workgroups: {t:.1f} us, "
+    print(f"attn_prefill {variant}: {L} tokens, {nq}/{nkv} heads of {d}, {len(wk) * nkv} workgroups: {t:.1f} us, "
           f"{flops / t / 1e6:.0f} TFLOP/s")
   return 0
 

@@ -101,6 +101,7 @@ _SIGS["attention_mfma"] = {
                            c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int,
                            c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
   "mi_attn_prefill_tokens_per_block": [c_int, c_int],
+  "mi_attn_prefill_tokens_per_block_wide": [c_int, c_int],
 }
 
 _SIGS["gemm_skinny"] = {
@@ -689,10 +690,24 @@ def mfma_attention_supported(dtype: torch.dtype, nq: int, nkv: int, d: int, page
           and page_size >= 8)
 
 
-def attn_prefill_tokens_per_block(nq: int, nkv: int, d: int) -> int:
-  """Query tokens one work item of the prefill launch takes (the granule of its work list)."""
+def attn_prefill_tokens_per_block(nq: int, nkv: int, d: int, wide: bool = False) -> int:
+  """Query tokens one work item of the prefill launch takes (the granule of its work list).  wide: of the variant
+  "wide", whose waves take two blocks of query columns (0 where the head size has no such instance)."""
   lib = _lib("attention_mfma", (("HEAD_DIM", d),))
-  return lib.mi_attn_prefill_tokens_per_block(nq, nkv)
+  return lib.mi_attn_prefill_tokens_per_block_wide(nq, nkv) if wide else lib.mi_attn_prefill_tokens_per_block(nq, nkv)
+
+
+PREFILL_WIDE_MIN_WORKGROUPS = 1024     # from here on (four for every compute unit) the "wide" prefill variant pays
+
+
+def attn_prefill_wide_pays(q_lens, nq: int, nkv: int, d: int) -> int:
+  """The work granule of the "wide" prefill variant if the step's prompt portions make workgroups enough for it
+  (long prompts: 672 against 619 TFLOP/s at 8,192 tokens, 789 against 665 at 32,768), else 0."""
+  tpb = attn_prefill_tokens_per_block(nq, nkv, d, wide=True)
+  if tpb <= 0:
+    return 0
+  items = sum(-(-n // tpb) for n in q_lens if n > 1)
+  return tpb if items * nkv >= PREFILL_WIDE_MIN_WORKGROUPS else 0
 
 
 def attn_decode_geometry(d: int):
@@ -718,7 +733,7 @@ def _attn_common(what, q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, 
   return B
 
 
-_PREFILL_VARIANTS = {"auto": 0, "two_tiles": 1, "dense": 2}
+_PREFILL_VARIANTS = {"auto": 0, "two_tiles": 1, "dense": 2, "wide": 3}
 
 
 def attn_prefill(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
@@ -726,7 +741,9 @@ def attn_prefill(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, 
                  kv_len: torch.Tensor, scale: float, window: int = 0, variant: str = "auto") -> None:
   """MFMA attention of the entries named in `work` [n, 2] = (entry, block of `attn_prefill_tokens_per_block` query
   tokens within it).  Other arguments as `paged_attention`.  variant: "auto" (by the number of work items),
-  "two_tiles" (8 waves a workgroup, for few work items) or "dense" (4 waves, three waves a SIMD)."""
+  "two_tiles" (8 waves a workgroup, for few work items), "dense" (4 waves, three waves a SIMD) or "wide" (4 waves
+  with two blocks of query columns each, for long prompts; its work items count
+  `attn_prefill_tokens_per_block(.., wide=True)` tokens)."""
   if variant not in _PREFILL_VARIANTS:
     raise KernelError(f"attn_prefill: variant {variant!r}; known: {sorted(_PREFILL_VARIANTS)}")
   _attn_common("attn_prefill", q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len)

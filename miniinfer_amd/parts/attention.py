@@ -118,8 +118,10 @@ class PagedAttention(Part):
       return
     # entries with several tokens come first, single tokens last
     if ctx.num_multi > 0:
-      work = ctx.prefill_work(ops.attn_prefill_tokens_per_block(nq, nkv, d))
-      ops.attn_prefill(qkv, nq, nkv, d, out, cache.k, cache.v, table, work, ctx.cu_q, ctx.kv_len, self.scale, window)
+      wide = ops.attn_prefill_wide_pays(ctx.q_lens[:ctx.num_multi], nq, nkv, d)
+      work = ctx.prefill_work(wide or ops.attn_prefill_tokens_per_block(nq, nkv, d))
+      ops.attn_prefill(qkv, nq, nkv, d, out, cache.k, cache.v, table, work, ctx.cu_q, ctx.kv_len, self.scale, window,
+                       variant="wide" if wide else "auto")
     n_single = ctx.num_requests - ctx.num_multi
     if n_single > 0:
       self._attend_decode(qkv, out, ctx, cache, ctx.num_multi, n_single)

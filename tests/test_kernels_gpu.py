@@ -279,13 +279,20 @@ MFMA_SHAPES = [(16, 8, 128, 16, 0), (6, 3, 48, 16, 0), (8, 2, 32, 8, 0), (4, 4, 
                (16, 1, 64, 16, 0), (12, 4, 96, 64, 0), (4, 2, 256, 16, 0), (8, 4, 128, 16, 50), (6, 2, 64, 8, 17)]
 
 
-@pytest.mark.parametrize("variant", ["two_tiles", "dense"])
+@pytest.mark.parametrize("variant", ["two_tiles", "dense", "wide"])
 @pytest.mark.parametrize("nq,nkv,d,P,window", MFMA_SHAPES)
 def test_mfma_prefill_attention(nq, nkv, d, P, window, variant):
   from miniinfer_amd.kernels import ops
   reqs = [(0, 70), (129, 2), (40, 33), (0, 2), (63, 17), (300, 5), (0, 200), (190, 130)]
   c = _paged_case(reqs, nq, nkv, d, P, window, seed=6)
-  tpb = ops.attn_prefill_tokens_per_block(nq, nkv, d)
+  tpb = ops.attn_prefill_tokens_per_block(nq, nkv, d, wide=variant == "wide")
+  if tpb == 0:
+    assert variant == "wide" and d > 128       # head sizes above 128 have no instance with two column blocks
+    with pytest.raises(ops.KernelError):
+      ops.attn_prefill(c["q"], nq, nkv, d, torch.zeros(c["T"], nq * d, dtype=torch.bfloat16, device=DEV), c["kp"],
+                       c["vp"], c["table"], torch.zeros(1, 2, dtype=torch.int32, device=DEV), c["cu"], c["kv"],
+                       d ** -0.5, window, variant=variant)
+    return
   work = [(b, i) for b, n in enumerate(c["q_lens"]) for i in range(-(-n // tpb))]
   out = torch.zeros(c["T"], nq * d, dtype=torch.bfloat16, device=DEV)
   ops.attn_prefill(c["q"], nq, nkv, d, out, c["kp"], c["vp"], c["table"],

@@ -96,6 +96,27 @@ def test_regime(tmp_path, name, dtype, regime):
       _bf16_check(got[rid], want[rid], f"{name} {regime} request {rid}")
 
 
+@pytest.mark.parametrize("name", ["B", "C", "D"])
+def test_prefill_variant_for_long_prompts_through_the_engine(tmp_path, name, monkeypatch):
+  """The prefill attention's instance with two blocks of query columns per wave is chosen for steps with thousands of
+  workgroups; with the threshold lowered to one, the tiny configurations run through it, whole and mixed."""
+  from miniinfer_amd.kernels import ops
+  monkeypatch.setattr(ops, "PREFILL_WIDE_MIN_WORKGROUPS", 1)
+  seen = []
+  real = ops.attn_prefill
+  monkeypatch.setattr(ops, "attn_prefill", lambda *a, **k: (seen.append(k.get("variant")), real(*a, **k))[1])
+  cfg, w = tm.make_model(str(tmp_path / "m"), name, seed=7, dtype=torch.bfloat16, std=0.05)
+  requests = _requests(name, cfg)
+  want = _plain_logits(cfg, w, requests)
+  for regime in ("whole", "mixed"):
+    steps = REGIMES[regime](requests)
+    outs = _replay(tmp_path / "m", "bfloat16", steps, requests, tm.PAGE_SIZE[name], tt.peak_tokens(steps, requests))
+    got = tt.gather(steps, outs, requests, cfg["vocab_size"])
+    for rid in requests:
+      _bf16_check(got[rid], want[rid], f"{name} wide prefill {regime} request {rid}")
+  assert seen and all(v == "wide" for v in seen)
+
+
 def _drawn_config(rng):
   """A Qwen3 configuration with every size drawn: head sizes that are and are not multiples of 16, any number of heads
   and groups, widths and vocabularies that are no powers of two, windows in some layers."""
