@@ -174,7 +174,9 @@ def main() -> int:
   ap.add_argument("--eager", action="store_true")
   ap.add_argument("--no-tune", action="store_true", help="choose product kernels by rule instead of timing them at start")
   ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
-  ap.add_argument("--only-prefill", action="store_true", help="run only the 2,048-token prefill (for profiling)")
+  ap.add_argument("--only-prefill", action="store_true", help="run only the prefill (for profiling)")
+  ap.add_argument("--prefill-tokens", type=int, default=2048,
+                  help="with --only-prefill: tokens of the prompt (one step of that many tokens; default 2,048)")
   ap.add_argument("--no-overlap", action="store_true", help="read every step's tokens back before the next step is launched")
   ap.add_argument("--mixed", action="store_true", help="the serving workload: many requests, prompts and decodes mixed")
   ap.add_argument("--num-seqs", type=int, default=64)
@@ -201,19 +203,23 @@ def main() -> int:
   layers = cfg.num_hidden_layers
   hbm_gbs, mfma_tflops = ops.measured_peaks()     # what a bare read loop and a bare matrix-core loop reach here
   mfma_flops = mfma_tflops * 1e12 if args.dtype == "bfloat16" else None
+  if args.only_prefill:
+    args.context, args.batch, args.no_points = max(args.context, args.prefill_tokens), 1, True
   max_batch = max(args.batch, 1 if args.no_points else 64)
   page_size = 16
   room = args.context + args.steps + args.warmup + (-(-max_batch * args.context // 8192)) + 16
   max_len = max(4096, room)
   pages = max_batch * (-(-room // page_size)) + 16
   engine = LLMEngine(model="", model_config=cfg, random_weights_seed=0, dtype=args.dtype, page_size=page_size,
-                     num_pages=pages, max_num_seqs=max_batch, max_model_len=max_len, max_num_batched_tokens=8192,
+                     num_pages=pages, max_num_seqs=max_batch, max_model_len=max_len,
+                     max_num_batched_tokens=max(8192, args.prefill_tokens if args.only_prefill else 0),
                      enforce_eager=args.eager, tune_products=not args.no_tune, enable_overlap=not args.no_overlap)
   esize = 2 if args.dtype == "bfloat16" else 4
   if args.only_prefill:
-    psec = time_prefill(engine, 2048, reps=max(1, args.steps), seed=2)
-    fl = prefill_flops(cfg, layers, 2048)
-    print(json.dumps({"prefill": {"value": round(2048 / psec, 1), "tokens": 2048, "ms": round(psec * 1e3, 3),
+    T = args.prefill_tokens
+    psec = time_prefill(engine, T, reps=max(1, args.steps), seed=2)
+    fl = prefill_flops(cfg, layers, T)
+    print(json.dumps({"prefill": {"value": round(T / psec, 1), "tokens": T, "ms": round(psec * 1e3, 3),
                                   "frac": round(fl / psec / PEAK_FLOPS[args.dtype], 4),
                                   "frac_measured": round(fl / psec / mfma_flops, 4) if mfma_flops else None}}))
     return 0
