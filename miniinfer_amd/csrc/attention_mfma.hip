@@ -285,7 +285,12 @@ __device__ __forceinline__ void store_output(const State<NB>& st, uint16_t* out_
 #ifndef PREFILL_NB
 #define PREFILL_NB 1
 #endif
-constexpr int LDS_KSTR = D + 8;                  // elements per key row in LDS
+// Elements per key row in LDS.  An operand read takes 16 bytes per lane from 16 rows (lanes l and l + 16 read
+// neighbouring pieces of a row); the LDS serves lanes l .. l + 3 and l + 16 .. l + 19 together, so these 4 rows x 2
+// pieces must fall into different banks: a row stride of 8 (mod 16) banks of 4 bytes, D + 16 elements for head
+// sizes that are multiples of 32 and D itself for the others.  (With D + 8 a third of the kernel's LDS cycles
+// were bank conflicts of these reads: SQ_LDS_BANK_CONFLICT 2.0e8 against 0.7e8 for 16,384 tokens.)
+constexpr int LDS_KSTR = (D % 32 == 0) ? D + 16 : D;
 constexpr int LDS_VSTR = MKEYS + 4;              // elements per dim row of the transposed values in LDS: rows 2 banks
                                                  // apart, so the 16 rows x 8 bytes of an operand read hit 32 banks
 constexpr int LDS_KCHUNKS = MKEYS * (D / 8);     // 16-byte chunks of a key tile

@@ -533,7 +533,10 @@ MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t ld
 // row scale from partial sums of squares, gate|up activation, or residual add + next operand + sums of squares.
 constexpr int SK_KC = 128;
 constexpr int SK_STEPS = SK_KC / 32;
-constexpr int SK_STRIDE = SK_KC + 8;      // LDS row stride in elements: 16 rows of an operand read spread over the banks
+// LDS row stride in elements.  An operand read takes 16 bytes per lane from 16 rows, and the LDS serves lanes l .. l + 3
+// and l + 16 .. l + 19 (the next 16 bytes of the same rows) together: 4 rows x 2 pieces fall into different banks when
+// the stride is 8 (mod 16) banks of 4 bytes.
+constexpr int SK_STRIDE = SK_KC + 16;
 constexpr int SK_MAX_CHUNKS = 32;         // chunks of one split at most: columns per split <= 4096
 
 // A wave owns RB blocks of 16 weight rows, a workgroup WN waves: 16 RB WN weight rows share every A chunk, and what
