@@ -334,7 +334,7 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor
 SKINNY_MAX_ROWS = 64
 SKINNY_OWN_ROWS = 16                 # without a measurement: up to here the weight-streaming kernel for every matrix,
 SKINNY_OWN_ELEMENTS = 8 << 20        # and for more rows (up to SKINNY_MAX_ROWS) while the matrix is smaller than this
-TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_products` times the two candidates
+TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_products` times the candidates
 # (rows point, matrix rows, k, gate|up) -> the quickest: LIBRARY, or this library's kernel in which every workgroup
 # owns whole rows of the result (OWN_ROWS), or the one that splits k across workgroups (OWN_KSPLIT)
 LIBRARY, OWN_ROWS, OWN_KSPLIT = 0, 1, 2
@@ -454,11 +454,19 @@ def _ksplit_scratch(device, floats: int) -> torch.Tensor:
   return t
 
 
+_SKINNY_PLANS: Dict[tuple, Tuple[int, int]] = {}
+
+
 def _skinny_plan(lib, variant: int, gate_up: bool, M: int, N: int, K: int) -> Tuple[int, int]:
   """(rows of the table of partial sums of squares, floats of scratch) of a launch of the chosen kernel."""
-  parts, floats = ctypes.c_int(0), ctypes.c_int64(0)
-  _check(lib, lib.mi_gemm_skinny_plan(variant, 1 if gate_up else 0, M, N, K, ctypes.byref(parts), ctypes.byref(floats)))
-  return parts.value, floats.value
+  key = (variant, bool(gate_up), M, N, K)
+  plan = _SKINNY_PLANS.get(key)
+  if plan is None:
+    parts, floats = ctypes.c_int(0), ctypes.c_int64(0)
+    _check(lib, lib.mi_gemm_skinny_plan(variant, 1 if gate_up else 0, M, N, K, ctypes.byref(parts),
+                                        ctypes.byref(floats)))
+    plan = _SKINNY_PLANS[key] = (parts.value, floats.value)
+  return plan
 
 
 def gemm_skinny_supported(a: torch.Tensor, w: torch.Tensor) -> bool:
