@@ -35,6 +35,9 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.f + expf(-g)); 
 // Before the second product's result is stored (`row_ss` set): row m is scaled by rsqrt(sum_p row_ss[p][m] / K +
 // eps), the norm's missing factor (K, the length of the normed rows, is this product's K).
 #define SS_ROW(rows) ((rows) <= 16 ? 16 : 64)
+#define SKINNY_CH(mb) ((mb) == 1 ? 8 : ((mb) == 2 ? 4 : 2))   // steps of K whose loads are asked for together
+// KB of LDS in which a wave stages a chunk of the left operand: 16 mb rows of 4 CH pieces of 16 bytes
+#define SKINNY_STAGE_KB(mb) ((mb) * SKINNY_CH(mb))
 struct NormHalves {
   const float* row_ss;      // [ss_parts][SS_ROW(M)]
   int ss_parts;
@@ -45,14 +48,26 @@ struct NormHalves {
   float* ss_out;            // [gridDim.x][SS_ROW(M)]
 };
 
-template <int MB, int RB, bool OUT_F32, bool GATE_UP>
+// MODE 0 takes every shape.  MODE 1 and 2 are the same product for K a multiple of 32 and operands below 4 GB, with
+// the loop's instructions cut to what the loads and products need: a decode step's matrices are a few MB, a
+// workgroup's share of one is tens of KB, and 16 waves that each spend 200 vector instructions on addresses and
+// masks before and between their loads take longer over those than over the bytes.  So: the wave's number is
+// made a scalar (its k range and every test on it then cost scalar instructions), addresses are a scalar base plus
+// one 32-bit lane offset plus a constant, and no load is masked (lanes of rows past the end read a live row again;
+// their results are dropped at the end as before).
+// MODE 2: the left operand comes through LDS.  Straight from memory, an operand load takes 16 bytes per lane from 16
+// rows of A, half a memory line from each, and every workgroup reads all of A that way.  Instead a wave asks for
+// its columns of A in runs that are contiguous in each row, has them written straight into its own piece of LDS
+// (global_load_lds: lane i's 16 bytes land at base + 16 i), and takes the operands from there.  The staging
+// pieces lie where the sums are added later.
+template <int MB, int RB, bool OUT_F32, bool GATE_UP, int MODE>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __restrict__ A, int64_t lda,
                                                            const uint16_t* __restrict__ W, int64_t ldw,
                                                            void* __restrict__ C, int64_t ldc, int M, int N, int K,
                                                            int rpg, NormHalves nh) {
   extern __shared__ float red[];   // [(waves + 1) / 2][RB * MB][256], then (norm halves) [OB * 256] squares, [waves][64] sums
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in every lane: said so
   const int nw = blockDim.x >> 6;
   // GATE_UP: RB == 2, row block 0 = gate rows n0.., row block 1 = up rows N + n0..; N counts output columns
   // rpg: rows of W per workgroup and row block: 16, or fewer so that the workgroups fill whole rounds of the
@@ -90,67 +105,173 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     arow[mb] = A + (int64_t)(mok[mb] ? m : 0) * lda;
   }
 
-  // What the norm halves read is asked for before the weights, so that the end of the kernel does not wait for
-  // memory again: the partial sums of squares of row (thread % SS), parts (thread / SS), + threads / SS, ...; and
-  // the residual and norm weight of the first two result elements this thread will finish.
+  // What the norm halves read is asked for early, so that the end of the kernel does not wait for memory again:
+  // the partial sums of squares of row (thread % SS), parts (thread / SS), + threads / SS, ... (four loads at a
+  // time, added in the order of the parts); and the residual and norm weight of the first two result elements
+  // this thread will finish.  MODE 0 asks before the weights; the other modes right after a wave's first weight
+  // loads, which are what the kernel's time hangs on.
   constexpr int OBLK = GATE_UP ? MB : RB * MB;
   constexpr int SS = SS_ROW(16 * MB);
   float my_ss = 0.f;
-  if (nh.row_ss) {
-    const int m = threadIdx.x % SS;
-    for (int p = threadIdx.x / SS; p < nh.ss_parts; p += blockDim.x / SS) my_ss += nh.row_ss[(int64_t)p * SS + m];
-  }
   float r_pre[2] = {0.f, 0.f}, w_pre[2] = {0.f, 0.f};
-  if (nh.residual) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int e = threadIdx.x + j * blockDim.x;
-      const int blk = e >> 8, ln = (e & 255) >> 2, i = e & 3;
-      const int r = 4 * (ln >> 4) + i;            // row within its block
-      const int n = n0 + rpg * (blk / MB) + r;
-      const int m = 16 * (blk % MB) + (ln & 15);
-      if (e < OBLK * 256 && r < rpg && n < n_end && m < M) {
-        r_pre[j] = nh.residual[(int64_t)m * N + n];
-        w_pre[j] = nh.norm_weight[n];
-      }
-    }
+#define SKINNY_NORM_PREFETCH()                                                                                       \
+  {                                                                                                                  \
+    int tid = threadIdx.x;                                                                                           \
+    if (MODE != 0) asm volatile("" : "+v"(tid)); /* keeps the compiler from moving the index work in front of the loop */ \
+    if (nh.row_ss) {                                                                                                 \
+      const int m = tid % SS, stride = blockDim.x / SS;                                                            \
+      for (int p = tid / SS; p < nh.ss_parts; p += 4 * stride) {                                                     \
+        float v[4];                                                                                                  \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                                \
+          v[j] = p + j * stride < nh.ss_parts ? nh.row_ss[(int64_t)(p + j * stride) * SS + m] : 0.f;                 \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) my_ss += v[j];                                                 \
+      }                                                                                                              \
+    }                                                                                                                \
+    if (nh.residual) {                                                                                               \
+      _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                                \
+        const int e = tid + j * blockDim.x;                                                                          \
+        const int blk = e >> 8, ln = (e & 255) >> 2, i = e & 3;                                                      \
+        const int r = 4 * (ln >> 4) + i; /* row within its block */                                                  \
+        const int n = n0 + rpg * (blk / MB) + r;                                                                     \
+        const int m = 16 * (blk % MB) + (ln & 15);                                                                   \
+        if (e < OBLK * 256 && r < rpg && n < n_end && m < M) {                                                       \
+          r_pre[j] = nh.residual[(int64_t)m * N + n];                                                                \
+          w_pre[j] = nh.norm_weight[n];                                                                              \
+        }                                                                                                            \
+      }                                                                                                              \
+    }                                                                                                                \
   }
+  if constexpr (MODE == 0) SKINNY_NORM_PREFETCH()
 
   // Steps are taken CH at a time: first every load of the chunk is issued (weights, and the raw left operand),
   // then the operands are converted and multiplied, so one memory round trip covers CH steps.
-  constexpr int CH = MB == 1 ? 8 : (MB == 2 ? 4 : 2);   // what fits the 128 registers of a 16-wave workgroup
-  for (int s0 = s_begin; s0 < s_end; s0 += CH) {
-    bf16x8 w[CH][RB];
-    u32x4 ar[CH][MB];
+  constexpr int CH = SKINNY_CH(MB);                     // what fits the 128 registers of a 16-wave workgroup
+  if constexpr (MODE == 0) {
+    for (int s0 = s_begin; s0 < s_end; s0 += CH) {
+      bf16x8 w[CH][RB];
+      u32x4 ar[CH][MB];
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      const int k = 32 * (s0 + c) + 8 * (lane >> 4);
-      const bool kok = (s0 + c < s_end) && k < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
-        w[c][rb] = (kok && w_live) ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const bool ok = kok && mok[mb];
-        ar[c][mb] = ok ? *reinterpret_cast<const u32x4*>(arow[mb] + k) : u32x4{0, 0, 0, 0};
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      if (s0 + c >= s_end) break;
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        union {
-          u32x4 u;
-          bf16x8 v;
-        } a;
-        a.u = ar[c][mb];
+      for (int c = 0; c < CH; ++c) {
+        const int k = 32 * (s0 + c) + 8 * (lane >> 4);
+        const bool kok = (s0 + c < s_end) && k < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
-          acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[c][rb], a.v, acc[rb][mb], 0, 0, 0);
+          w[c][rb] = (kok && w_live) ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          const bool ok = kok && mok[mb];
+          ar[c][mb] = ok ? *reinterpret_cast<const u32x4*>(arow[mb] + k) : u32x4{0, 0, 0, 0};
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (s0 + c >= s_end) break;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          union {
+            u32x4 u;
+            bf16x8 v;
+          } a;
+          a.u = ar[c][mb];
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb)
+            acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[c][rb], a.v, acc[rb][mb], 0, 0, 0);
+        }
       }
     }
+  } else {
+    const int q = lane >> 4, r = lane & 15;
+    // byte offsets of the lane's 16 bytes in step 0 of the wave's range, from W + 64 s_begin and A + 64 s_begin
+    uint32_t woff[RB], aoff[MB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      int row = n0 + (GATE_UP ? 0 : rpg * rb) + min(r, rpg - 1);
+      row = min(row, N - 1);
+      if (GATE_UP && rb == 1) row += N;
+      woff[rb] = ((uint32_t)row * (uint32_t)ldw + 8 * q) * 2;
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) aoff[mb] = ((uint32_t)min(16 * mb + r, M - 1) * (uint32_t)lda + 8 * q) * 2;
+    const char* wb = reinterpret_cast<const char*>(W) + (int64_t)s_begin * 64;
+    const char* ab = reinterpret_cast<const char*>(A) + (int64_t)s_begin * 64;
+    // MODE 2: the chunk's columns of A are rowp = 4 cs pieces of 16 bytes per row (cs: the steps of a wave's chunk
+    // at most).  Request f / 64, lane f % 64 fetches piece f % rowp of row f / rowp, which lands at stage + 16 f
+    // bytes.  (Rows padded to a stride that frees the operand reads of bank conflicts gained nothing here: these
+    // few reads wait for the loads, not for LDS.)
+    constexpr int NI = SKINNY_STAGE_KB(MB);             // requests per chunk at most
+    uint16_t* stage = reinterpret_cast<uint16_t*>(red) + (size_t)wave * (NI * 512);
+    const int rowp = 4 * min(CH, spw);
+    uint32_t s_off[MODE == 2 ? NI : 1];
+    int s_stp[MODE == 2 ? NI : 1];
+    // (worked out after the first weight loads are on their way, like the norm halves' loads: a hundred vector
+    // instructions in each of a unit's 16 waves before the first load cost the kernel 0.4 us)
+#define SKINNY_STAGE_SETUP()                                                                                         \
+  if constexpr (MODE == 2) {                                                                                         \
+    int lane_late = lane;                                                                                            \
+    asm volatile("" : "+v"(lane_late)); /* keeps the compiler from moving this in front of the loop */               \
+    const uint32_t inv = (65536u + rowp - 1) / rowp; /* f / rowp = (f inv) >> 16 for f < 1024, rowp = 4 .. 32 */      \
+    _Pragma("unroll") for (int i = 0; i < NI; ++i) {                                                                 \
+      const int f = 64 * i + lane_late;                                                                              \
+      const int row = (int)(((uint32_t)f * inv) >> 16), piece = f - row * rowp;                                      \
+      const bool live = row < M;                                                                                     \
+      s_off[i] = live ? ((uint32_t)row * (uint32_t)lda + 8 * piece) * 2 : 0;                                         \
+      s_stp[i] = live ? piece >> 2 : CH; /* the step of the chunk it belongs to; CH: never fetched */                \
+    }                                                                                                                \
   }
+    bool first = true;
+    for (int left = s_end - s_begin; left > 0; left -= CH, wb += 64 * CH, ab += 64 * CH) {
+      const int n = min(left, CH);                      // steps of this chunk: the same for the whole wave
+      bf16x8 w[CH][RB];
+      u32x4 ar[MODE == 2 ? 1 : CH][MB];
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (c < n) {
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) w[c][rb] = *reinterpret_cast<const bf16x8*>(wb + woff[rb] + 64 * c);
+          if constexpr (MODE == 1) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) ar[c][mb] = *reinterpret_cast<const u32x4*>(ab + aoff[mb] + 64 * c);
+          }
+        }
+      }
+      if (first) {
+        first = false;
+        SKINNY_NORM_PREFETCH()
+        SKINNY_STAGE_SETUP()
+      }
+      if constexpr (MODE == 2) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          if (s_stp[i] < n)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ab + s_off[i]),
+                                             (__attribute__((address_space(3))) void*)(stage + 512 * i), 16, 0, 0);
+        // The compiler does not count the requests that write LDS when it places the waits of the reads below:
+        // the wait is written out, and nothing moves across it.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        if (c < n) {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            union {
+              u32x4 u;
+              bf16x8 v;
+            } a;
+            if constexpr (MODE == 2) a.u = *reinterpret_cast<const u32x4*>(stage + 8 * ((16 * mb + r) * rowp + 4 * c + q));
+            else a.u = ar[c][mb];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+              acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[c][rb], a.v, acc[rb][mb], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (first) SKINNY_NORM_PREFETCH()                   // a wave without a step of its own
+    if constexpr (MODE == 2) __syncthreads();           // the staging pieces are given up: the sums go where they were
+  }
+#undef SKINNY_NORM_PREFETCH
+#undef SKINNY_STAGE_SETUP
 
   // lane holds C^T[n0 + 16 rb + 4 (lane / 16) + i][16 mb + lane % 16].  The waves' blocks are added through LDS in
   // two rounds, which halves the LDS they need: the upper half of the waves leaves its blocks there, the lower
@@ -384,9 +505,11 @@ MI_EXPORT int mi_norm_gemm_skinny(int gate_up, const float* R, const void* X, fl
   return 0;
 }
 
-static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up) {
+static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up, bool a_lds = false) {
   const int OB = gate_up ? MB : RB * MB;
-  return ((size_t)((waves + 1) / 2) * RB * MB * 256 + (size_t)OB * 256 + (size_t)waves * 64) * sizeof(float);
+  const size_t sums = ((size_t)((waves + 1) / 2) * RB * MB * 256 + (size_t)OB * 256 + (size_t)waves * 64) * sizeof(float);
+  const size_t stage = a_lds ? (size_t)waves * SKINNY_STAGE_KB(MB) * 1024 : 0;    // the left operand's staging pieces
+  return sums > stage ? sums : stage;
 }
 
 // Rows of W per workgroup and workgroups of the launch.  A matrix of few rows is cut finer than the 16 rows of a
@@ -446,24 +569,47 @@ static SkinnyGrid skinny_grid(bool gate_up, int N, int M) {
   return g;
 }
 
+template <int MB, int RB, bool F32, bool GU, int MODE>
+static void launch_instance(dim3 grid, dim3 block, size_t lds, hipStream_t stream, const void* A, int64_t lda,
+                            const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K, int rpg,
+                            const NormHalves& nh) {
+  auto kernel = gemm_skinny_kernel<MB, RB, F32, GU, MODE>;
+  if (MODE == 2) {     // its staging pieces may need more than the default allotment of LDS
+    static bool allowed = false;
+    if (!allowed) {
+      (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      allowed = true;
+    }
+  }
+  kernel<<<grid, block, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, ldw, C, ldc, M, N, K, rpg, nh);
+}
+
 template <int MB, int RB>
 static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                   int64_t ldc, int M, int N, int K, int waves, const SkinnyGrid& sg, const NormHalves& nh,
-                  hipStream_t stream) {
+                  bool staged, hipStream_t stream) {
   const dim3 grid(sg.groups);
   const dim3 block(64 * waves);
-  const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up);
-#define GO(F32, GU)                                                                                              \
-  gemm_skinny_kernel<MB, RB, F32, GU><<<grid, block, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, \
-                                                                    ldw, C, ldc, M, N, K, sg.rpg, nh)
+  const int64_t w_rows = gate_up ? 2 * (int64_t)N : N;
+  const bool lean = K % 32 == 0 && w_rows * ldw * 2 < ((int64_t)1 << 32) && (int64_t)M * lda * 2 < ((int64_t)1 << 32) &&
+                    (((uintptr_t)A | (uintptr_t)W) & 15) == 0;
+  // the left operand goes through LDS where the caller asks for it and the staging pieces fit
+  const int mode = !lean ? 0 : (staged && skinny_lds_bytes(waves, RB, MB, gate_up, true) <= 144 * 1024 ? 2 : 1);
+  const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up, mode == 2);
+#define GO(F32, GU)                                                                                                  \
+  {                                                                                                                  \
+    if (mode == 2) launch_instance<MB, RB, F32, GU, 2>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
+    else if (mode == 1) launch_instance<MB, RB, F32, GU, 1>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
+    else launch_instance<MB, RB, F32, GU, 0>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh);  \
+  }
   if (gate_up) {
     if constexpr (RB == 2) {
-      if (out_f32) GO(true, true);
-      else GO(false, true);
+      if (out_f32) GO(true, true)
+      else GO(false, true)
     }
   } else {
-    if (out_f32) GO(true, false);
-    else GO(false, false);
+    if (out_f32) GO(true, false)
+    else GO(false, false)
   }
 #undef GO
   return 0;
@@ -476,10 +622,10 @@ MI_EXPORT int mi_gemm_skinny_ss_row(int M) { return SS_ROW(M); }
 // A [M, K], C [M, N] bfloat16 or float32; W [N, K], or with gate_up the fused matrix [2 N, K].
 // Norm halves (see NormHalves; all optional): row_ss [ss_parts][ss_row(M)] and eps scale the rows of the result;
 // residual [M, N] float32 + norm_weight [N] + a_out [M, N] bfloat16 + ss_out [groups][ss_row(M)] replace C.
-MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw,
-                                void* C, int64_t ldc, int M, int N, int K, const float* row_ss, int ss_parts,
-                                float eps, float* residual, const float* norm_weight, void* a_out, float* ss_out,
-                                hipStream_t stream) {
+static int skinny_rows(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                       int64_t ldc, int M, int N, int K, const float* row_ss, int ss_parts, float eps,
+                       float* residual, const float* norm_weight, void* a_out, float* ss_out, bool staged,
+                       hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);
   MI_REQUIRE(lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: row strides (%lld, %lld) must be multiples of 8", (long long)lda,
@@ -506,13 +652,21 @@ MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t
   const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \
-    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, stream);          \
+    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, staged, stream);  \
     MI_CHECK_LAUNCH("gemm_skinny");                                                                           \
     return 0;                                                                                                 \
   }
   CASE(1, 1) CASE(2, 1) CASE(3, 1) CASE(4, 1) CASE(1, 2) CASE(2, 2) CASE(3, 2) CASE(4, 2)
 #undef CASE
   MI_FAIL("gemm_skinny: no instance for M=%d", M);
+}
+
+MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw,
+                                void* C, int64_t ldc, int M, int N, int K, const float* row_ss, int ss_parts,
+                                float eps, float* residual, const float* norm_weight, void* a_out, float* ss_out,
+                                hipStream_t stream) {
+  return skinny_rows(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual, norm_weight,
+                     a_out, ss_out, false, stream);
 }
 
 MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
@@ -787,11 +941,11 @@ static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
 }
 
 // What a caller needs before a call of mi_gemm_skinny_v: rows of ss_out / row_ss that this product leaves when it
-// is the first half of a norm (`ss_parts`), and the floats of scratch it needs (0 for variant 0).
+// is the first half of a norm (`ss_parts`), and the floats of scratch it needs (0 for variants 0 and 2).
 MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K, int* ss_parts, int64_t* scratch_floats) {
   MI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_plan: M=%d N=%d K=%d", M, N, K);
-  MI_REQUIRE(variant == 0 || variant == 1, "gemm_skinny_plan: variant %d", variant);
-  if (variant == 0) {
+  MI_REQUIRE(variant >= 0 && variant <= 2, "gemm_skinny_plan: variant %d", variant);
+  if (variant != 1) {
     if (ss_parts) *ss_parts = skinny_grid(gate_up != 0, N, M).groups;
     if (scratch_floats) *scratch_floats = 0;
     return 0;
@@ -804,14 +958,16 @@ MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K,
 
 // mi_gemm_skinny_ex with a choice of kernel: variant 0 = every workgroup owns whole rows of the result (above),
 // variant 1 = k split across workgroups, partial results in `scratch` (float, at least the plan's scratch_floats),
-// added in the order of the splits by a second kernel that also does the endings.
+// added in the order of the splits by a second kernel that also does the endings; variant 2 = variant 0 with the left
+// operand staged through LDS (where the shape allows it; else it is variant 0).  Variants 0 and 2 add the same
+// products in the same order: their results are equal bit for bit.
 MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void* A, int64_t lda, const void* W,
                                int64_t ldw, void* C, int64_t ldc, int M, int N, int K, const float* row_ss,
                                int ss_parts, float eps, float* residual, const float* norm_weight, void* a_out,
                                float* ss_out, float* scratch, int64_t scratch_floats, hipStream_t stream) {
-  if (variant == 0)
-    return mi_gemm_skinny_ex(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual,
-                             norm_weight, a_out, ss_out, stream);
+  if (variant == 0 || variant == 2)
+    return skinny_rows(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual, norm_weight,
+                       a_out, ss_out, variant == 2, stream);
   MI_REQUIRE(variant == 1, "gemm_skinny: variant %d", variant);
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);

@@ -336,15 +336,18 @@ SKINNY_OWN_ROWS = 16                 # without a measurement: up to here the wei
 SKINNY_OWN_ELEMENTS = 8 << 20        # and for more rows (up to SKINNY_MAX_ROWS) while the matrix is smaller than this
 TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_products` times the candidates
 # (rows point, matrix rows, k, gate|up) -> the quickest: LIBRARY, or this library's kernel in which every workgroup
-# owns whole rows of the result (OWN_ROWS), or the one that splits k across workgroups (OWN_KSPLIT)
-LIBRARY, OWN_ROWS, OWN_KSPLIT = 0, 1, 2
+# owns whole rows of the result (OWN_ROWS; OWN_ROWS_STAGED: with the left operand staged through LDS), or the one
+# that splits k across workgroups (OWN_KSPLIT)
+LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED = 0, 1, 2, 3
 _PRODUCT_CHOICE: Dict[tuple, int] = {}
 KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
 KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)
+STAGED_MIN_ROWS = 4                  # without a measurement: the left operand is staged from this many rows
+STAGED_MIN_ELEMENTS = 48 << 10       # and this many elements (8 rows of 6,144 columns, 16 of 3,072, 64 of 768)
 
 
 def set_product_choice(rows_point: int, matrix_rows: int, k: int, gate_up: bool, choice) -> None:
-  """choice: LIBRARY / OWN_ROWS / OWN_KSPLIT (False and True stand for the first two)."""
+  """choice: LIBRARY / OWN_ROWS / OWN_KSPLIT / OWN_ROWS_STAGED (False and True stand for the first two)."""
   _PRODUCT_CHOICE[(rows_point, matrix_rows, k, bool(gate_up))] = int(choice)
 
 
@@ -425,18 +428,23 @@ def _measured_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> 
 
 
 def skinny_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> int:
-  """Which of this library's two kernels runs a product that `skinny_preferred` keeps: 0 = every workgroup owns whole
-  rows of the result and reads the whole left operand (which is what its time grows with beyond 16 rows); 1 = k is
-  split across workgroups, which read a slice of the left operand each and leave 32-bit partial results that a
-  second kernel adds in a fixed order.  Measured where `tuning.tune_products` has been; else by the rule above."""
-  if gate_up and (matrix_rows // 2) % 4:
-    return 0
+  """Which of this library's kernels runs a product that `skinny_preferred` keeps: 0 = every workgroup owns whole
+  rows of the result and reads the whole left operand (which is what its time grows with beyond 16 rows); 2 = the
+  same with the left operand staged through LDS (read in whole memory lines, which costs a little when the operand
+  is small and saves much when it is not; the same sums bit for bit); 1 = k is split across workgroups, which read
+  a slice of the left operand each and leave 32-bit partial results that a second kernel adds in a fixed order.
+  Measured where `tuning.tune_products` has been; else by rule."""
   c = _measured_choice(num_rows, matrix_rows, k, gate_up)
+  can_split = not (gate_up and (matrix_rows // 2) % 4)
   if c == OWN_ROWS:
     return 0
-  if c == OWN_KSPLIT:
+  if c == OWN_ROWS_STAGED:
+    return 2
+  if c == OWN_KSPLIT and can_split:
     return 1
-  return 1 if num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K else 0
+  if can_split and num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K:
+    return 1
+  return 2 if num_rows >= STAGED_MIN_ROWS and num_rows * k >= STAGED_MIN_ELEMENTS else 0
 
 
 _KSPLIT_SCRATCH: Dict[tuple, torch.Tensor] = {}

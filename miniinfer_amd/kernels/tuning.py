@@ -1,9 +1,9 @@
 """Which kernel runs a product of few rows is measured, not guessed.
 
 For a matrix of tens of MB and a handful of rows there are three candidates: this library's weight-streaming kernel
-(`ops.gemm_skinny`, whose epilogue can take a norm's halves or the gated activation) in its two forms (every
-workgroup owns whole rows of the result, or k is split across workgroups and a second kernel adds the partial
-results), and the library product
+(`ops.gemm_skinny`, whose epilogue can take a norm's halves or the gated activation) in its forms (every
+workgroup owns whole rows of the result, with the left operand straight from memory or staged through LDS, or k is
+split across workgroups and a second kernel adds the partial results), and the library product
 (hipBLASLt through `torch.matmul`, which splits k across workgroups and so reads the left operand less often, but
 needs the norm and the activation as kernels of their own).  Which is quicker depends on the shape and the number
 of rows in ways no short rule covers, so `tune_products` times them on the model's own matrices once, when an
@@ -89,11 +89,20 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
         ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=1)
         turn[0] += 1
 
+      def own_staged():
+        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=2)
+        turn[0] += 1
+
       def library():
         torch.matmul(a, ws[turn[0] % len(ws)].t())
         turn[0] += 1
 
       t_rows = graph_time_us(own_rows, calls, flush)
+      # with its left operand staged through LDS the same kernel is a few tenths of a microsecond slower when the
+      # operand is small and up to a quarter quicker when it is not; which, depends on the shape
+      t_staged = graph_time_us(own_staged, calls, flush) if M >= ops.STAGED_MIN_ROWS and K % 32 == 0 else float("inf")
+      staged = t_staged < t_rows
+      t_rows = min(t_rows, t_staged)
       # k is split from 16 rows up only: below, the left operand is too small for its re-reads to matter, and the
       # second kernel costs more than they do (at 16 rows it wins where k is long: 68 against 76 us for [5120, 25600])
       t_split = graph_time_us(own_ksplit, calls, flush) if M >= 16 and not (gate_up and N % 4) else float("inf")
@@ -104,10 +113,11 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
       if t_split < t_rows:
         choice = ops.OWN_KSPLIT if t_split <= KSPLIT_MARGIN * t_lib else ops.LIBRARY
       else:
-        choice = ops.OWN_ROWS if t_rows <= t_lib else ops.LIBRARY
+        choice = (ops.OWN_ROWS_STAGED if staged else ops.OWN_ROWS) if t_rows <= t_lib else ops.LIBRARY
       ops.set_product_choice(M, rows_w, K, gate_up, choice)
       if log is not None:
-        log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: own {t_rows:.1f} us, "
+        log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: own {t_rows:.1f} us"
+            f"{' (operand staged)' if staged else ''}, "
             f"own with k split {t_split:.1f} us, library {t_lib:.1f} us with its extra kernels")
     timed += 1
   if timed:
