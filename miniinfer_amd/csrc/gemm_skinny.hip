@@ -77,8 +77,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   const int n0 = blockIdx.x * rpg * BLOCKS;
   const int n_end = min(N, n0 + rpg * BLOCKS);
   const bool w_live = (lane & 15) < rpg;
+  constexpr bool WL = MODE >= 3;                  // weights fetched in whole memory lines (see below)
+  constexpr bool STAGED = MODE == 2 || MODE == 4; // left operand through LDS
   const int steps = (K + 31) / 32;
-  const int spw = (steps + nw - 1) / nw;
+  // steps of K per wave; with WL a wave's range is a whole number of pairs of steps (K is a multiple of 64 then)
+  const int spw = WL ? 2 * ((steps / 2 + nw - 1) / nw) : (steps + nw - 1) / nw;
   const int s_begin = wave * spw;
   const int s_end = min(steps, s_begin + spw);
 
@@ -145,7 +148,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
 
   // Steps are taken CH at a time: first every load of the chunk is issued (weights, and the raw left operand),
   // then the operands are converted and multiplied, so one memory round trip covers CH steps.
-  constexpr int CH = SKINNY_CH(MB);                     // what fits the 128 registers of a 16-wave workgroup
+  // what fits the 128 registers of a 16-wave workgroup (the exchange between lanes of the whole-line loads needs a
+  // few registers more: two row blocks then take 4 steps at a time)
+  constexpr int CH = (MODE >= 3 && RB == 2 && MB == 1) ? 4 : SKINNY_CH(MB);
   if constexpr (MODE == 0) {
     for (int s0 = s_begin; s0 < s_end; s0 += CH) {
       bf16x8 w[CH][RB];
@@ -182,16 +187,27 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   } else {
     const int q = lane >> 4, r = lane & 15;
     // byte offsets of the lane's 16 bytes in step 0 of the wave's range, from W + 64 s_begin and A + 64 s_begin
-    uint32_t woff[RB], aoff[MB];
+    // WL: an operand load as above takes 64 bytes from each of 16 rows, half a memory line; large matrices stream
+    // a tenth to a sixth faster when every request is for whole lines.  So two steps are fetched together, by two
+    // loads of 8 rows x 128 bytes: load i, lane (r, q) takes piece 2 q + r / 8 of row 8 i + r % 8.  Lanes r and
+    // r + 8 then hold each other's data: the lower one its own row's even piece (load 0) and the other's (load 1),
+    // the upper one the lower's odd piece and its own.  One rotation by 8 within the rows of 16 lanes
+    // (update_dpp) puts both pieces of a row into its lane: piece 2 q serves the first step of the pair, 2 q + 1
+    // the second; the left operand follows the same order of k.
+    const int h = r >> 3, r8 = r & 7;
+    uint32_t woff[RB][WL ? 2 : 1], aoff[MB];
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      int row = n0 + (GATE_UP ? 0 : rpg * rb) + min(r, rpg - 1);
-      row = min(row, N - 1);
-      if (GATE_UP && rb == 1) row += N;
-      woff[rb] = ((uint32_t)row * (uint32_t)ldw + 8 * q) * 2;
-    }
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) aoff[mb] = ((uint32_t)min(16 * mb + r, M - 1) * (uint32_t)lda + 8 * q) * 2;
+      for (int i = 0; i < (WL ? 2 : 1); ++i) {
+        int row = n0 + (GATE_UP ? 0 : rpg * rb) + min(WL ? 8 * i + r8 : r, rpg - 1);
+        row = min(row, N - 1);
+        if (GATE_UP && rb == 1) row += N;
+        woff[rb][i] = ((uint32_t)row * (uint32_t)ldw + 8 * (WL ? 2 * q + h : q)) * 2;
+      }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      aoff[mb] = ((uint32_t)min(16 * mb + r, M - 1) * (uint32_t)lda + (WL ? 16 : 8) * q) * 2;
     const char* wb = reinterpret_cast<const char*>(W) + (int64_t)s_begin * 64;
     const char* ab = reinterpret_cast<const char*>(A) + (int64_t)s_begin * 64;
     // MODE 2: the chunk's columns of A are rowp = 4 cs pieces of 16 bytes per row (cs: the steps of a wave's chunk
@@ -201,12 +217,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     constexpr int NI = SKINNY_STAGE_KB(MB);             // requests per chunk at most
     uint16_t* stage = reinterpret_cast<uint16_t*>(red) + (size_t)wave * (NI * 512);
     const int rowp = 4 * min(CH, spw);
-    uint32_t s_off[MODE == 2 ? NI : 1];
-    int s_stp[MODE == 2 ? NI : 1];
+    uint32_t s_off[STAGED ? NI : 1];
+    int s_stp[STAGED ? NI : 1];
     // (worked out after the first weight loads are on their way, like the norm halves' loads: a hundred vector
     // instructions in each of a unit's 16 waves before the first load cost the kernel 0.4 us)
 #define SKINNY_STAGE_SETUP()                                                                                         \
-  if constexpr (MODE == 2) {                                                                                         \
+  if constexpr (STAGED) {                                                                                            \
     int lane_late = lane;                                                                                            \
     asm volatile("" : "+v"(lane_late)); /* keeps the compiler from moving this in front of the loop */               \
     const uint32_t inv = (65536u + rowp - 1) / rowp; /* f / rowp = (f inv) >> 16 for f < 1024, rowp = 4 .. 32 */      \
@@ -221,16 +237,18 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     bool first = true;
     for (int left = s_end - s_begin; left > 0; left -= CH, wb += 64 * CH, ab += 64 * CH) {
       const int n = min(left, CH);                      // steps of this chunk: the same for the whole wave
-      bf16x8 w[CH][RB];
-      u32x4 ar[MODE == 2 ? 1 : CH][MB];
+      u32x4 w[CH][RB];
+      u32x4 ar[STAGED ? 1 : CH][MB];
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         if (c < n) {
 #pragma unroll
-          for (int rb = 0; rb < RB; ++rb) w[c][rb] = *reinterpret_cast<const bf16x8*>(wb + woff[rb] + 64 * c);
-          if constexpr (MODE == 1) {
+          for (int rb = 0; rb < RB; ++rb)
+            w[c][rb] = *reinterpret_cast<const u32x4*>(wb + woff[rb][WL ? c & 1 : 0] + (WL ? 128 * (c >> 1) : 64 * c));
+          if constexpr (!STAGED) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) ar[c][mb] = *reinterpret_cast<const u32x4*>(ab + aoff[mb] + 64 * c);
+            for (int mb = 0; mb < MB; ++mb)
+              ar[c][mb] = *reinterpret_cast<const u32x4*>(ab + aoff[mb] + (WL ? 128 * (c >> 1) + 16 * (c & 1) : 64 * c));
           }
         }
       }
@@ -239,7 +257,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         SKINNY_NORM_PREFETCH()
         SKINNY_STAGE_SETUP()
       }
-      if constexpr (MODE == 2) {
+      if constexpr (STAGED) {
 #pragma unroll
         for (int i = 0; i < NI; ++i)
           if (s_stp[i] < n)
@@ -249,6 +267,24 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         // the wait is written out, and nothing moves across it.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
+      if constexpr (WL) {
+        constexpr int ROR8 = 0x128;                     // row_ror:8
+#pragma unroll
+        for (int c = 0; c < CH; c += 2) {
+          if (c < n) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+              const u32x4 l0 = w[c][rb], l1 = w[c + 1][rb];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                // lanes 8 .. 15 of a row take the lower lanes' load 1, lanes 0 .. 7 the upper lanes' load 0
+                w[c][rb][e] = __builtin_amdgcn_update_dpp((int)l0[e], (int)l1[e], ROR8, 0xF, 0xC, false);
+                w[c + 1][rb][e] = __builtin_amdgcn_update_dpp((int)l1[e], (int)l0[e], ROR8, 0xF, 0x3, false);
+              }
+            }
+          }
+        }
+      }
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
         if (c < n) {
@@ -257,18 +293,22 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
             union {
               u32x4 u;
               bf16x8 v;
-            } a;
-            if constexpr (MODE == 2) a.u = *reinterpret_cast<const u32x4*>(stage + 8 * ((16 * mb + r) * rowp + 4 * c + q));
+            } a, b;
+            if constexpr (STAGED)
+              a.u = *reinterpret_cast<const u32x4*>(
+                  stage + 8 * ((16 * mb + r) * rowp + (WL ? 8 * (c >> 1) + 2 * q + (c & 1) : 4 * c + q)));
             else a.u = ar[c][mb];
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb)
-              acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[c][rb], a.v, acc[rb][mb], 0, 0, 0);
+            for (int rb = 0; rb < RB; ++rb) {
+              b.u = w[c][rb];
+              acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, a.v, acc[rb][mb], 0, 0, 0);
+            }
           }
         }
       }
     }
     if (first) SKINNY_NORM_PREFETCH()                   // a wave without a step of its own
-    if constexpr (MODE == 2) __syncthreads();           // the staging pieces are given up: the sums go where they were
+    if constexpr (STAGED) __syncthreads();              // the staging pieces are given up: the sums go where they were
   }
 #undef SKINNY_NORM_PREFETCH
 #undef SKINNY_STAGE_SETUP
@@ -574,7 +614,7 @@ static void launch_instance(dim3 grid, dim3 block, size_t lds, hipStream_t strea
                             const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K, int rpg,
                             const NormHalves& nh) {
   auto kernel = gemm_skinny_kernel<MB, RB, F32, GU, MODE>;
-  if (MODE == 2) {     // its staging pieces may need more than the default allotment of LDS
+  if (MODE == 2 || MODE == 4) {     // its staging pieces may need more than the default allotment of LDS
     static bool allowed = false;
     if (!allowed) {
       (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -587,18 +627,25 @@ static void launch_instance(dim3 grid, dim3 block, size_t lds, hipStream_t strea
 template <int MB, int RB>
 static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                   int64_t ldc, int M, int N, int K, int waves, const SkinnyGrid& sg, const NormHalves& nh,
-                  bool staged, hipStream_t stream) {
+                  bool staged, bool lines, hipStream_t stream) {
   const dim3 grid(sg.groups);
   const dim3 block(64 * waves);
   const int64_t w_rows = gate_up ? 2 * (int64_t)N : N;
   const bool lean = K % 32 == 0 && w_rows * ldw * 2 < ((int64_t)1 << 32) && (int64_t)M * lda * 2 < ((int64_t)1 << 32) &&
                     (((uintptr_t)A | (uintptr_t)W) & 15) == 0;
-  // the left operand goes through LDS where the caller asks for it and the staging pieces fit
-  const int mode = !lean ? 0 : (staged && skinny_lds_bytes(waves, RB, MB, gate_up, true) <= 144 * 1024 ? 2 : 1);
-  const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up, mode == 2);
+  // the left operand goes through LDS where the caller asks for it and the staging pieces fit; the weights come in
+  // whole memory lines where the caller asks for that and K is a multiple of 64
+  int mode = 0;
+  if (lean) {
+    mode = staged && skinny_lds_bytes(waves, RB, MB, gate_up, true) <= 144 * 1024 ? 2 : 1;
+    if (lines && K % 64 == 0) mode += 2;
+  }
+  const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up, mode == 2 || mode == 4);
 #define GO(F32, GU)                                                                                                  \
   {                                                                                                                  \
-    if (mode == 2) launch_instance<MB, RB, F32, GU, 2>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
+    if (mode == 4) launch_instance<MB, RB, F32, GU, 4>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
+    else if (mode == 3) launch_instance<MB, RB, F32, GU, 3>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
+    else if (mode == 2) launch_instance<MB, RB, F32, GU, 2>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
     else if (mode == 1) launch_instance<MB, RB, F32, GU, 1>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
     else launch_instance<MB, RB, F32, GU, 0>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh);  \
   }
@@ -625,7 +672,7 @@ MI_EXPORT int mi_gemm_skinny_ss_row(int M) { return SS_ROW(M); }
 static int skinny_rows(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                        int64_t ldc, int M, int N, int K, const float* row_ss, int ss_parts, float eps,
                        float* residual, const float* norm_weight, void* a_out, float* ss_out, bool staged,
-                       hipStream_t stream) {
+                       bool lines, hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);
   MI_REQUIRE(lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: row strides (%lld, %lld) must be multiples of 8", (long long)lda,
@@ -652,7 +699,8 @@ static int skinny_rows(int out_f32, int gate_up, const void* A, int64_t lda, con
   const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \
-    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, staged, stream);  \
+    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, staged, lines,    \
+                   stream);                                                                                 \
     MI_CHECK_LAUNCH("gemm_skinny");                                                                           \
     return 0;                                                                                                 \
   }
@@ -666,7 +714,7 @@ MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t
                                 float eps, float* residual, const float* norm_weight, void* a_out, float* ss_out,
                                 hipStream_t stream) {
   return skinny_rows(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual, norm_weight,
-                     a_out, ss_out, false, stream);
+                     a_out, ss_out, false, false, stream);
 }
 
 MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
@@ -941,10 +989,10 @@ static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
 }
 
 // What a caller needs before a call of mi_gemm_skinny_v: rows of ss_out / row_ss that this product leaves when it
-// is the first half of a norm (`ss_parts`), and the floats of scratch it needs (0 for variants 0 and 2).
+// is the first half of a norm (`ss_parts`), and the floats of scratch it needs (0 for every variant but 1).
 MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K, int* ss_parts, int64_t* scratch_floats) {
   MI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_plan: M=%d N=%d K=%d", M, N, K);
-  MI_REQUIRE(variant >= 0 && variant <= 2, "gemm_skinny_plan: variant %d", variant);
+  MI_REQUIRE(variant >= 0 && variant <= 4, "gemm_skinny_plan: variant %d", variant);
   if (variant != 1) {
     if (ss_parts) *ss_parts = skinny_grid(gate_up != 0, N, M).groups;
     if (scratch_floats) *scratch_floats = 0;
@@ -959,15 +1007,16 @@ MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K,
 // mi_gemm_skinny_ex with a choice of kernel: variant 0 = every workgroup owns whole rows of the result (above),
 // variant 1 = k split across workgroups, partial results in `scratch` (float, at least the plan's scratch_floats),
 // added in the order of the splits by a second kernel that also does the endings; variant 2 = variant 0 with the left
-// operand staged through LDS (where the shape allows it; else it is variant 0).  Variants 0 and 2 add the same
-// products in the same order: their results are equal bit for bit.
+// operand staged through LDS; variants 3 and 4 = variants 0 and 2 with the weights fetched in whole memory lines
+// (each where the shape allows it; else without).  Variants 0 and 2 add the same products in the same order: their
+// results are equal bit for bit, and so are those of 3 and 4.
 MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void* A, int64_t lda, const void* W,
                                int64_t ldw, void* C, int64_t ldc, int M, int N, int K, const float* row_ss,
                                int ss_parts, float eps, float* residual, const float* norm_weight, void* a_out,
                                float* ss_out, float* scratch, int64_t scratch_floats, hipStream_t stream) {
-  if (variant == 0 || variant == 2)
+  if (variant != 1 && variant >= 0 && variant <= 4)
     return skinny_rows(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual, norm_weight,
-                       a_out, ss_out, variant == 2, stream);
+                       a_out, ss_out, variant == 2 || variant == 4, variant >= 3, stream);
   MI_REQUIRE(variant == 1, "gemm_skinny: variant %d", variant);
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);

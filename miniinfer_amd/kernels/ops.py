@@ -336,18 +336,21 @@ SKINNY_OWN_ROWS = 16                 # without a measurement: up to here the wei
 SKINNY_OWN_ELEMENTS = 8 << 20        # and for more rows (up to SKINNY_MAX_ROWS) while the matrix is smaller than this
 TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_products` times the candidates
 # (rows point, matrix rows, k, gate|up) -> the quickest: LIBRARY, or this library's kernel in which every workgroup
-# owns whole rows of the result (OWN_ROWS; OWN_ROWS_STAGED: with the left operand staged through LDS), or the one
-# that splits k across workgroups (OWN_KSPLIT)
-LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED = 0, 1, 2, 3
+# owns whole rows of the result (OWN_ROWS; OWN_ROWS_STAGED: with the left operand staged through LDS; OWN_ROWS_LINES,
+# OWN_ROWS_STAGED_LINES: the same two with the weights fetched in whole memory lines), or the one that splits k
+# across workgroups (OWN_KSPLIT).  An own kernel's choice is its variant number + 1.
+LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES = 0, 1, 2, 3, 4, 5
 _PRODUCT_CHOICE: Dict[tuple, int] = {}
 KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
 KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)
 STAGED_MIN_ROWS = 4                  # without a measurement: the left operand is staged from this many rows
-STAGED_MIN_ELEMENTS = 48 << 10       # and this many elements (8 rows of 6,144 columns, 16 of 3,072, 64 of 768)
+STAGED_MIN_ELEMENTS = 12 << 10       # and this many elements (4 rows of 3,072 columns, 8 of 1,536)
+LINES_MIN_ELEMENTS = 40 << 20        # without a measurement: the weights come in whole lines for matrices of this size
+LINES_MIN_K = 5120                   # with rows of at least this many columns (a multiple of 64)
 
 
 def set_product_choice(rows_point: int, matrix_rows: int, k: int, gate_up: bool, choice) -> None:
-  """choice: LIBRARY / OWN_ROWS / OWN_KSPLIT / OWN_ROWS_STAGED (False and True stand for the first two)."""
+  """choice: LIBRARY or one of the OWN_... constants (False and True stand for LIBRARY and OWN_ROWS)."""
   _PRODUCT_CHOICE[(rows_point, matrix_rows, k, bool(gate_up))] = int(choice)
 
 
@@ -416,7 +419,7 @@ def skinny_preferred(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fa
   c = _measured_choice(num_rows, matrix_rows, k, gate_up)
   if c is not None:
     return c != LIBRARY
-  return num_rows <= SKINNY_OWN_ROWS or matrix_rows * k < SKINNY_OWN_ELEMENTS
+  return rule_choice(num_rows, matrix_rows, k, gate_up) != LIBRARY
 
 
 def _measured_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> Optional[int]:
@@ -431,20 +434,32 @@ def skinny_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fals
   """Which of this library's kernels runs a product that `skinny_preferred` keeps: 0 = every workgroup owns whole
   rows of the result and reads the whole left operand (which is what its time grows with beyond 16 rows); 2 = the
   same with the left operand staged through LDS (read in whole memory lines, which costs a little when the operand
-  is small and saves much when it is not; the same sums bit for bit); 1 = k is split across workgroups, which read
-  a slice of the left operand each and leave 32-bit partial results that a second kernel adds in a fixed order.
+  is small and saves much when it is not; the same sums bit for bit); 3, 4 = 0 and 2 with the weights fetched in
+  whole memory lines too (two steps of k at a time, put in place by an exchange between lanes: large matrices
+  stream faster that way); 1 = k is split across workgroups, which read a slice of the left operand each and
+  leave 32-bit partial results that a second kernel adds in a fixed order.
   Measured where `tuning.tune_products` has been; else by rule."""
   c = _measured_choice(num_rows, matrix_rows, k, gate_up)
   can_split = not (gate_up and (matrix_rows // 2) % 4)
-  if c == OWN_ROWS:
-    return 0
-  if c == OWN_ROWS_STAGED:
-    return 2
-  if c == OWN_KSPLIT and can_split:
-    return 1
+  if c is not None and c != LIBRARY and (c != OWN_KSPLIT or can_split):
+    return c - 1
+  return _rule_variant(num_rows, matrix_rows, k, gate_up)
+
+
+def _rule_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> int:
+  can_split = not (gate_up and (matrix_rows // 2) % 4)
   if can_split and num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K:
     return 1
-  return 2 if num_rows >= STAGED_MIN_ROWS and num_rows * k >= STAGED_MIN_ELEMENTS else 0
+  if num_rows >= STAGED_MIN_ROWS and num_rows * k >= STAGED_MIN_ELEMENTS:
+    return 4 if matrix_rows * k >= LINES_MIN_ELEMENTS and k >= LINES_MIN_K and k % 64 == 0 else 2
+  return 0
+
+
+def rule_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> int:
+  """What runs a product of up to SKINNY_MAX_ROWS rows when nothing has been measured: LIBRARY, or an OWN_... kernel."""
+  if num_rows <= SKINNY_OWN_ROWS or matrix_rows * k < SKINNY_OWN_ELEMENTS:
+    return _rule_variant(num_rows, matrix_rows, k, gate_up) + 1
+  return LIBRARY
 
 
 _KSPLIT_SCRATCH: Dict[tuple, torch.Tensor] = {}

@@ -20,8 +20,11 @@ import torch
 from . import ops
 
 MIN_ELEMENTS = 2 << 20
-UNFUSED_US = 3.0          # what a norm or activation kernel of its own costs inside a decode step
+UNFUSED_US = 4.5          # what a norm or activation kernel of its own costs inside a decode step (2.7 us + the gap before it)
+LINES_MIN_ELEMENTS = 16 << 20   # matrices from this size up are also timed with their weights fetched in whole lines
 KSPLIT_MARGIN = 0.9       # the k-split kernel replaces the library's product only if it takes at most this much of its time
+LIBRARY_MARGIN = 0.92     # and the library's replaces a one-kernel product of this library only at this much of its time
+RULE_MARGIN = 1.05        # what the rule would run stays unless the quickest candidate beats it by this factor
 
 
 def graph_time_us(fn: Callable[[], None], calls: int, flush: Optional[torch.Tensor] = None) -> float:
@@ -81,44 +84,58 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
       out = torch.empty(M, N, dtype=torch.bfloat16, device=a.device)
       turn = [0]
 
-      def own_rows():
-        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=0)
-        turn[0] += 1
-
-      def own_ksplit():
-        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=1)
-        turn[0] += 1
-
-      def own_staged():
-        ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=2)
-        turn[0] += 1
+      def own(variant):
+        def run():
+          ops.gemm_skinny(a, ws[turn[0] % len(ws)], out, gate_up=gate_up, variant=variant)
+          turn[0] += 1
+        return run
 
       def library():
         torch.matmul(a, ws[turn[0] % len(ws)].t())
         turn[0] += 1
 
-      t_rows = graph_time_us(own_rows, calls, flush)
-      # with its left operand staged through LDS the same kernel is a few tenths of a microsecond slower when the
-      # operand is small and up to a quarter quicker when it is not; which, depends on the shape
-      t_staged = graph_time_us(own_staged, calls, flush) if M >= ops.STAGED_MIN_ROWS and K % 32 == 0 else float("inf")
-      staged = t_staged < t_rows
-      t_rows = min(t_rows, t_staged)
+      # The kernel in which a workgroup owns whole rows of the result, in its forms: with the left operand staged
+      # through LDS it is a few tenths of a microsecond slower when the operand is small and up to a quarter quicker
+      # when it is not; with the weights fetched in whole memory lines large matrices stream up to a tenth faster
+      # and small ones slower.  Which, depends on the shape.
+      forms = {ops.OWN_ROWS: graph_time_us(own(0), calls, flush)}
+      stage = M >= ops.STAGED_MIN_ROWS and K % 32 == 0
+      if stage:
+        forms[ops.OWN_ROWS_STAGED] = graph_time_us(own(2), calls, flush)
+      if K % 64 == 0 and rows_w * K >= LINES_MIN_ELEMENTS:
+        c = ops.OWN_ROWS_STAGED_LINES if stage else ops.OWN_ROWS_LINES
+        forms[c] = graph_time_us(own(c - 1), calls, flush)
+      rows_choice = min(forms, key=forms.get)
+      t_rows = forms[rows_choice]
       # k is split from 16 rows up only: below, the left operand is too small for its re-reads to matter, and the
       # second kernel costs more than they do (at 16 rows it wins where k is long: 68 against 76 us for [5120, 25600])
-      t_split = graph_time_us(own_ksplit, calls, flush) if M >= 16 and not (gate_up and N % 4) else float("inf")
+      t_split = graph_time_us(own(1), calls, flush) if M >= 16 and not (gate_up and N % 4) else float("inf")
       t_lib = graph_time_us(library, calls, flush) + (2 if gate_up else 1) * UNFUSED_US
-      # The two own kernels end alike, so they are compared as timed.  Against the library the k-split kernel must
+      # The own kernels end alike, so they are compared as timed.  Against the library the k-split kernel must
       # win by a tenth: inside a step of the 8B shape at 64 rows it lost 4 us a layer to the library's product for
-      # the down projection although it had won this timing by 3 us (its partial results are 17 MB there).
+      # the down projection although it had won this timing by 3 us (its partial results are 17 MB there).  And
+      # the library must beat a one-kernel product by a twelfth: the 32B shape's gate|up product at 8 rows, 103 us
+      # in the library against 121 here when timed alone, made the whole step 3% slower than this library's
+      # kernel with the norm and the activation in it.
       if t_split < t_rows:
         choice = ops.OWN_KSPLIT if t_split <= KSPLIT_MARGIN * t_lib else ops.LIBRARY
       else:
-        choice = (ops.OWN_ROWS_STAGED if staged else ops.OWN_ROWS) if t_rows <= t_lib else ops.LIBRARY
+        choice = rows_choice if LIBRARY_MARGIN * t_rows <= t_lib else ops.LIBRARY
+      # Timings of candidates that lie close together change places from run to run, and with them the step's time
+      # by a few percent: the rule's candidate is kept unless the winner is clearly quicker.
+      timed_us = dict(forms)
+      timed_us[ops.OWN_KSPLIT], timed_us[ops.LIBRARY] = t_split, t_lib
+      rule = ops.rule_choice(M, rows_w, K, gate_up)
+      if rule in timed_us and timed_us[rule] <= RULE_MARGIN * timed_us[choice]:
+        choice = rule
       ops.set_product_choice(M, rows_w, K, gate_up, choice)
       if log is not None:
-        log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: own {t_rows:.1f} us"
-            f"{' (operand staged)' if staged else ''}, "
-            f"own with k split {t_split:.1f} us, library {t_lib:.1f} us with its extra kernels")
+        names = {ops.LIBRARY: "library", ops.OWN_ROWS: "own", ops.OWN_KSPLIT: "own with k split",
+                 ops.OWN_ROWS_STAGED: "own, left operand staged", ops.OWN_ROWS_LINES: "own, weights in whole lines",
+                 ops.OWN_ROWS_STAGED_LINES: "own, left operand staged, weights in whole lines"}
+        log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: "
+            + ", ".join(f"{names[c]} {t:.1f} us" for c, t in forms.items())
+            + f", own with k split {t_split:.1f} us, library {t_lib:.1f} us with its extra kernels -> {names[choice]}")
     timed += 1
   if timed:
     # give the timing's buffers back to the driver: what is allocated next (the cache pools) then lies as it would

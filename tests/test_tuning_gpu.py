@@ -35,8 +35,9 @@ def test_products_are_timed_once_per_shape_and_small_ones_are_left_alone(clean_c
   assert not ops.skinny_preferred(65, 2048, 1024)
 
 
-# the library / whole rows per workgroup / k split across workgroups / whole rows with the left operand staged
-@pytest.mark.parametrize("choice", [0, 1, 2, 3])
+# the library / whole rows per workgroup / k split across workgroups / whole rows with the left operand staged /
+# whole rows with the weights in whole lines / both
+@pytest.mark.parametrize("choice", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("M", [3, 16, 40])
 def test_either_choice_gives_the_product(clean_choices, choice, M):
   ops = clean_choices
@@ -51,7 +52,7 @@ def test_either_choice_gives_the_product(clean_choices, choice, M):
     ops.set_product_choice(p, N, K, False, choice)
     ops.set_product_choice(p, 2 * inter, K, True, choice)
   assert ops.skinny_preferred(M, N, K) == own and ops.skinny_preferred(M, 2 * inter, K, True) == own
-  assert ops.skinny_variant(M, N, K) == {ops.OWN_KSPLIT: 1, ops.OWN_ROWS_STAGED: 2}.get(choice, 0)
+  assert ops.skinny_variant(M, N, K) == (choice - 1 if own else 0)
   y = linear(x.to(DEV), w.to(DEV))
   torch.testing.assert_close(y.double().cpu(), x.double() @ w.double().T, rtol=2e-2, atol=2e-2)
   a = gate_up_activation(x.to(DEV), wgu.to(DEV))
