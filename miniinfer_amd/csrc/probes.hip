@@ -7,23 +7,26 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// Every thread walks the buffer in strides of the whole grid, 16 bytes at a time, UNROLL loads in flight, and
-// xors what it read into one word, which is stored only if it has a value that random data practically never
-// gives (the compiler must keep the loads, memory sees no write traffic).
+// Every workgroup reads a contiguous slice of the buffer, 16 bytes a lane and UNROLL loads in flight, and xors what
+// it read into one word, which is stored only if it has a value that random data practically never gives (the
+// compiler must keep the loads, memory sees no write traffic).  (Slices per workgroup stream faster than one
+// stride of the whole grid: 6.2 against 5.8 TB/s.)
 template <int UNROLL>
 __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* __restrict__ src, int64_t n16,
                                                           uint32_t* __restrict__ sink) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t per_block = (n16 + gridDim.x - 1) / gridDim.x;
+  const int64_t begin = (int64_t)blockIdx.x * per_block;
+  const int64_t end = begin + per_block < n16 ? begin + per_block : n16;
+  int64_t i = begin + threadIdx.x;
   u32x4 acc = {0, 0, 0, 0};
-  for (; i + (UNROLL - 1) * stride < n16; i += UNROLL * stride) {
+  for (; i + (UNROLL - 1) * 256 < end; i += UNROLL * 256) {
     u32x4 v[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+    for (int u = 0; u < UNROLL; ++u) v[u] = src[i + u * 256];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) acc ^= v[u];
   }
-  for (; i < n16; i += stride) acc ^= src[i];
+  for (; i < end; i += 256) acc ^= src[i];
   const uint32_t x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
   if (x == 0x9e3779b9u) sink[0] = x;
 }
@@ -35,7 +38,7 @@ MI_EXPORT int mi_probe_stream_read(const void* src, int64_t bytes, void* sink, h
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
     cus = 256;
-  stream_read_kernel<8><<<cus * 8, 256, 0, stream>>>((const u32x4*)src, bytes / 16, (uint32_t*)sink);
+  stream_read_kernel<16><<<cus * 8, 256, 0, stream>>>((const u32x4*)src, bytes / 16, (uint32_t*)sink);
   MI_CHECK_LAUNCH("probe_stream_read");
   return 0;
 }
