@@ -48,18 +48,19 @@ struct NormHalves {
   float* ss_out;            // [gridDim.x][SS_ROW(M)]
 };
 
-// MODE 0 takes every shape.  MODE 1 and 2 are the same product for K a multiple of 32 and operands below 4 GB, with
-// the loop's instructions cut to what the loads and products need: a decode step's matrices are a few MB, a
-// workgroup's share of one is tens of KB, and 16 waves that each spend 200 vector instructions on addresses and
-// masks before and between their loads take longer over those than over the bytes.  So: the wave's number is
-// made a scalar (its k range and every test on it then cost scalar instructions), addresses are a scalar base plus
-// one 32-bit lane offset plus a constant, and no load is masked (lanes of rows past the end read a live row again;
-// their results are dropped at the end as before).
-// MODE 2: the left operand comes through LDS.  Straight from memory, an operand load takes 16 bytes per lane from 16
-// rows of A, half a memory line from each, and every workgroup reads all of A that way.  Instead a wave asks for
-// its columns of A in runs that are contiguous in each row, has them written straight into its own piece of LDS
-// (global_load_lds: lane i's 16 bytes land at base + 16 i), and takes the operands from there.  The staging
+// MODE 0 takes every shape.  MODES 1 to 4 are the same product for K a multiple of 32 and operands below 4 GB: the
+// wave's number is made a scalar (its k range and every test on it then cost scalar instructions), addresses are a
+// scalar base plus one 32-bit lane offset plus a constant, no load is masked (lanes of rows past the end read a live
+// row again; their results are dropped at the end as before), and a wave's first weight loads go out before the
+// index work of the norm halves' loads and of the staging below: what a unit's 16 waves do before their first
+// loads is time added to the kernel (a hundred vector instructions each: 0.4 us), what they do after them is not.
+// MODES 2 and 4: the left operand comes through LDS.  Straight from memory, an operand load takes 16 bytes per lane
+// from 16 rows of A, half a memory line from each, and every workgroup reads all of A that way.  Instead a wave asks
+// for its columns of A in runs that are contiguous in each row, has them written straight into its own piece of
+// LDS (global_load_lds: lane i's 16 bytes land at base + 16 i), and takes the operands from there.  The staging
 // pieces lie where the sums are added later.
+// MODES 3 and 4 (K a multiple of 64): the weights come in whole memory lines too, two steps of k per pair of loads
+// (see the loop).  Modes 1 and 2 add the same products in the same order, and so do 3 and 4.
 template <int MB, int RB, bool OUT_F32, bool GATE_UP, int MODE>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __restrict__ A, int64_t lda,
                                                            const uint16_t* __restrict__ W, int64_t ldw,
