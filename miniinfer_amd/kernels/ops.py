@@ -450,7 +450,8 @@ def _rule_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> int
   can_split = not (gate_up and (matrix_rows // 2) % 4)
   if can_split and num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K:
     return 1
-  if num_rows >= STAGED_MIN_ROWS and num_rows * k >= STAGED_MIN_ELEMENTS:
+  # (a matrix of very many rows, the output head, has as many workgroups re-reading the left operand: staged too)
+  if num_rows >= STAGED_MIN_ROWS and (num_rows * k >= STAGED_MIN_ELEMENTS or matrix_rows * k >= LINES_MIN_ELEMENTS):
     return 4 if matrix_rows * k >= LINES_MIN_ELEMENTS and k >= LINES_MIN_K and k % 64 == 0 else 2
   return 0
 

@@ -39,7 +39,7 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     assert ops.skinny_variant(4, 1024, 2048) == 0 and ops.skinny_variant(8, 4096, 1024) == 0
     assert ops.skinny_variant(4, 1024, 3072) == 2 and ops.skinny_variant(8, 4096, 4096) == 2
     assert ops.skinny_variant(8, 4096, 12288) == 4 and ops.skinny_variant(3, 4096, 25600) == 0
-    assert ops.skinny_variant(16, 6144, 4096) == 2
+    assert ops.skinny_variant(16, 6144, 4096) == 2 and ops.skinny_variant(8, 151936, 1024) == 2
     assert ops.skinny_variant(8, 51200, 5120, True) == 4 and ops.skinny_variant(8, 5120, 25632) == 2
     assert ops.skinny_variant(64, 2 * 1026, 4096, True) == 2 and ops.skinny_variant(64, 2 * 1028, 4096, True) == 1
     for p in ops.TUNE_ROWS:
