@@ -38,6 +38,9 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.f + expf(-g)); 
 #define SKINNY_CH(mb) ((mb) == 1 ? 8 : ((mb) == 2 ? 4 : 2))   // steps of K whose loads are asked for together
 // KB of LDS in which a wave stages a chunk of the left operand: 16 mb rows of 4 CH pieces of 16 bytes
 #define SKINNY_STAGE_KB(mb) ((mb) * SKINNY_CH(mb))
+// The mode that stages both operands: steps per chunk, and KB for 16 blocks rows of 4 steps + 2 pieces each
+#define SKINNY_STAGE5_STEPS 4
+#define SKINNY_STAGE5_KB(blocks) ((16 * (blocks) * (4 * SKINNY_STAGE5_STEPS + 2) + 63) / 64)
 struct NormHalves {
   const float* row_ss;      // [ss_parts][SS_ROW(M)]
   int ss_parts;
@@ -78,7 +81,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   const int n0 = blockIdx.x * rpg * BLOCKS;
   const int n_end = min(N, n0 + rpg * BLOCKS);
   const bool w_live = (lane & 15) < rpg;
-  constexpr bool WL = MODE >= 3;                  // weights fetched in whole memory lines (see below)
+  constexpr bool WL = MODE == 3 || MODE == 4;     // weights fetched in whole memory lines (see below)
   constexpr bool STAGED = MODE == 2 || MODE == 4; // left operand through LDS
   const int steps = (K + 31) / 32;
   // steps of K per wave; with WL a wave's range is a whole number of pairs of steps (K is a multiple of 64 then)
@@ -151,7 +154,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
   // then the operands are converted and multiplied, so one memory round trip covers CH steps.
   // what fits the 128 registers of a 16-wave workgroup (the exchange between lanes of the whole-line loads needs a
   // few registers more: two row blocks then take 4 steps at a time)
-  constexpr int CH = (MODE >= 3 && RB == 2 && MB == 1) ? 4 : SKINNY_CH(MB);
+  constexpr int CH = (WL && RB == 2 && MB == 1) ? 4 : SKINNY_CH(MB);
   if constexpr (MODE == 0) {
     for (int s0 = s_begin; s0 < s_end; s0 += CH) {
       bf16x8 w[CH][RB];
@@ -185,6 +188,87 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         }
       }
     }
+  } else if constexpr (MODE == 5) {
+    // Both operands through LDS (at most 16 rows of A).  Every request reads runs that are contiguous in a row, and
+    // 16 lanes that are served together read one or two rows' runs: whole memory lines, the shape in which a large
+    // matrix streams fastest (a bare read loop: 5.95 TB/s against 5.04 in the operand shape for [51200, 5120]).
+    // Nothing is held in registers meanwhile, so the chunks are short and the waves many.  Rows are staged 18
+    // pieces apart (16 of a chunk's 4 steps and 2 of padding): the operand reads then find their rows 8 (mod 16)
+    // banks apart (see SK_STRIDE below).  Request f / 64, lane f % 64 fetches piece f % 18 of staged row f / 18.
+    static_assert(MB == 1, "this mode takes up to 16 rows of the left operand");
+    constexpr int C5 = SKINNY_STAGE5_STEPS, ROWP = 4 * C5 + 2;
+    constexpr int NIW = SKINNY_STAGE5_KB(RB), NIA = SKINNY_STAGE5_KB(1);
+    const int q = lane >> 4, r = lane & 15;
+    // a wave's pieces: NIW KB for the weights, then as many KB as the M rows of the left operand need (rows past M
+    // are read from whatever lies there; their results are dropped)
+    const int kb_a = (M * ROWP + 63) / 64;
+    uint16_t* stage_w = reinterpret_cast<uint16_t*>(red) + (size_t)wave * ((NIW + kb_a) * 512);
+    uint16_t* stage_a = stage_w + NIW * 512;
+    uint32_t w_off[NIW], a_off[NIA];
+    int w_stp[NIW], a_stp[NIA];       // the step of the chunk a lane's piece belongs to; C5: never fetched
+#pragma unroll
+    for (int i = 0; i < NIW; ++i) {
+      const int f = 64 * i + lane;
+      const int R = f / ROWP, piece = f - R * ROWP;
+      const bool live = R < 16 * RB && piece < 4 * C5;
+      int row = n0 + (GATE_UP ? 0 : rpg * (R >> 4)) + min(R & 15, rpg - 1);
+      row = min(row, N - 1);
+      if (GATE_UP && (R >> 4) == 1) row += N;
+      w_off[i] = live ? ((uint32_t)row * (uint32_t)ldw + 8 * piece) * 2 : 0;
+      w_stp[i] = live ? piece >> 2 : C5;
+    }
+    const char* wb = reinterpret_cast<const char*>(W) + (int64_t)s_begin * 64;
+    const char* ab = reinterpret_cast<const char*>(A) + (int64_t)s_begin * 64;
+    bool first = true;
+    for (int left = s_end - s_begin; left > 0; left -= C5, wb += 64 * C5, ab += 64 * C5) {
+      const int n = min(left, C5);                      // steps of this chunk: the same for the whole wave
+#pragma unroll
+      for (int i = 0; i < NIW; ++i)
+        if (w_stp[i] < n)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wb + w_off[i]),
+                                           (__attribute__((address_space(3))) void*)(stage_w + 512 * i), 16, 0, 0);
+      if (first) {
+        first = false;
+        SKINNY_NORM_PREFETCH()
+        int lane_late = lane;
+        asm volatile("" : "+v"(lane_late));             // keeps the compiler from moving this in front of the loop
+#pragma unroll
+        for (int i = 0; i < NIA; ++i) {
+          const int f = 64 * i + lane_late;
+          const int R = f / ROWP, piece = f - R * ROWP;
+          const bool live = R < M && piece < 4 * C5;
+          a_off[i] = live ? ((uint32_t)R * (uint32_t)lda + 8 * piece) * 2 : 0;
+          a_stp[i] = live ? piece >> 2 : C5;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NIA; ++i)
+        if (a_stp[i] < n)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ab + a_off[i]),
+                                           (__attribute__((address_space(3))) void*)(stage_a + 512 * i), 16, 0, 0);
+      // The compiler does not count the requests that write LDS when it places the waits of the reads below: the
+      // wait is written out, and nothing moves across it.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int c = 0; c < C5; ++c) {
+        if (c < n) {
+          union {
+            u32x4 u;
+            bf16x8 v;
+          } a, b;
+          a.u = *reinterpret_cast<const u32x4*>(stage_a + 8 * (r * ROWP + 4 * c + q));
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            b.u = *reinterpret_cast<const u32x4*>(stage_w + 8 * ((16 * rb + r) * ROWP + 4 * c + q));
+            acc[rb][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, a.v, acc[rb][0], 0, 0, 0);
+          }
+        }
+      }
+      // the reads above are done (their products have been issued) before the next chunk's requests overwrite them
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    if (first) SKINNY_NORM_PREFETCH()                   // a wave without a step of its own
+    __syncthreads();                                    // the staging pieces are given up: the sums go where they were
   } else {
     const int q = lane >> 4, r = lane & 15;
     // byte offsets of the lane's 16 bytes in step 0 of the wave's range, from W + 64 s_begin and A + 64 s_begin
@@ -546,10 +630,15 @@ MI_EXPORT int mi_norm_gemm_skinny(int gate_up, const float* R, const void* X, fl
   return 0;
 }
 
-static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up, bool a_lds = false) {
+// staging: 0 none, 1 the left operand's pieces, 2 both operands' (the mode for up to 16 rows)
+static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up, int staging = 0, int M = 16) {
   const int OB = gate_up ? MB : RB * MB;
   const size_t sums = ((size_t)((waves + 1) / 2) * RB * MB * 256 + (size_t)OB * 256 + (size_t)waves * 64) * sizeof(float);
-  const size_t stage = a_lds ? (size_t)waves * SKINNY_STAGE_KB(MB) * 1024 : 0;    // the left operand's staging pieces
+  const size_t stage = staging == 1   ? (size_t)waves * SKINNY_STAGE_KB(MB) * 1024
+                       : staging == 2
+                           ? (size_t)waves * (SKINNY_STAGE5_KB(RB) + (M * (4 * SKINNY_STAGE5_STEPS + 2) + 63) / 64) * 1024 +
+                                 16 * (4 * SKINNY_STAGE5_STEPS + 2) * 16      // the last wave's reads of rows past M
+                           : 0;
   return sums > stage ? sums : stage;
 }
 
@@ -615,7 +704,7 @@ static void launch_instance(dim3 grid, dim3 block, size_t lds, hipStream_t strea
                             const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K, int rpg,
                             const NormHalves& nh) {
   auto kernel = gemm_skinny_kernel<MB, RB, F32, GU, MODE>;
-  if (MODE == 2 || MODE == 4) {     // its staging pieces may need more than the default allotment of LDS
+  if (MODE == 2 || MODE >= 4) {     // its staging pieces may need more than the default allotment of LDS
     static bool allowed = false;
     if (!allowed) {
       (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -628,23 +717,28 @@ static void launch_instance(dim3 grid, dim3 block, size_t lds, hipStream_t strea
 template <int MB, int RB>
 static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                   int64_t ldc, int M, int N, int K, int waves, const SkinnyGrid& sg, const NormHalves& nh,
-                  bool staged, bool lines, hipStream_t stream) {
+                  int want, hipStream_t stream) {
   const dim3 grid(sg.groups);
   const dim3 block(64 * waves);
   const int64_t w_rows = gate_up ? 2 * (int64_t)N : N;
   const bool lean = K % 32 == 0 && w_rows * ldw * 2 < ((int64_t)1 << 32) && (int64_t)M * lda * 2 < ((int64_t)1 << 32) &&
                     (((uintptr_t)A | (uintptr_t)W) & 15) == 0;
-  // the left operand goes through LDS where the caller asks for it and the staging pieces fit; the weights come in
-  // whole memory lines where the caller asks for that and K is a multiple of 64
+  // want: the kernel's mode the caller asks for (1 .. 5); it is taken as far as the shape allows
   int mode = 0;
   if (lean) {
-    mode = staged && skinny_lds_bytes(waves, RB, MB, gate_up, true) <= 144 * 1024 ? 2 : 1;
-    if (lines && K % 64 == 0) mode += 2;
+    mode = want < 1 ? 1 : want;
+    const size_t room = 144 * 1024;
+    if (mode == 5 && (MB != 1 || skinny_lds_bytes(waves, RB, MB, gate_up, 2, M) > room)) mode = 2;
+    if ((mode == 3 || mode == 4) && K % 64 != 0) mode -= 2;
+    if ((mode == 2 || mode == 4) && skinny_lds_bytes(waves, RB, MB, gate_up, 1) > room) mode -= 1;
   }
-  const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up, mode == 2 || mode == 4);
+  const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up, mode == 5 ? 2 : (mode == 2 || mode == 4) ? 1 : 0, M);
 #define GO(F32, GU)                                                                                                  \
   {                                                                                                                  \
-    if (mode == 4) launch_instance<MB, RB, F32, GU, 4>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
+    if (mode == 5) {                                                                                                 \
+      if constexpr (MB == 1)                                                                                         \
+        launch_instance<MB, RB, F32, GU, 5>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh);  \
+    } else if (mode == 4) launch_instance<MB, RB, F32, GU, 4>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
     else if (mode == 3) launch_instance<MB, RB, F32, GU, 3>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
     else if (mode == 2) launch_instance<MB, RB, F32, GU, 2>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
     else if (mode == 1) launch_instance<MB, RB, F32, GU, 1>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
@@ -672,8 +766,8 @@ MI_EXPORT int mi_gemm_skinny_ss_row(int M) { return SS_ROW(M); }
 // residual [M, N] float32 + norm_weight [N] + a_out [M, N] bfloat16 + ss_out [groups][ss_row(M)] replace C.
 static int skinny_rows(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                        int64_t ldc, int M, int N, int K, const float* row_ss, int ss_parts, float eps,
-                       float* residual, const float* norm_weight, void* a_out, float* ss_out, bool staged,
-                       bool lines, hipStream_t stream) {
+                       float* residual, const float* norm_weight, void* a_out, float* ss_out, int want,
+                       hipStream_t stream) {
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);
   MI_REQUIRE(lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: row strides (%lld, %lld) must be multiples of 8", (long long)lda,
@@ -700,8 +794,7 @@ static int skinny_rows(int out_f32, int gate_up, const void* A, int64_t lda, con
   const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \
-    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, staged, lines,    \
-                   stream);                                                                                 \
+    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, want, stream);    \
     MI_CHECK_LAUNCH("gemm_skinny");                                                                           \
     return 0;                                                                                                 \
   }
@@ -715,7 +808,7 @@ MI_EXPORT int mi_gemm_skinny_ex(int out_f32, int gate_up, const void* A, int64_t
                                 float eps, float* residual, const float* norm_weight, void* a_out, float* ss_out,
                                 hipStream_t stream) {
   return skinny_rows(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual, norm_weight,
-                     a_out, ss_out, false, false, stream);
+                     a_out, ss_out, 1, stream);
 }
 
 MI_EXPORT int mi_gemm_skinny(int out_f32, int gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
@@ -993,7 +1086,7 @@ static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
 // is the first half of a norm (`ss_parts`), and the floats of scratch it needs (0 for every variant but 1).
 MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K, int* ss_parts, int64_t* scratch_floats) {
   MI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_plan: M=%d N=%d K=%d", M, N, K);
-  MI_REQUIRE(variant >= 0 && variant <= 4, "gemm_skinny_plan: variant %d", variant);
+  MI_REQUIRE(variant >= 0 && variant <= 5, "gemm_skinny_plan: variant %d", variant);
   if (variant != 1) {
     if (ss_parts) *ss_parts = skinny_grid(gate_up != 0, N, M).groups;
     if (scratch_floats) *scratch_floats = 0;
@@ -1008,16 +1101,17 @@ MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K,
 // mi_gemm_skinny_ex with a choice of kernel: variant 0 = every workgroup owns whole rows of the result (above),
 // variant 1 = k split across workgroups, partial results in `scratch` (float, at least the plan's scratch_floats),
 // added in the order of the splits by a second kernel that also does the endings; variant 2 = variant 0 with the left
-// operand staged through LDS; variants 3 and 4 = variants 0 and 2 with the weights fetched in whole memory lines
-// (each where the shape allows it; else without).  Variants 0 and 2 add the same products in the same order: their
-// results are equal bit for bit, and so are those of 3 and 4.
+// operand staged through LDS; variants 3 and 4 = variants 0 and 2 with the weights fetched in whole memory lines;
+// variant 5 = both operands staged through LDS, for up to 16 rows (each where the shape allows it; else the nearest
+// that it does).  Variants 0, 2 and 5 add the same products in the same order: their results are equal bit for
+// bit, and so are those of 3 and 4.
 MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void* A, int64_t lda, const void* W,
                                int64_t ldw, void* C, int64_t ldc, int M, int N, int K, const float* row_ss,
                                int ss_parts, float eps, float* residual, const float* norm_weight, void* a_out,
                                float* ss_out, float* scratch, int64_t scratch_floats, hipStream_t stream) {
-  if (variant != 1 && variant >= 0 && variant <= 4)
+  if (variant != 1 && variant >= 0 && variant <= 5)
     return skinny_rows(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual, norm_weight,
-                       a_out, ss_out, variant == 2 || variant == 4, variant >= 3, stream);
+                       a_out, ss_out, variant == 0 ? 1 : variant, stream);
   MI_REQUIRE(variant == 1, "gemm_skinny: variant %d", variant);
   MI_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: M=%d; this kernel takes at most 64 rows", M);
   MI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: N=%d K=%d (K must be a multiple of 8)", N, K);

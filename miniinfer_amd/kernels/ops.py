@@ -337,9 +337,13 @@ SKINNY_OWN_ELEMENTS = 8 << 20        # and for more rows (up to SKINNY_MAX_ROWS)
 TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_products` times the candidates
 # (rows point, matrix rows, k, gate|up) -> the quickest: LIBRARY, or this library's kernel in which every workgroup
 # owns whole rows of the result (OWN_ROWS; OWN_ROWS_STAGED: with the left operand staged through LDS; OWN_ROWS_LINES,
-# OWN_ROWS_STAGED_LINES: the same two with the weights fetched in whole memory lines), or the one that splits k
-# across workgroups (OWN_KSPLIT).  An own kernel's choice is its variant number + 1.
-LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES = 0, 1, 2, 3, 4, 5
+# OWN_ROWS_STAGED_LINES: the same two with the weights fetched in whole memory lines; OWN_ROWS_BOTH_STAGED: both
+# operands through LDS, for up to 16 rows), or the one that splits k across workgroups (OWN_KSPLIT).  An own kernel's
+# choice is its variant number + 1.
+LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES, OWN_ROWS_BOTH_STAGED = range(7)
+# (the kernel takes up to 16 rows; from 9 rows up its staging pieces leave room for 9 waves on a compute unit instead
+# of 12, and inside a step it then lost to the other forms what it had won when timed alone)
+BOTH_STAGED_MAX_ROWS = 8
 _PRODUCT_CHOICE: Dict[tuple, int] = {}
 KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
 KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)
@@ -436,7 +440,8 @@ def skinny_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fals
   same with the left operand staged through LDS (read in whole memory lines, which costs a little when the operand
   is small and saves much when it is not; the same sums bit for bit); 3, 4 = 0 and 2 with the weights fetched in
   whole memory lines too (two steps of k at a time, put in place by an exchange between lanes: large matrices
-  stream faster that way); 1 = k is split across workgroups, which read a slice of the left operand each and
+  stream faster that way); 5 = both operands staged through LDS, every request for whole lines (up to 16 rows;
+  the same sums as 0 bit for bit); 1 = k is split across workgroups, which read a slice of the left operand each and
   leave 32-bit partial results that a second kernel adds in a fixed order.
   Measured where `tuning.tune_products` has been; else by rule."""
   c = _measured_choice(num_rows, matrix_rows, k, gate_up)
@@ -451,8 +456,11 @@ def _rule_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> int
   if can_split and num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K:
     return 1
   # (a matrix of very many rows, the output head, has as many workgroups re-reading the left operand: staged too)
-  if num_rows >= STAGED_MIN_ROWS and (num_rows * k >= STAGED_MIN_ELEMENTS or matrix_rows * k >= LINES_MIN_ELEMENTS):
-    return 4 if matrix_rows * k >= LINES_MIN_ELEMENTS and k >= LINES_MIN_K and k % 64 == 0 else 2
+  large = matrix_rows * k >= LINES_MIN_ELEMENTS
+  if num_rows >= STAGED_MIN_ROWS and (num_rows * k >= STAGED_MIN_ELEMENTS or large):
+    if large and k >= LINES_MIN_K and k % 64 == 0 and not gate_up:
+      return 4
+    return 5 if large and num_rows <= BOTH_STAGED_MAX_ROWS and k % 32 == 0 else 2
   return 0
 
 

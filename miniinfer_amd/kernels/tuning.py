@@ -96,8 +96,9 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
 
       # The kernel in which a workgroup owns whole rows of the result, in its forms: with the left operand staged
       # through LDS it is a few tenths of a microsecond slower when the operand is small and up to a quarter quicker
-      # when it is not; with the weights fetched in whole memory lines large matrices stream up to a tenth faster
-      # and small ones slower.  Which, depends on the shape.
+      # when it is not; with the weights fetched in whole memory lines, by loads into registers and an exchange
+      # between lanes or through LDS like the left operand, large matrices stream up to a sixth faster and small
+      # ones slower.  Which, depends on the shape.
       forms = {ops.OWN_ROWS: graph_time_us(own(0), calls, flush)}
       stage = M >= ops.STAGED_MIN_ROWS and K % 32 == 0
       if stage:
@@ -105,6 +106,8 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
       if K % 64 == 0 and rows_w * K >= LINES_MIN_ELEMENTS:
         c = ops.OWN_ROWS_STAGED_LINES if stage else ops.OWN_ROWS_LINES
         forms[c] = graph_time_us(own(c - 1), calls, flush)
+      if stage and M <= ops.BOTH_STAGED_MAX_ROWS and rows_w * K >= LINES_MIN_ELEMENTS:
+        forms[ops.OWN_ROWS_BOTH_STAGED] = graph_time_us(own(5), calls, flush)
       rows_choice = min(forms, key=forms.get)
       t_rows = forms[rows_choice]
       # k is split from 16 rows up only: below, the left operand is too small for its re-reads to matter, and the
@@ -132,7 +135,8 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
       if log is not None:
         names = {ops.LIBRARY: "library", ops.OWN_ROWS: "own", ops.OWN_KSPLIT: "own with k split",
                  ops.OWN_ROWS_STAGED: "own, left operand staged", ops.OWN_ROWS_LINES: "own, weights in whole lines",
-                 ops.OWN_ROWS_STAGED_LINES: "own, left operand staged, weights in whole lines"}
+                 ops.OWN_ROWS_STAGED_LINES: "own, left operand staged, weights in whole lines",
+                 ops.OWN_ROWS_BOTH_STAGED: "own, both operands staged"}
         log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: "
             + ", ".join(f"{names[c]} {t:.1f} us" for c, t in forms.items())
             + f", own with k split {t_split:.1f} us, library {t_lib:.1f} us with its extra kernels -> {names[choice]}")

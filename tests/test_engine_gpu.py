@@ -265,7 +265,7 @@ def test_cache_is_sized_from_device_memory_when_no_page_count_is_given(tmp_path)
     LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, gpu_memory_utilization=1e-3)
 
 
-@pytest.mark.parametrize("products", ["own", "own_ksplit", "own_staged", "own_staged_lines", "library"])
+@pytest.mark.parametrize("products", ["own", "own_ksplit", "own_staged", "own_staged_lines", "own_both_staged", "library"])
 def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, products):
   """The engine's choice between its own weight-streaming products (whole rows per workgroup, with or without the
   left operand staged through LDS and the weights fetched in whole lines, or k split across workgroups) and the library's is a matter of speed: with every
@@ -282,7 +282,8 @@ def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, produ
         outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
     else:
       choice = {"own_ksplit": ops.OWN_KSPLIT, "own_staged": ops.OWN_ROWS_STAGED,
-                "own_staged_lines": ops.OWN_ROWS_STAGED_LINES, "library": ops.LIBRARY}[products]
+                "own_staged_lines": ops.OWN_ROWS_STAGED_LINES, "own_both_staged": ops.OWN_ROWS_BOTH_STAGED,
+                "library": ops.LIBRARY}[products]
       for rows in ops.TUNE_ROWS:
         for m in eng.model.products():
           ops.set_product_choice(rows, m[0].shape[0], m[0].shape[1], m[1], choice)

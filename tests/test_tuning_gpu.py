@@ -36,8 +36,8 @@ def test_products_are_timed_once_per_shape_and_small_ones_are_left_alone(clean_c
 
 
 # the library / whole rows per workgroup / k split across workgroups / whole rows with the left operand staged /
-# whole rows with the weights in whole lines / both
-@pytest.mark.parametrize("choice", [0, 1, 2, 3, 4, 5])
+# whole rows with the weights in whole lines / both / both operands staged
+@pytest.mark.parametrize("choice", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("M", [3, 16, 40])
 def test_either_choice_gives_the_product(clean_choices, choice, M):
   ops = clean_choices
