@@ -1,9 +1,10 @@
 """Which kernel runs a product of few rows is measured, not guessed.
 
-For a matrix of tens of MB and a handful of rows there are three candidates: this library's weight-streaming kernel
+For a matrix of tens of MB and a handful of rows there are these candidates: this library's weight-streaming kernel
 (`ops.gemm_skinny`, whose epilogue can take a norm's halves or the gated activation) in its forms (every
-workgroup owns whole rows of the result, with the left operand straight from memory or staged through LDS, or k is
-split across workgroups and a second kernel adds the partial results), and the library product
+workgroup owns whole rows of the result, with the operands straight from memory, the left one or both staged through
+LDS, the weights in half or whole memory lines; or k is split across workgroups and a second kernel adds the partial
+results), and the library product
 (hipBLASLt through `torch.matmul`, which splits k across workgroups and so reads the left operand less often, but
 needs the norm and the activation as kernels of their own).  Which is quicker depends on the shape and the number
 of rows in ways no short rule covers, so `tune_products` times them on the model's own matrices once, when an
