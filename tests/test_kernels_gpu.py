@@ -387,6 +387,38 @@ def test_gemm_skinny(M, N, K, out_dtype, variant):
     assert torch.equal(out, same)
 
 
+def test_gemm_skinny_drawn_shapes():
+  """Every form of the weight-streaming product on shapes drawn at random (rows 1 to 64, k a multiple of 8 from 8 to
+  6,400, 1 to 5,000 columns, left operands with a row stride of their own, a third of them gate|up), against 64-bit
+  arithmetic; and the forms that only change where the operands come from give the very same sums."""
+  import random
+  from miniinfer_amd.kernels import ops
+  rng = random.Random(3)
+  for it in range(48):
+    M = rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32, 33, 47, 48, 63, 64])
+    K = 8 * rng.choice([1, 3, 4, 5, 8, 9, 12, 16, 24, 31, 32, 40, 64, 72, 100, 128, 192, 264, 320, 512, 800])
+    N = rng.choice([1, 3, 5, 16, 17, 33, 64, 100, 129, 256, 500, 1000, 2050, 5000])
+    gate_up = rng.random() < 0.3
+    if gate_up and rng.random() < 0.7:
+      N = (N + 3) // 4 * 4
+    g = torch.Generator().manual_seed(it)
+    a = torch.randn(M, K + rng.choice([0, 0, 8, 16, 64]), generator=g).bfloat16().to(DEV)[:, :K]
+    w = (torch.randn(2 * N if gate_up else N, K, generator=g) * 0.1).bfloat16().to(DEV)
+    want = a.double() @ w.double().T
+    if gate_up:
+      want = torch.nn.functional.silu(want[:, :N]) * want[:, N:]
+    outs = {}
+    for variant in (0, 1, 2, 3, 4, 5):
+      if variant == 1 and gate_up and N % 4:
+        continue
+      out = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+      ops.gemm_skinny(a, w, out, gate_up=gate_up, variant=variant)
+      torch.testing.assert_close(out.double(), want, rtol=2e-4, atol=2e-4 * K ** 0.5,
+                                 msg=lambda m: f"variant {variant}, {M} x [{N}, {K}] gate_up={gate_up}: {m}")
+      outs[variant] = out
+    assert torch.equal(outs[2], outs[0]) and torch.equal(outs[5], outs[0]) and torch.equal(outs[4], outs[3]), (M, N, K)
+
+
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 112, 80), (40, 160, 96), (64, 100, 256), (33, 1028, 2200),
                                    (8, 1536, 4096), (16, 516, 2048), (48, 260, 1024), (3, 200, 5120), (20, 36, 448)])
