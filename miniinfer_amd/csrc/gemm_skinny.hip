@@ -38,9 +38,9 @@ __device__ __forceinline__ float silu_f(float g) { return g / (1.f + expf(-g)); 
 #define SKINNY_CH(mb) ((mb) == 1 ? 8 : ((mb) == 2 ? 4 : 2))   // steps of K whose loads are asked for together
 // KB of LDS in which a wave stages a chunk of the left operand: 16 mb rows of 4 CH pieces of 16 bytes
 #define SKINNY_STAGE_KB(mb) ((mb) * SKINNY_CH(mb))
-// The mode that stages both operands: steps per chunk, and KB for 16 blocks rows of 4 steps + 2 pieces each
+// The mode that stages both operands: steps per chunk, and KB for 16 blocks rows of 4 steps each
 #define SKINNY_STAGE5_STEPS 4
-#define SKINNY_STAGE5_KB(blocks) ((16 * (blocks) * (4 * SKINNY_STAGE5_STEPS + 2) + 63) / 64)
+#define SKINNY_STAGE5_KB(blocks) (16 * (blocks) * 4 * SKINNY_STAGE5_STEPS / 64)
 struct NormHalves {
   const float* row_ss;      // [ss_parts][SS_ROW(M)]
   int ss_parts;
@@ -190,13 +190,16 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     }
   } else if constexpr (MODE == 5) {
     // Both operands through LDS (at most 16 rows of A).  Every request reads runs that are contiguous in a row, and
-    // 16 lanes that are served together read one or two rows' runs: whole memory lines, the shape in which a large
-    // matrix streams fastest (a bare read loop: 5.95 TB/s against 5.04 in the operand shape for [51200, 5120]).
-    // Nothing is held in registers meanwhile, so the chunks are short and the waves many.  Rows are staged 18
-    // pieces apart (16 of a chunk's 4 steps and 2 of padding): the operand reads then find their rows 8 (mod 16)
-    // banks apart (see SK_STRIDE below).  Request f / 64, lane f % 64 fetches piece f % 18 of staged row f / 18.
+    // 16 lanes that are served together read one row's run: whole memory lines, the shape in which a large matrix
+    // streams fastest (a bare read loop: 5.95 TB/s against 5.04 in the operand shape for [51200, 5120]).  Nothing
+    // is held in registers meanwhile, so the chunks are short (4 steps: 16 pieces of 16 bytes per row) and the
+    // waves many: what is in flight is what fits a compute unit's LDS.  Request f / 64, lane f % 64 fetches for the
+    // place f % 16 of staged row f / 16 the piece (f % 16) ^ 2 (row % 4): an operand read (lanes l .. l + 3 with
+    // l + 16 .. l + 19: 4 rows x 2 neighbouring pieces) then finds its 8 pieces in 8 different places (mod 8), that
+    // is in different banks, without a byte of padding.
     static_assert(MB == 1, "this mode takes up to 16 rows of the left operand");
-    constexpr int C5 = SKINNY_STAGE5_STEPS, ROWP = 4 * C5 + 2;
+    constexpr int C5 = SKINNY_STAGE5_STEPS, ROWP = 4 * C5;
+    static_assert(ROWP == 16, "the places of a row are swapped among 16");
     constexpr int NIW = SKINNY_STAGE5_KB(RB), NIA = SKINNY_STAGE5_KB(1);
     const int q = lane >> 4, r = lane & 15;
     // a wave's pieces: NIW KB for the weights, then as many KB as the M rows of the left operand need (rows past M
@@ -208,17 +211,17 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
     int w_stp[NIW], a_stp[NIA];       // the step of the chunk a lane's piece belongs to; C5: never fetched
 #pragma unroll
     for (int i = 0; i < NIW; ++i) {
-      const int f = 64 * i + lane;
-      const int R = f / ROWP, piece = f - R * ROWP;
-      const bool live = R < 16 * RB && piece < 4 * C5;
+      const int R = 4 * i + (lane >> 4);                // staged row; 16 lanes per row
+      const int piece = (lane & 15) ^ (2 * (R & 3));
       int row = n0 + (GATE_UP ? 0 : rpg * (R >> 4)) + min(R & 15, rpg - 1);
       row = min(row, N - 1);
       if (GATE_UP && (R >> 4) == 1) row += N;
-      w_off[i] = live ? ((uint32_t)row * (uint32_t)ldw + 8 * piece) * 2 : 0;
-      w_stp[i] = live ? piece >> 2 : C5;
+      w_off[i] = ((uint32_t)row * (uint32_t)ldw + 8 * piece) * 2;
+      w_stp[i] = piece >> 2;
     }
     const char* wb = reinterpret_cast<const char*>(W) + (int64_t)s_begin * 64;
     const char* ab = reinterpret_cast<const char*>(A) + (int64_t)s_begin * 64;
+    const int swz = 2 * (r & 3);                        // how this lane's row has its places swapped
     bool first = true;
     for (int left = s_end - s_begin; left > 0; left -= C5, wb += 64 * C5, ab += 64 * C5) {
       const int n = min(left, C5);                      // steps of this chunk: the same for the whole wave
@@ -234,11 +237,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         asm volatile("" : "+v"(lane_late));             // keeps the compiler from moving this in front of the loop
 #pragma unroll
         for (int i = 0; i < NIA; ++i) {
-          const int f = 64 * i + lane_late;
-          const int R = f / ROWP, piece = f - R * ROWP;
-          const bool live = R < M && piece < 4 * C5;
-          a_off[i] = live ? ((uint32_t)R * (uint32_t)lda + 8 * piece) * 2 : 0;
-          a_stp[i] = live ? piece >> 2 : C5;
+          const int R = 4 * i + (lane_late >> 4);
+          const int piece = (lane_late & 15) ^ (2 * (R & 3));
+          a_off[i] = R < M ? ((uint32_t)R * (uint32_t)lda + 8 * piece) * 2 : 0;
+          a_stp[i] = R < M ? piece >> 2 : C5;
         }
       }
 #pragma unroll
@@ -256,10 +258,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
             u32x4 u;
             bf16x8 v;
           } a, b;
-          a.u = *reinterpret_cast<const u32x4*>(stage_a + 8 * (r * ROWP + 4 * c + q));
+          const int place = (4 * c + q) ^ swz;
+          a.u = *reinterpret_cast<const u32x4*>(stage_a + 8 * (r * ROWP + place));
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
-            b.u = *reinterpret_cast<const u32x4*>(stage_w + 8 * ((16 * rb + r) * ROWP + 4 * c + q));
+            b.u = *reinterpret_cast<const u32x4*>(stage_w + 8 * ((16 * rb + r) * ROWP + place));
             acc[rb][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b.v, a.v, acc[rb][0], 0, 0, 0);
           }
         }
@@ -636,8 +639,8 @@ static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up, int stag
   const size_t sums = ((size_t)((waves + 1) / 2) * RB * MB * 256 + (size_t)OB * 256 + (size_t)waves * 64) * sizeof(float);
   const size_t stage = staging == 1   ? (size_t)waves * SKINNY_STAGE_KB(MB) * 1024
                        : staging == 2
-                           ? (size_t)waves * (SKINNY_STAGE5_KB(RB) + (M * (4 * SKINNY_STAGE5_STEPS + 2) + 63) / 64) * 1024 +
-                                 16 * (4 * SKINNY_STAGE5_STEPS + 2) * 16      // the last wave's reads of rows past M
+                           ? (size_t)waves * (SKINNY_STAGE5_KB(RB) + (M * 4 * SKINNY_STAGE5_STEPS + 63) / 64) * 1024 +
+                                 16 * 4 * SKINNY_STAGE5_STEPS * 16            // the last wave's reads of rows past M
                            : 0;
   return sums > stage ? sums : stage;
 }

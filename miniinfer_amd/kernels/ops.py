@@ -341,9 +341,7 @@ TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_produ
 # operands through LDS, for up to 16 rows), or the one that splits k across workgroups (OWN_KSPLIT).  An own kernel's
 # choice is its variant number + 1.
 LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES, OWN_ROWS_BOTH_STAGED = range(7)
-# (the kernel takes up to 16 rows; from 9 rows up its staging pieces leave room for 9 waves on a compute unit instead
-# of 12, and inside a step it then lost to the other forms what it had won when timed alone)
-BOTH_STAGED_MAX_ROWS = 8
+BOTH_STAGED_MAX_ROWS = 16
 _PRODUCT_CHOICE: Dict[tuple, int] = {}
 KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
 KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)

@@ -34,7 +34,7 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     # gate|up matrix whose halves are no multiple of 4 rows; else the left operand is staged through LDS when it
     # has at least 4 rows and 12 K elements, and the weights come in whole lines when, besides, the matrix has 40 M
     # elements in rows of 5,120 or more (a multiple of 64); other matrices of that size (gate|up, shorter rows) have
-    # both operands staged for up to 8 rows
+    # both operands staged for up to 16 rows
     assert ops.skinny_variant(64, 1024, 3072) == 1 and ops.skinny_variant(17, 1024, 2048) == 1
     assert ops.skinny_variant(16, 1024, 3072) == 2 and ops.skinny_variant(64, 4096, 1024) == 2
     assert ops.skinny_variant(4, 1024, 2048) == 0 and ops.skinny_variant(8, 4096, 1024) == 0
@@ -42,7 +42,7 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     assert ops.skinny_variant(8, 4096, 12288) == 4 and ops.skinny_variant(3, 4096, 25600) == 0
     assert ops.skinny_variant(16, 6144, 4096) == 2 and ops.skinny_variant(8, 151936, 1024) == 5
     assert ops.skinny_variant(8, 51200, 5120, True) == 5 and ops.skinny_variant(8, 5120, 25632) == 5
-    assert ops.skinny_variant(8, 5120, 25600) == 4 and ops.skinny_variant(16, 24576, 4096, True) == 2 and ops.skinny_variant(8, 24576, 4096, True) == 5
+    assert ops.skinny_variant(8, 5120, 25600) == 4 and ops.skinny_variant(16, 24576, 4096, True) == 5 and ops.skinny_variant(8, 24576, 4096, True) == 5
     assert ops.skinny_variant(64, 2 * 1026, 4096, True) == 2 and ops.skinny_variant(64, 2 * 1028, 4096, True) == 1
     for p in ops.TUNE_ROWS:
       ops.set_product_choice(p, 4096, 4096, False, p > 8)
