@@ -342,6 +342,8 @@ TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_produ
 # choice is its variant number + 1.
 LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES, OWN_ROWS_BOTH_STAGED = range(7)
 BOTH_STAGED_MAX_ROWS = 16
+BOTH_STAGED_ANY_ELEMENTS = 16 << 20  # without a measurement: both operands are staged for matrices of this size,
+BOTH_STAGED_MIN_K = 2048             # or with rows of at least this many columns where no activation follows
 _PRODUCT_CHOICE: Dict[tuple, int] = {}
 KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
 KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)
@@ -453,13 +455,23 @@ def _rule_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> int
   can_split = not (gate_up and (matrix_rows // 2) % 4)
   if can_split and num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K:
     return 1
-  # (a matrix of very many rows, the output head, has as many workgroups re-reading the left operand: staged too)
   large = matrix_rows * k >= LINES_MIN_ELEMENTS
+  if num_rows >= STAGED_MIN_ROWS and large and k >= LINES_MIN_K and k % 64 == 0 and not gate_up:
+    return 4
+  if both_staged_offered(num_rows, matrix_rows, k, gate_up):
+    return 5
+  # (a matrix of very many rows, the output head, has as many workgroups re-reading the left operand: staged too)
   if num_rows >= STAGED_MIN_ROWS and (num_rows * k >= STAGED_MIN_ELEMENTS or large):
-    if large and k >= LINES_MIN_K and k % 64 == 0 and not gate_up:
-      return 4
-    return 5 if large and num_rows <= BOTH_STAGED_MAX_ROWS and k % 32 == 0 else 2
+    return 2
   return 0
+
+
+def both_staged_offered(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> bool:
+  """Whether the form with both operands staged through LDS is a candidate.  A small gate|up matrix, or one with
+  short rows, is none: timed alone it is as quick or quicker that way, but inside a decode step (Qwen3-0.6B's
+  [4096, 1024] and gate|up [6144, 1024], 1 to 16 rows) the step takes a quarter of a microsecond more per product."""
+  return (num_rows <= BOTH_STAGED_MAX_ROWS and k % 32 == 0
+          and (matrix_rows * k >= BOTH_STAGED_ANY_ELEMENTS or (not gate_up and k >= BOTH_STAGED_MIN_K)))
 
 
 def rule_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> int:

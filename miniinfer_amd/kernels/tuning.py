@@ -98,8 +98,9 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
       # The kernel in which a workgroup owns whole rows of the result, in its forms: with the left operand staged
       # through LDS it is a few tenths of a microsecond slower when the operand is small and up to a quarter quicker
       # when it is not; with the weights fetched in whole memory lines, by loads into registers and an exchange
-      # between lanes or through LDS like the left operand, large matrices stream up to a sixth faster and small
-      # ones slower.  Which, depends on the shape.
+      # between lanes, large matrices stream up to a sixth faster and small ones slower; with both operands through
+      # LDS (up to 16 rows) most shapes run a few percent quicker (small ones do not inside a step, and are not timed).
+      # Which, depends on the shape.
       forms = {ops.OWN_ROWS: graph_time_us(own(0), calls, flush)}
       stage = M >= ops.STAGED_MIN_ROWS and K % 32 == 0
       if stage:
@@ -107,7 +108,7 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
       if K % 64 == 0 and rows_w * K >= LINES_MIN_ELEMENTS:
         c = ops.OWN_ROWS_STAGED_LINES if stage else ops.OWN_ROWS_LINES
         forms[c] = graph_time_us(own(c - 1), calls, flush)
-      if stage and M <= ops.BOTH_STAGED_MAX_ROWS and rows_w * K >= LINES_MIN_ELEMENTS:
+      if ops.both_staged_offered(M, rows_w, K, gate_up):
         forms[ops.OWN_ROWS_BOTH_STAGED] = graph_time_us(own(5), calls, flush)
       rows_choice = min(forms, key=forms.get)
       t_rows = forms[rows_choice]

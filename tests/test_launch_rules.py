@@ -31,18 +31,25 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     assert not ops.skinny_preferred(17, 4096, 4096)                   # a large one with more than 16 rows
     assert not ops.skinny_preferred(65, 64, 64)                       # more rows than the kernel takes
     # which of the own kernels: k is split for more than 16 rows of 2,048 columns and more, and never for a
-    # gate|up matrix whose halves are no multiple of 4 rows; else the left operand is staged through LDS when it
-    # has at least 4 rows and 12 K elements, and the weights come in whole lines when, besides, the matrix has 40 M
-    # elements in rows of 5,120 or more (a multiple of 64); other matrices of that size (gate|up, shorter rows) have
-    # both operands staged for up to 16 rows
+    # gate|up matrix whose halves are no multiple of 4 rows; from 4 rows up the weights come in whole lines, with the
+    # left operand staged, when the matrix has 40 M elements in rows of 5,120 or more (a multiple of 64; not gate|up);
+    # else up to 16 rows have both operands staged through LDS (k a multiple of 32) when the matrix has 16 M
+    # elements, or rows of 2,048 columns and no activation behind it; what is left has the left operand staged from
+    # 4 rows and 12 K elements
     assert ops.skinny_variant(64, 1024, 3072) == 1 and ops.skinny_variant(17, 1024, 2048) == 1
-    assert ops.skinny_variant(16, 1024, 3072) == 2 and ops.skinny_variant(64, 4096, 1024) == 2
-    assert ops.skinny_variant(4, 1024, 2048) == 0 and ops.skinny_variant(8, 4096, 1024) == 0
-    assert ops.skinny_variant(4, 1024, 3072) == 2 and ops.skinny_variant(8, 4096, 4096) == 2
-    assert ops.skinny_variant(8, 4096, 12288) == 4 and ops.skinny_variant(3, 4096, 25600) == 0
-    assert ops.skinny_variant(16, 6144, 4096) == 2 and ops.skinny_variant(8, 151936, 1024) == 5
+    assert ops.skinny_variant(16, 1024, 3072) == 5 and ops.skinny_variant(64, 4096, 1024) == 2
+    assert ops.skinny_variant(4, 1024, 2048) == 5 and ops.skinny_variant(8, 4096, 1024) == 0
+    assert ops.skinny_variant(16, 4096, 1024) == 2 and ops.skinny_variant(8, 6144, 2048, True) == 2
+    assert ops.skinny_variant(8, 4096, 4096) == 5 and ops.skinny_variant(16, 6144, 4096) == 5
+    assert ops.skinny_variant(8, 4096, 12288) == 4 and ops.skinny_variant(3, 4096, 25600) == 5
+    assert ops.skinny_variant(8, 151936, 1024) == 5 and ops.skinny_variant(2, 151936, 1024) == 5
     assert ops.skinny_variant(8, 51200, 5120, True) == 5 and ops.skinny_variant(8, 5120, 25632) == 5
-    assert ops.skinny_variant(8, 5120, 25600) == 4 and ops.skinny_variant(16, 24576, 4096, True) == 5 and ops.skinny_variant(8, 24576, 4096, True) == 5
+    assert ops.skinny_variant(8, 5120, 25600) == 4 and ops.skinny_variant(16, 24576, 4096, True) == 5
+    assert ops.skinny_variant(1, 6144, 1024, True) == 0 and ops.skinny_variant(1, 4096, 1024) == 0
+    assert ops.skinny_variant(1, 1024, 2048) == 5 and ops.skinny_variant(1, 4096, 4096) == 5
+    assert ops.skinny_variant(3, 24576, 4096, True) == 5 and ops.skinny_variant(3, 6144, 2048, True) == 0
+    assert ops.skinny_variant(8, 1024, 2000) == 2 and ops.skinny_variant(2, 1024, 2000) == 0
+    assert ops.skinny_variant(20, 1024, 1024) == 2 and ops.skinny_variant(4, 1024, 1000) == 0
     assert ops.skinny_variant(64, 2 * 1026, 4096, True) == 2 and ops.skinny_variant(64, 2 * 1028, 4096, True) == 1
     for p in ops.TUNE_ROWS:
       ops.set_product_choice(p, 4096, 4096, False, p > 8)
