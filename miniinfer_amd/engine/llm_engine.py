@@ -75,20 +75,22 @@ class LLMEngine:
       fill_random(self.model, random_weights_seed)
     else:
       load_weights(self.model, cfg.model_path)
-    # the timed choices between own and library product kernels are process-wide and keyed by shape: an engine
-    # starts from none, so that it never inherits what an earlier engine in the process measured
-    ops.clear_product_choices()
-    if cfg.tune_products and self.dtype == torch.bfloat16:
-      try:
-        tune_products(self.model.products())
-      except (RuntimeError, torch.cuda.OutOfMemoryError) as e:      # the rule stands in for the measurement
-        warnings.warn(f"timing the product kernels failed ({e}); they are chosen by rule")
     spec = self.model.spec
     self.max_model_len = min(cfg.max_model_len or spec.max_positions, spec.max_positions)
     needs = self.model.cache_needs()
     self.num_pages = cfg.num_pages if cfg.num_pages is not None else self._pages_from_memory(needs)
     self.cache = CacheManager(needs, page_size=cfg.page_size, num_pages=self.num_pages, max_requests=cfg.max_num_seqs,
                               max_model_len=self.max_model_len, dtype=self.dtype, device=self.device)
+    # the timed choices between own and library product kernels are process-wide and keyed by shape: an engine
+    # starts from none, so that it never inherits what an earlier engine in the process measured.  They are timed
+    # after the cache pools exist: where the pools come to lie in memory must not depend on what the timing
+    # allocated and gave back (decode attention over 48 requests' pages ran 11% slower in pools allocated after it).
+    ops.clear_product_choices()
+    if cfg.tune_products and self.dtype == torch.bfloat16:
+      try:
+        tune_products(self.model.products())
+      except (RuntimeError, torch.cuda.OutOfMemoryError) as e:      # the rule stands in for the measurement
+        warnings.warn(f"timing the product kernels failed ({e}); they are chosen by rule")
     self.runner = ModelRunner(self.model, self.cache, use_graphs=not cfg.enforce_eager)
     eos = cfg.eos if cfg.eos is not None else self._eos_of_folder(cfg.model_path)
     if eos is None:

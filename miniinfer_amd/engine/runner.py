@@ -160,20 +160,29 @@ class _DecodeGraph:
     ctx.future_tokens = runner.future_tokens
     self.ctx = ctx
     # every entry is padding while warming up and capturing: it reads and writes the scratch page only
-    before = ops.library_products_run()
+    before, off_rule = ops.library_products_run(), ops.off_rule_products_run()
     self.graph, self.logits = self._capture(runner, ctx)
     self.ok = True
     after = ops.library_products_run()
     library, avoidable = after[0] != before[0], after[1] != before[1]
+    # Which kernel runs a product was measured on each product alone (or follows a rule).  Inside a step that can
+    # still lose: to this library's own kernels, which need no norm and activation kernels beside them, where a
+    # product went to the library; or to the rule's choices, where the measurement chose otherwise (at 48 requests
+    # of the Qwen3-8B shape by 4% of the step).  Such a step is captured those ways too and the quickest graph kept.
+    others = []
     if avoidable:
-      # The step sends some products of few rows to the library (by measurement of each product alone, or by
-      # rule).  Inside a step that can still lose to this library's own kernels, which need no norm and activation
-      # kernels beside them: the step is captured both ways and the quicker graph is kept.
       with ops.own_products_only():
-        own_graph, own_logits = self._capture(runner, ctx)
-      if self._replay_ms(own_graph) <= self._replay_ms(self.graph):
-        self.graph, self.logits = own_graph, own_logits
-        library = (after[0] - before[0]) > (after[1] - before[1])     # library products that were not avoidable
+        others.append(self._capture(runner, ctx) + ((after[0] - before[0]) > (after[1] - before[1]),))
+    if ops.off_rule_products_run() != off_rule:
+      mark = ops.library_products_run()
+      with ops.rule_products_only():
+        others.append(self._capture(runner, ctx) + (ops.library_products_run()[0] != mark[0],))
+    if others:
+      best = self._replay_ms(self.graph)
+      for graph, logits, uses_library in others:
+        ms = self._replay_ms(graph)
+        if ms <= best:
+          best, self.graph, self.logits, library = ms, graph, logits, uses_library
     if library and runner.check_graphs:
       # What a library records into a graph is its own affair (clears of a workspace have replayed wrongly): the
       # graph is replayed a few times, with eager work in between, against the eager result of the same (padding)

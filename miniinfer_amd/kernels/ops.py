@@ -347,10 +347,11 @@ BOTH_STAGED_MIN_K = 2048             # or with rows of at least this many column
 _PRODUCT_CHOICE: Dict[tuple, int] = {}
 KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
 KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)
+KSPLIT_OVER_LIBRARY_K = 16384        # and for large matrices too, instead of the library, when the rows are this long
 STAGED_MIN_ROWS = 4                  # without a measurement: the left operand is staged from this many rows
 STAGED_MIN_ELEMENTS = 12 << 10       # and this many elements (4 rows of 3,072 columns, 8 of 1,536)
 LINES_MIN_ELEMENTS = 40 << 20        # without a measurement: the weights come in whole lines for matrices of this size
-LINES_MIN_K = 5120                   # with rows of at least this many columns (a multiple of 64)
+LINES_MIN_K = 16384                  # with rows of at least this many columns (a multiple of 64)
 
 
 def set_product_choice(rows_point: int, matrix_rows: int, k: int, gate_up: bool, choice) -> None:
@@ -397,6 +398,27 @@ class own_products_only:
     return False
 
 
+_RULE_ONLY = [False]
+_OFF_RULE = [0]
+
+
+class rule_products_only:
+  """While active, measurements are set aside: every product of few rows goes where the rule sends it."""
+
+  def __enter__(self):
+    self.was, _RULE_ONLY[0] = _RULE_ONLY[0], True
+    return self
+
+  def __exit__(self, *exc):
+    _RULE_ONLY[0] = self.was
+    return False
+
+
+def off_rule_products_run() -> int:
+  """How many products have so far been sent, by measurement, elsewhere than the rule would have sent them."""
+  return _OFF_RULE[0]
+
+
 def library_products_run() -> Tuple[int, int]:
   """(all, avoidable): how many products have gone to the library so far, and how many of them this library's
   weight-streaming kernel could have run instead (`linear` counts them with `note_library_product`)."""
@@ -421,13 +443,16 @@ def skinny_preferred(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fa
   if _OWN_ONLY[0]:
     return True
   c = _measured_choice(num_rows, matrix_rows, k, gate_up)
+  rule = rule_choice(num_rows, matrix_rows, k, gate_up)
   if c is not None:
+    if c != rule:
+      _OFF_RULE[0] += 1
     return c != LIBRARY
-  return rule_choice(num_rows, matrix_rows, k, gate_up) != LIBRARY
+  return rule != LIBRARY
 
 
 def _measured_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> Optional[int]:
-  if _PRODUCT_CHOICE:
+  if _PRODUCT_CHOICE and not _RULE_ONLY[0]:
     for p in TUNE_ROWS:
       if p >= num_rows:
         return _PRODUCT_CHOICE.get((p, matrix_rows, k, bool(gate_up)))
@@ -478,6 +503,11 @@ def rule_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) 
   """What runs a product of up to SKINNY_MAX_ROWS rows when nothing has been measured: LIBRARY, or an OWN_... kernel."""
   if num_rows <= SKINNY_OWN_ROWS or matrix_rows * k < SKINNY_OWN_ELEMENTS:
     return _rule_variant(num_rows, matrix_rows, k, gate_up) + 1
+  # more than 16 rows of a large matrix: the library, but for very long rows (its kernels split k too little for
+  # them: [5120, 25600] at 64 rows 168 us against 81 with k split here; at 12,288 columns and 32 rows the library
+  # is still the quicker one inside a step)
+  if k >= KSPLIT_OVER_LIBRARY_K and not (gate_up and (matrix_rows // 2) % 4):
+    return OWN_KSPLIT
   return LIBRARY
 
 

@@ -30,9 +30,11 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     assert ops.skinny_preferred(64, 1024, 3072)                       # a small matrix
     assert not ops.skinny_preferred(17, 4096, 4096)                   # a large one with more than 16 rows
     assert not ops.skinny_preferred(65, 64, 64)                       # more rows than the kernel takes
+    assert ops.rule_choice(64, 5120, 25600) == ops.OWN_KSPLIT and ops.rule_choice(32, 4096, 12288) == ops.LIBRARY
+    assert ops.rule_choice(32, 6144, 4096) == ops.LIBRARY and ops.rule_choice(64, 24576, 4096, True) == ops.LIBRARY
     # which of the own kernels: k is split for more than 16 rows of 2,048 columns and more, and never for a
     # gate|up matrix whose halves are no multiple of 4 rows; from 4 rows up the weights come in whole lines, with the
-    # left operand staged, when the matrix has 40 M elements in rows of 5,120 or more (a multiple of 64; not gate|up);
+    # left operand staged, when the matrix has 40 M elements in rows of 16,384 or more (a multiple of 64; not gate|up);
     # else up to 16 rows have both operands staged through LDS (k a multiple of 32) when the matrix has 16 M
     # elements, or rows of 2,048 columns and no activation behind it; what is left has the left operand staged from
     # 4 rows and 12 K elements
@@ -41,7 +43,7 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     assert ops.skinny_variant(4, 1024, 2048) == 5 and ops.skinny_variant(8, 4096, 1024) == 0
     assert ops.skinny_variant(16, 4096, 1024) == 2 and ops.skinny_variant(8, 6144, 2048, True) == 2
     assert ops.skinny_variant(8, 4096, 4096) == 5 and ops.skinny_variant(16, 6144, 4096) == 5
-    assert ops.skinny_variant(8, 4096, 12288) == 4 and ops.skinny_variant(3, 4096, 25600) == 5
+    assert ops.skinny_variant(8, 4096, 12288) == 5 and ops.skinny_variant(32, 5120, 25600) == 1 and ops.skinny_variant(3, 4096, 25600) == 5
     assert ops.skinny_variant(8, 151936, 1024) == 5 and ops.skinny_variant(2, 151936, 1024) == 5
     assert ops.skinny_variant(8, 51200, 5120, True) == 5 and ops.skinny_variant(8, 5120, 25632) == 5
     assert ops.skinny_variant(8, 5120, 25600) == 4 and ops.skinny_variant(16, 24576, 4096, True) == 5
@@ -68,6 +70,13 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
       assert ops.skinny_preferred(3, 4096, 4096) and ops.skinny_preferred(40, 51200, 5120)
       assert not ops.skinny_preferred(65, 4096, 4096)
     assert not ops.skinny_preferred(3, 4096, 4096)
+    # measurements can be set aside, and products that they send elsewhere than the rule would are counted
+    count = ops.off_rule_products_run()
+    assert not ops.skinny_preferred(3, 4096, 4096) and ops.off_rule_products_run() == count + 1
+    with ops.rule_products_only():
+      assert ops.skinny_preferred(3, 4096, 4096) and ops.skinny_variant(12, 4096, 4096) == 5
+      assert ops.off_rule_products_run() == count + 1
+    assert ops.skinny_variant(12, 4096, 4096) == 4
     assert ops.product_choice_known(4096, 4096, False) and not ops.product_choice_known(4096, 4096, True)
   finally:
     ops.clear_product_choices()
