@@ -2,10 +2,10 @@
 // and the output head, whose time is the time to stream W once from HBM.
 //
 // The product is computed transposed on the matrix cores, C^T[n, m] = W[n, :] . A[m, :], so that the
-// 16 rows of an MFMA block are weight rows: each lane reads 16 contiguous bytes of a weight row straight
-// from global memory into its operand slot (no LDS staging), and the few rows of A (which stay in L2)
-// fill the other operand.  A workgroup owns 16 * RB weight rows; its waves split K and add their partial
-// blocks through LDS.  32-bit accumulation; the result is stored as bfloat16 or float32.
+// 16 rows of an MFMA block are weight rows: each lane's operand slot holds 16 contiguous bytes of a weight row,
+// read straight from global memory or (see the modes below) written into LDS by loads of whole memory lines, and
+// the few rows of A (which stay in L2) fill the other operand.  A workgroup owns 16 * RB weight rows; its waves
+// split K and add their partial blocks through LDS.  32-bit accumulation; the result is stored as bfloat16 or float32.
 // A second form, further down, splits K across workgroups instead (for 17 to 64 rows of A, where reading all of A
 // in every workgroup is what the first form's time grows with); mi_gemm_skinny_v takes either.
 //
@@ -51,7 +51,7 @@ struct NormHalves {
   float* ss_out;            // [gridDim.x][SS_ROW(M)]
 };
 
-// MODE 0 takes every shape.  MODES 1 to 4 are the same product for K a multiple of 32 and operands below 4 GB: the
+// MODE 0 takes every shape.  MODES 1 to 5 are the same product for K a multiple of 32 and operands below 4 GB: the
 // wave's number is made a scalar (its k range and every test on it then cost scalar instructions), addresses are a
 // scalar base plus one 32-bit lane offset plus a constant, no load is masked (lanes of rows past the end read a live
 // row again; their results are dropped at the end as before), and a wave's first weight loads go out before the
@@ -63,7 +63,8 @@ struct NormHalves {
 // LDS (global_load_lds: lane i's 16 bytes land at base + 16 i), and takes the operands from there.  The staging
 // pieces lie where the sums are added later.
 // MODES 3 and 4 (K a multiple of 64): the weights come in whole memory lines too, two steps of k per pair of loads
-// (see the loop).  Modes 1 and 2 add the same products in the same order, and so do 3 and 4.
+// (see the loop).  MODE 5 (up to 16 rows of A): both operands come through LDS (see its block).  Modes 1, 2 and 5
+// add the same products in the same order, and so do 3 and 4.
 template <int MB, int RB, bool OUT_F32, bool GATE_UP, int MODE>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __restrict__ A, int64_t lda,
                                                            const uint16_t* __restrict__ W, int64_t ldw,
