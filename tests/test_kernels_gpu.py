@@ -125,8 +125,22 @@ def _rope_ref(x, pos, theta, rotary_dim):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T", [11, 75])
-@pytest.mark.parametrize("nq,nkv,d,rd,P", [(6, 3, 48, 48, 16), (4, 4, 128, 128, 8), (5, 1, 16, 16, 4), (2, 2, 80, 32, 16)])
+@pytest.mark.parametrize("nq,nkv,d,rd,P", [(6, 3, 48, 48, 16), (4, 4, 128, 128, 8), (5, 1, 16, 16, 4), (2, 2, 80, 32, 16),
+                                           (3, 1, 72, 72, 8), (2, 1, 256, 256, 16), (7, 1, 32, 32, 16)])
 def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P, T):
+  _check_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P, T, 0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("offset", [1, 4, 8])
+def test_qk_norm_rope_cache_of_a_view(dtype, offset):
+  """The many-token kernel reads 4 elements a lane, which it can where the projection lies on a multiple of as many
+  bytes, and leaves anything else to the kernel that reads single elements: a projection that starts 1, 4 or 8
+  elements into a wider buffer."""
+  _check_qk_norm_rope_cache(dtype, 4, 2, 64, 64, 16, 75, offset)
+
+
+def _check_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P, T, offset):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(4)
   pages, max_pos, theta, eps = 12 + 2 * T // P, 300, 12345.0, 1e-5
@@ -136,11 +150,15 @@ def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P, T):
   pos = torch.randint(0, max_pos, (T,), generator=g)
   slots = torch.randperm(pages * P, generator=g)[:T] + P   # never page 0
   if T > 32:
-    # like a prompt's portion: runs of consecutive slots (one starts in the middle of a page), then scattered ones
-    slots[:29] = torch.arange(29) + 3 * P + 5
-    slots[29:50] = torch.arange(21) + ((3 * P + 5 + 29) // P + 2) * P
-    rest = [x for x in range(P, (pages + 1) * P) if x not in set(slots[:50].tolist())]
-    slots[50:] = torch.tensor(rest)[torch.randperm(len(rest), generator=g)[:T - 50]]
+    # like a prompt's portion: runs of consecutive slots (16 tokens that fill slots from a multiple of 16 on, a run
+    # that starts in the middle of a page, one that starts with a page but not with a block of 16 tokens), then
+    # scattered ones
+    slots[:16] = torch.arange(16) + 3 * P
+    second = ((3 * P + 16) // P + 2) * P + 5
+    slots[16:45] = torch.arange(29) + second
+    slots[45:66] = torch.arange(21) + ((second + 29) // P + 2) * P
+    rest = [x for x in range(P, (pages + 1) * P) if x not in set(slots[:66].tolist())]
+    slots[66:] = torch.tensor(rest)[torch.randperm(len(rest), generator=g)[:T - 66]]
   assert len(set(slots.tolist())) == T
   j = torch.arange(0, rd, 2, dtype=torch.float32)
   ang = torch.outer(torch.arange(max_pos, dtype=torch.float32), 1.0 / theta ** (j / rd))
@@ -152,7 +170,9 @@ def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P, T):
   kn = torch.nn.functional.rms_norm(k, (d,), kw, eps)
   q_want, k_want = _rope_ref(qn, pos, theta, rd), _rope_ref(kn, pos, theta, rd)
 
-  dq = qkv.to(DEV)
+  wide = torch.zeros(T, qkv.shape[1] + 16, dtype=dtype, device=DEV)
+  dq = wide[:, offset:offset + qkv.shape[1]]
+  dq.copy_(qkv)
   kp = torch.zeros(pages + 1, nkv, P, d, dtype=dtype, device=DEV)
   vp = torch.zeros(pages + 1, nkv, d, P, dtype=dtype, device=DEV)   # value pages are stored transposed
   ops.qk_norm_rope_cache(dq, nq, nkv, d, qw.to(DEV), kw.to(DEV), eps, table.to(DEV), pos.to(torch.int32).to(DEV),
@@ -168,6 +188,7 @@ def test_qk_norm_rope_cache(dtype, nq, nkv, d, rd, P, T):
     assert torch.equal(vc[page, :, off], v[t])
   # nothing else was written
   assert int((kc.abs().sum(-1) > 0).sum()) == T * nkv
+  assert not wide[:, :offset].any() and not wide[:, offset + qkv.shape[1]:].any()
 
 
 def _attention_ref(q, k, v, scale, window):
