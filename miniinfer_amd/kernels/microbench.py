@@ -3,13 +3,15 @@
     python -m miniinfer_amd.kernels.microbench product --rows 8 --n 25600 --k 5120 --gate-up
     python -m miniinfer_amd.kernels.microbench prefill-attention --tokens 2048 --heads 16 --kv-heads 8 --head-dim 128
     python -m miniinfer_amd.kernels.microbench decode-attention --batch 8 --context 2048 --heads 16 --kv-heads 8
+    python -m miniinfer_amd.kernels.microbench prompt-front --tokens 2048
     python -m miniinfer_amd.kernels.microbench choices --preset qwen3-8b
 
 `product` times the weight-streaming product (`ops.gemm_skinny`) beside the library's product for the same operands;
 the weights cycle through several copies so that they stream from memory, not from a cache.  `prefill-attention`
 times `ops.attn_prefill` for one prompt in both of its variants; `decode-attention` times the split-key decode
 kernel and its merge for a batch of requests, with and without the fused norm, rotation and cache write, over
-several caches in turn; `choices` builds a preset's model with random weights and prints what an engine measures
+several caches in turn; `prompt-front` times what precedes attention for a prompt's portion (head norms, rotation,
+both cache writes: `ops.qk_norm_rope_cache`) beside a plain read and write of the same projection; `choices` builds a preset's model with random weights and prints what an engine measures
 at its start: the time of the own and of the library kernel for each of the model's products at 1 to 64 rows.
 All print one line per measurement; under
 `rocprofv3 --pmc ...` the same commands give the kernels' counters.
@@ -149,6 +151,43 @@ def cmd_decode_attention(args) -> int:
   return 0
 
 
+def cmd_prompt_front(args) -> int:
+  """What precedes attention for a prompt's portion: head norms, rotation, and both cache writes, one launch."""
+  nq, nkv, d, P, T = args.heads, args.kv_heads, args.head_dim, args.page_size, args.tokens
+  g = torch.Generator(device=DEV).manual_seed(0)
+  copies = max(2, min(8, (1024 << 20) // max(1, T * (nq + 2 * nkv) * d * 2 * 2)))
+  pages = -(-T // P) + 1
+  qkvs = [torch.randn(T, (nq + 2 * nkv) * d, device=DEV, generator=g).bfloat16() for _ in range(copies)]
+  kps = [torch.zeros(pages + 1, nkv, P, d, device=DEV, dtype=torch.bfloat16) for _ in range(copies)]
+  vps = [torch.zeros(pages + 1, nkv, d, P, device=DEV, dtype=torch.bfloat16) for _ in range(copies)]
+  weight = torch.ones(d, device=DEV)
+  angles = torch.rand(T, d // 2, device=DEV, generator=g)
+  cos_sin = torch.cat([angles.cos(), angles.sin()], dim=1).contiguous()
+  positions = torch.arange(T, device=DEV, dtype=torch.int32)
+  slots = torch.arange(T, device=DEV, dtype=torch.int32) + P         # a prompt's tokens fill pages one after the other
+  turn = [0]
+
+  def front():
+    i = turn[0] % copies
+    turn[0] += 1
+    ops.qk_norm_rope_cache(qkvs[i], nq, nkv, d, weight, weight, 1e-6, cos_sin, positions, kps[i], vps[i], slots, P)
+
+  def scale():
+    i = turn[0] % copies
+    turn[0] += 1
+    qkvs[i].mul_(1.0)
+
+  calls = copies * max(1, args.calls // copies)
+  moved = T * ((nq + nkv) * d * 2 * 2 + nkv * d * 2 * 3)      # q, k read and written in place; k, v into the cache; v read
+  t = graph_time_us(front, calls)
+  print(f"qk_norm_rope_cache: {T} tokens, {nq}/{nkv} heads of {d}, pages of {P}: {t:.1f} us, "
+        f"{moved / 1e6:.1f} MB moved, {moved / t / 1e6:.2f} TB/s")
+  t = graph_time_us(scale, calls)
+  print(f"for comparison, x *= 1 over the same projection (torch): {t:.1f} us, "
+        f"{T * (nq + 2 * nkv) * d * 4 / t / 1e6:.2f} TB/s")
+  return 0
+
+
 def cmd_choices(args) -> int:
   from ..config import model_spec_of
   from ..presets import preset
@@ -193,6 +232,14 @@ def main(argv=None) -> int:
   d.add_argument("--copies", type=int, default=0,
                  help="caches the calls cycle through, as a model's layers do (default: 2 to 8, 1.5 GB at most)")
   d.set_defaults(fn=cmd_decode_attention)
+  f = sub.add_parser("prompt-front", help="head norms, rotation and cache writes of a prompt's portion")
+  f.add_argument("--tokens", type=int, default=2048)
+  f.add_argument("--heads", type=int, default=16)
+  f.add_argument("--kv-heads", type=int, default=8)
+  f.add_argument("--head-dim", type=int, default=128)
+  f.add_argument("--page-size", type=int, default=16)
+  f.add_argument("--calls", type=int, default=24)
+  f.set_defaults(fn=cmd_prompt_front)
   c = sub.add_parser("choices", help="own against library kernel for each product of a preset's model")
   c.add_argument("--preset", default="qwen3-0.6b")
   c.add_argument("--num-hidden-layers", type=int, default=None)

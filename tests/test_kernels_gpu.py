@@ -611,7 +611,10 @@ def test_microbench_commands_run_at_small_sizes(capsys):
                           "--calls", "2"]) == 0
   assert microbench.main(["decode-attention", "--batch", "3", "--context", "300", "--heads", "4", "--kv-heads", "2",
                           "--head-dim", "64", "--calls", "4"]) == 0
+  assert microbench.main(["prompt-front", "--tokens", "100", "--heads", "4", "--kv-heads", "2", "--head-dim", "64",
+                          "--calls", "4"]) == 0
   out = capsys.readouterr().out
+  assert "qk_norm_rope_cache: 100 tokens" in out
   assert out.count("gemm_skinny:") == 2 and out.count("gemm_skinny with k split:") == 2
   assert out.count("gemm_skinny with the left operand staged and the weights in whole lines:") == 2
   assert out.count("gemm_skinny with both operands staged:") == 2
