@@ -703,6 +703,30 @@ static SkinnyGrid skinny_grid(bool gate_up, int N, int M) {
   return g;
 }
 
+// Waves per workgroup: enough to fill the chip (where one would do, four: a launch of thousands of workgroups then
+// ends in smaller pieces; the output head takes 263 instead of 288 us); at least 2 steps of K per wave, at most 16.
+static int skinny_waves(int groups, int steps, int RB, int MB, bool gate_up) {
+  int waves = (4096 + groups - 1) / groups;
+  if (waves < 2) waves = 4;
+  if (waves > 16) waves = 16;
+  if (waves > steps / 2) waves = steps / 2;
+  if (waves < 1) waves = 1;
+  while (skinny_lds_bytes(waves, RB, MB, gate_up) > 64 * 1024 && waves > 1) waves /= 2;   // the default LDS allotment
+  return waves;
+}
+
+constexpr size_t SKINNY_LDS_ROOM = 160 * 1024;      // what a workgroup may be given (launch_instance asks for it)
+
+// The form that stages both operands keeps a wave's pieces of both in LDS: with two row blocks 16 waves' pieces are
+// more than a compute unit has, and a few waves fewer still stream faster than 16 in another form (the 8B shape's
+// [6144, 4096] at 16 rows: 14.9 -> 12.8 us; [5120, 8192] at 8 rows: 21.3 -> 18.5).  Returns 0 if even 8 do not fit.
+// (Fewer waves cut k into other slices: the sums are then no longer those of the other forms bit for bit.)
+static int both_staged_waves(int waves, int RB, int MB, bool gate_up, int M) {
+  if (MB != 1) return 0;
+  while (waves > 8 && skinny_lds_bytes(waves, RB, MB, gate_up, 2, M) > SKINNY_LDS_ROOM) --waves;
+  return skinny_lds_bytes(waves, RB, MB, gate_up, 2, M) > SKINNY_LDS_ROOM ? 0 : waves;
+}
+
 template <int MB, int RB, bool F32, bool GU, int MODE>
 static void launch_instance(dim3 grid, dim3 block, size_t lds, hipStream_t stream, const void* A, int64_t lda,
                             const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K, int rpg,
@@ -723,7 +747,6 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
                   int64_t ldc, int M, int N, int K, int waves, const SkinnyGrid& sg, const NormHalves& nh,
                   int want, hipStream_t stream) {
   const dim3 grid(sg.groups);
-  const dim3 block(64 * waves);
   const int64_t w_rows = gate_up ? 2 * (int64_t)N : N;
   const bool lean = K % 32 == 0 && w_rows * ldw * 2 < ((int64_t)1 << 32) && (int64_t)M * lda * 2 < ((int64_t)1 << 32) &&
                     (((uintptr_t)A | (uintptr_t)W) & 15) == 0;
@@ -731,11 +754,16 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
   int mode = 0;
   if (lean) {
     mode = want < 1 ? 1 : want;
-    const size_t room = 144 * 1024;
-    if (mode == 5 && (MB != 1 || skinny_lds_bytes(waves, RB, MB, gate_up, 2, M) > room)) mode = 2;
+    const size_t room = SKINNY_LDS_ROOM;
+    if (mode == 5) {
+      const int nw = both_staged_waves(waves, RB, MB, gate_up, M);
+      if (nw == 0) mode = 2;
+      else waves = nw;
+    }
     if ((mode == 3 || mode == 4) && K % 64 != 0) mode -= 2;
     if ((mode == 2 || mode == 4) && skinny_lds_bytes(waves, RB, MB, gate_up, 1) > room) mode -= 1;
   }
+  const dim3 block(64 * waves);
   const size_t lds = skinny_lds_bytes(waves, RB, MB, gate_up, mode == 5 ? 2 : (mode == 2 || mode == 4) ? 1 : 0, M);
 #define GO(F32, GU)                                                                                                  \
   {                                                                                                                  \
@@ -759,6 +787,20 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
   }
 #undef GO
   return 0;
+}
+
+// Waves per workgroup of the launch (variant as in mi_gemm_skinny_v, the kernel that owns whole rows; operands taken
+// to be aligned): forms with the same number add the same products in the same order.
+MI_EXPORT int mi_gemm_skinny_waves(int variant, int gate_up, int M, int N, int K) {
+  if (M < 1 || M > 64 || N < 1 || K < 1) return 0;
+  const SkinnyGrid sg = skinny_grid(gate_up != 0, N, M);
+  const int MB = (M + 15) / 16;
+  const int waves = skinny_waves(sg.groups, (K + 31) / 32, sg.RB, MB, gate_up != 0);
+  if (variant == 5 && K % 32 == 0) {
+    const int nw = both_staged_waves(waves, sg.RB, MB, gate_up != 0, M);
+    if (nw) return nw;
+  }
+  return waves;
 }
 
 // Workgroups of the launch for M rows and an [N, K] matrix: `ss_out` holds that many rows of mi_gemm_skinny_ss_row(M).
@@ -785,16 +827,8 @@ static int skinny_rows(int out_f32, int gate_up, const void* A, int64_t lda, con
   const SkinnyGrid sg = skinny_grid(gate_up != 0, N, M);
   const int RB = sg.RB, groups = sg.groups;
   const int steps = (K + 31) / 32;
-  // enough waves to fill the chip (where one would do, four: a launch of thousands of workgroups then ends in
-  // smaller pieces; the output head takes 263 instead of 288 us); at least 2 steps of K per wave, at most 16 waves
-  // per workgroup
-  int waves = (4096 + groups - 1) / groups;
-  if (waves < 2) waves = 4;
-  if (waves > 16) waves = 16;
-  if (waves > steps / 2) waves = steps / 2;
-  if (waves < 1) waves = 1;
   const int MB = (M + 15) / 16;
-  while (skinny_lds_bytes(waves, RB, MB, gate_up != 0) > 64 * 1024 && waves > 1) waves /= 2;   // the default LDS allotment
+  const int waves = skinny_waves(groups, steps, RB, MB, gate_up != 0);
   const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \

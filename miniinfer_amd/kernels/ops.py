@@ -118,6 +118,7 @@ _SIGS["gemm_skinny"]["mi_gemm_skinny_v"] = [c_int, c_int, c_int, c_void_p, c_int
                                             c_void_p, c_void_p, c_int64, c_void_p]
 _SIGS["gemm_skinny"]["mi_gemm_skinny_plan"] = [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]
 _SIGS["gemm_skinny"]["mi_gemm_skinny_ss_row"] = [c_int]
+_SIGS["gemm_skinny"]["mi_gemm_skinny_waves"] = [c_int, c_int, c_int, c_int, c_int]
 _SIGS["gemm_skinny"]["mi_norm_gemm_skinny"] = [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                                c_void_p, c_int64, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]
 
@@ -585,6 +586,13 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bo
   _skinny_call(lib, variant, out.dtype == torch.float32, gate_up, a, w, _ptr(out), out.stride(0) if M > 1 else N,
                M, N, K)
   return out
+
+
+def gemm_skinny_waves(variant: int, num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> int:
+  """Waves per workgroup of `gemm_skinny` in a form that owns whole rows of the result (variant 0, 2 to 5); the waves
+  share out k, so forms with the same number add the same products in the same order."""
+  n = matrix_rows // 2 if gate_up else matrix_rows
+  return int(_lib("gemm_skinny").mi_gemm_skinny_waves(variant, 1 if gate_up else 0, num_rows, n, k))
 
 
 def gemm_skinny_scaled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_ss: torch.Tensor, eps: float,

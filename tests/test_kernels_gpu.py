@@ -403,9 +403,15 @@ def test_gemm_skinny(M, N, K, out_dtype, variant):
   else:
     torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2)
   if variant in (2, 4, 5):      # the staged operands change where the operands come from, not one sum
+    other = {2: 0, 4: 3, 5: 0}[variant]
     same = torch.empty_like(out)
-    ops.gemm_skinny(a, w, same, variant={2: 0, 4: 3, 5: 0}[variant])
-    assert torch.equal(out, same)
+    ops.gemm_skinny(a, w, same, variant=other)
+    # (with two row blocks, 16 waves' pieces of both operands do not fit a unit's LDS: that form then runs fewer
+    # waves, which cut k into other slices)
+    if ops.gemm_skinny_waves(variant, M, N, K) == ops.gemm_skinny_waves(other, M, N, K):
+      assert torch.equal(out, same)
+    else:
+      assert variant == 5 and (M, N, K) == (16, 5120, 2560)
 
 
 def test_gemm_skinny_drawn_shapes():
@@ -437,7 +443,10 @@ def test_gemm_skinny_drawn_shapes():
       torch.testing.assert_close(out.double(), want, rtol=2e-4, atol=2e-4 * K ** 0.5,
                                  msg=lambda m: f"variant {variant}, {M} x [{N}, {K}] gate_up={gate_up}: {m}")
       outs[variant] = out
-    assert torch.equal(outs[2], outs[0]) and torch.equal(outs[5], outs[0]) and torch.equal(outs[4], outs[3]), (M, N, K)
+    assert torch.equal(outs[2], outs[0]) and torch.equal(outs[4], outs[3]), (M, N, K)
+    rows_w = 2 * N if gate_up else N
+    if ops.gemm_skinny_waves(5, M, rows_w, K, gate_up) == ops.gemm_skinny_waves(0, M, rows_w, K, gate_up):
+      assert torch.equal(outs[5], outs[0]), (M, N, K)
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
