@@ -264,6 +264,51 @@ __global__ void silu_mul4_kernel(const T* __restrict__ gu, T* __restrict__ out, 
   }
 }
 
+// The same for a product whose operand was an RMS norm's first half (bfloat16(residual * weight), with the sums of
+// squares of each row left in parts: see gemm_skinny.hip, NormHalves): the norm's missing factor,
+// rsqrt(sum_p row_ss[p][m] / K + eps), scales row m of gate and up before the activation.  Grid (column blocks, M).
+template <typename T>
+__global__ void silu_mul_scaled_kernel(const T* __restrict__ gu, T* __restrict__ out, int I,
+                                       const float* __restrict__ row_ss, int ss_parts, int ss_row, float eps, int K) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.y;
+  float part = 0.f;
+  for (int p = threadIdx.x; p < ss_parts; p += blockDim.x) part += row_ss[(int64_t)p * ss_row + m];
+  const float rstd = rsqrtf(block_sum(part, scratch) / (float)K + eps);
+  const int q = I / 4;
+  for (int c4 = blockIdx.x * blockDim.x + threadIdx.x; c4 < q; c4 += gridDim.x * blockDim.x) {
+    const int c = 4 * c4;
+    float g[4], u[4], r[4];
+    load4(gu + (int64_t)m * 2 * I + c, g);
+    load4(gu + (int64_t)m * 2 * I + I + c, u);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float gs = g[j] * rstd;
+      r[j] = gs / (1.f + expf(-gs)) * (u[j] * rstd);
+    }
+    store4(out + (int64_t)m * I + c, r);
+  }
+}
+
+MI_EXPORT int mi_silu_mul_scaled(int dtype, const void* gu, void* out, int M, int I, const float* row_ss, int ss_parts,
+                                 int ss_row, float eps, int K, hipStream_t stream) {
+  MI_REQUIRE(M >= 0 && M <= 65535 && I > 0 && I % 4 == 0, "silu_mul_scaled: M=%d I=%d (I must be a multiple of 4)", M, I);
+  MI_REQUIRE(row_ss && ss_parts > 0 && ss_row >= M && K > 0, "silu_mul_scaled: parts=%d rows per part=%d K=%d", ss_parts,
+             ss_row, K);
+  if (M == 0) return 0;
+  const dim3 grid((I / 4 + 255) / 256, M);
+  if (dtype == MI_DTYPE_F32)
+    silu_mul_scaled_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, I, row_ss, ss_parts, ss_row,
+                                                            eps, K);
+  else if (dtype == MI_DTYPE_BF16)
+    silu_mul_scaled_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, I, row_ss, ss_parts, ss_row, eps,
+                                                           K);
+  else
+    MI_FAIL("silu_mul_scaled: unknown dtype %d", dtype);
+  MI_CHECK_LAUNCH("silu_mul_scaled");
+  return 0;
+}
+
 MI_EXPORT int mi_silu_mul(int dtype, const void* gu, void* out, int M, int I, hipStream_t stream) {
   MI_REQUIRE(M >= 0 && I > 0, "silu_mul: bad sizes M=%d I=%d", M, I);
   if (M == 0) return 0;

@@ -77,6 +77,7 @@ _SIGS = {
     "mi_add_rmsnorm": [c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int,
                        c_void_p],
     "mi_silu_mul": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "mi_silu_mul_scaled": [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
     "mi_add_bias": [c_int, c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p],
     "mi_qk_norm_rope_cache": [c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float,
                               c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
@@ -274,6 +275,24 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     raise KernelError(f"silu_mul: gate_up {tuple(gate_up.shape)} and out {tuple(out.shape)} do not fit")
   lib = _lib("elementwise")
   _check(lib, lib.mi_silu_mul(dtype_code(gate_up.dtype), _ptr(gate_up), _ptr(out), M, I2 // 2, _stream()))
+  return out
+
+
+def silu_mul_scaled(gate_up: torch.Tensor, out: torch.Tensor, row_ss: torch.Tensor, eps: float, k: int) -> torch.Tensor:
+  """`silu_mul` of a product whose left operand was the first half of an RMS norm (`gemm_skinny_into_norm`): row m of
+  gate and up is first scaled by rsqrt(sum_p row_ss[p, m] / k + eps), the norm's missing factor (k: the length of
+  the normed rows).  row_ss float32 [parts, rows per part]; the columns I a multiple of 4."""
+  _dev(gate_up, out, row_ss)
+  _contig("gate_up", gate_up)
+  _contig("out", out)
+  M, I2 = gate_up.shape
+  if I2 % 8 or out.shape != (M, I2 // 2) or out.dtype != gate_up.dtype:
+    raise KernelError(f"silu_mul_scaled: gate_up {tuple(gate_up.shape)} and out {tuple(out.shape)} do not fit")
+  if row_ss.dtype != torch.float32 or row_ss.dim() != 2 or row_ss.shape[1] < M or not row_ss.is_contiguous():
+    raise KernelError(f"silu_mul_scaled: row_ss must be a contiguous float32 [parts, >= {M}]")
+  lib = _lib("elementwise")
+  _check(lib, lib.mi_silu_mul_scaled(dtype_code(gate_up.dtype), _ptr(gate_up), _ptr(out), M, I2 // 2, _ptr(row_ss),
+                                     row_ss.shape[0], row_ss.shape[1], float(eps), int(k), _stream()))
   return out
 
 

@@ -51,13 +51,38 @@ def as_tensor(x) -> Optional[torch.Tensor]:
   return x.materialize() if isinstance(x, PendingLinear) else x
 
 
+def _fuse_norm_around_library(d, weight: torch.Tensor) -> Optional[torch.Tensor]:
+  """The gated activation of a deferred norm's product when the gate|up product itself goes to the library (more
+  than 16 rows of a large matrix): the norm still needs no kernel if the branch's last product is pending and runs in
+  this library's kernel, which adds to the residual stream and leaves bfloat16(residual * norm weight) and the rows'
+  sums of squares; the library multiplies that operand, and the activation kernel, which follows anyway, scales
+  each row by the norm's missing factor first."""
+  M = d.residual.shape[0]
+  p = d.x
+  inter = weight.shape[0] // 2
+  if not (isinstance(p, PendingLinear) and p.value is None and p.bias is None and M <= ops.SKINNY_MAX_ROWS
+          and inter % 4 == 0 and weight.dtype == torch.bfloat16 and weight.shape[1] == d.residual.shape[1]
+          and weight.is_contiguous()):
+    return None
+  if not (ops.skinny_preferred(M, p.weight.shape[0], p.weight.shape[1])
+          and ops.gemm_skinny_into_norm_supported(p.a, p.weight, d.residual, d.norm.weight)):
+    return None
+  operand, row_ss = ops.gemm_skinny_into_norm(p.a, p.weight, d.residual, d.norm.weight)
+  ops.note_library_product(True)
+  gu = torch.matmul(operand, weight.t())
+  act = torch.empty((M, inter), dtype=torch.bfloat16, device=d.device)
+  ops.silu_mul_scaled(gu, act, row_ss, d.norm.eps, weight.shape[1])
+  d.fused(d.residual)
+  return act
+
+
 def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]:
   """The product of a deferred norm with `weight` without a kernel for the norm, when the shapes allow it."""
   M = d.residual.shape[0]
   if d.consumed or d.dtype != torch.bfloat16:
     return None
   if not ops.skinny_preferred(M, weight.shape[0], weight.shape[1], gate_up):
-    return None
+    return _fuse_norm_around_library(d, weight) if gate_up else None
   N = weight.shape[0] // 2 if gate_up else weight.shape[0]
   if isinstance(d.x, PendingLinear) and d.x.value is None and d.x.bias is not None:
     d.x = d.x.materialize()              # a product with a bias is finished by its own kernels

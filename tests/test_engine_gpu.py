@@ -265,8 +265,9 @@ def test_cache_is_sized_from_device_memory_when_no_page_count_is_given(tmp_path)
     LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=8, gpu_memory_utilization=1e-3)
 
 
-@pytest.mark.parametrize("products", ["own", "own_ksplit", "own_staged", "own_staged_lines", "own_both_staged", "library"])
-def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, products):
+@pytest.mark.parametrize("products", ["own", "own_ksplit", "own_staged", "own_staged_lines", "own_both_staged", "library",
+                                      "library_gate_up"])
+def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, products, monkeypatch):
   """The engine's choice between its own weight-streaming products (whole rows per workgroup, with or without the
   left operand staged through LDS and the weights fetched in whole lines, or k split across workgroups) and the library's is a matter of speed: with every
   small product forced to one of them, each generated token is one the plain implementation all but ties for."""
@@ -277,22 +278,29 @@ def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, produ
   with LLMEngine(model=str(tmp_path / "m"), dtype="bfloat16", page_size=8, num_pages=64, max_num_seqs=4,
                  tune_products=False, max_num_batched_tokens=48) as eng:
     before = ops.library_products_run()[0]
+    scaled_activations = []
+    real = ops.silu_mul_scaled
+    monkeypatch.setattr(ops, "silu_mul_scaled", lambda *a, **k: (scaled_activations.append(1), real(*a, **k))[1])
     if products == "own":
       with ops.own_products_only():
         outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
     else:
       choice = {"own_ksplit": ops.OWN_KSPLIT, "own_staged": ops.OWN_ROWS_STAGED,
                 "own_staged_lines": ops.OWN_ROWS_STAGED_LINES, "own_both_staged": ops.OWN_ROWS_BOTH_STAGED,
-                "library": ops.LIBRARY}[products]
+                "library": ops.LIBRARY, "library_gate_up": ops.LIBRARY}[products]
       for rows in ops.TUNE_ROWS:
         for m in eng.model.products():
-          ops.set_product_choice(rows, m[0].shape[0], m[0].shape[1], m[1], choice)
+          # (library_gate_up: only the gate|up product goes to the library; the product before it keeps the norm's
+          # first half in its ending, and the activation kernel applies the norm's row factor)
+          mine = choice if products != "library_gate_up" or m[1] else ops.OWN_ROWS
+          ops.set_product_choice(rows, m[0].shape[0], m[0].shape[1], m[1], mine)
       try:
         outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
       finally:
         ops.clear_product_choices()
     ran_library = ops.library_products_run()[0] - before
-    assert (ran_library > 0) == (products == "library")
+    assert (ran_library > 0) == (products in ("library", "library_gate_up"))
+    assert (len(scaled_activations) > 0) == (products == "library_gate_up")
   for p, o in zip(prompts, outs):
     hist = list(p)
     for tok in o["token_ids"]:

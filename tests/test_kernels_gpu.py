@@ -635,3 +635,21 @@ def test_measured_peaks_are_plausible():
   gbs, tflops = ops.measured_peaks(stream_bytes=1 << 28)
   assert 500 < gbs < 8000 and 100 < tflops < 2500, (gbs, tflops)
   assert ops.measured_peaks() == (gbs, tflops)      # measured once per process and device
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,parts,ss_row", [(5, 112, 3, 16), (40, 1028, 256, 64), (64, 36, 1, 64), (1, 4096, 17, 16)])
+def test_silu_mul_scaled(dtype, M, I, parts, ss_row):
+  """The activation kernel that also applies an RMS norm's missing row factor, from the rows' partial sums of
+  squares, against the statement in 64-bit."""
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(M + I)
+  gu = torch.randn(M, 2 * I, generator=g).to(dtype)
+  row_ss = torch.rand(parts, ss_row, generator=g) * 50
+  eps, K = 1e-5, 96
+  rstd = torch.rsqrt(row_ss.double().sum(0)[:M] / K + eps)[:, None]
+  want = torch.nn.functional.silu(gu[:, :I].double() * rstd) * (gu[:, I:].double() * rstd)
+  out = ops.silu_mul_scaled(gu.to(DEV), torch.empty(M, I, dtype=dtype, device=DEV), row_ss.to(DEV), eps, K)
+  torch.testing.assert_close(out.double().cpu(), want, **_tol(dtype))
+  with pytest.raises(ops.KernelError):
+    ops.silu_mul_scaled(gu.to(DEV), torch.empty(M, I, dtype=dtype, device=DEV), row_ss[:, :0].contiguous().to(DEV), eps, K)
