@@ -1,10 +1,12 @@
-"""Command line:  python -m miniinfer_amd <generate | random-model | throughput> ...
+"""Command line:  python -m miniinfer_amd <generate | random-model | throughput | replay | bench> ...
 
 `generate` takes the options of the reference's example (examples/minimal_engine.py:24-55: --model,
 --max-tokens, --temperature, --max-num-seqs, --max-model-len); `throughput` those of its benchmark
 (benchmark/bench_miniinfer.py:16-26: --num-seqs, --max-input-len, --max-output-len, --max-num-seqs,
 --max-model-len, --page-size, --eager) with the same workload: seeded random token ids, random lengths,
-temperature 0.6, ignore_eos, throughput = total output tokens / time after a warm-up.
+temperature 0.6, ignore_eos, throughput = total output tokens / time after a warm-up.  `replay` feeds given token
+ids through the model step by step and writes logits (the program `bin/trace_run`; `engine/replay.py`); `bench`
+measures decode and prefill throughput and prints one JSON line (the program `bench.py`; `benchmark.py`).
 """
 
 from __future__ import annotations
@@ -34,6 +36,11 @@ def _engine_args(p):
   p.add_argument("--no-tune", action="store_true",
                  help="choose the kernels of small-batch products by rule instead of timing them at start")
   p.add_argument("--seed", type=int, default=0)
+  p.add_argument("--load-format", default="safetensors", choices=["safetensors", "random"],
+                 help="random: only the folder's config.json is read, the weights are drawn on the device from --seed")
+  p.add_argument("--fixed-kernel-choices", action="store_true",
+                 help="products of few rows go where a rule sends them, never where a timing at start-up did, so that "
+                      "a run's kernels and roundings do not depend on timings")
 
 
 def _engine(args):
@@ -48,7 +55,8 @@ def _engine(args):
                    max_model_len=args.max_model_len, page_size=args.page_size, num_pages=args.num_pages,
                    max_num_batched_tokens=args.max_num_batched_tokens,
                    enable_chunked_prefill=not args.no_chunked_prefill, enforce_eager=args.eager, enable_overlap=not args.no_overlap,
-                   tune_products=not args.no_tune, seed=args.seed)
+                   tune_products=not args.no_tune, seed=args.seed, timed_kernel_choices=not args.fixed_kernel_choices,
+                   **({} if args.preset is not None else {"load_format": args.load_format}))
 
 
 def cmd_generate(args) -> int:
@@ -116,7 +124,16 @@ def cmd_throughput(args) -> int:
   return 0
 
 
+def cmd_replay(args) -> int:
+  from miniinfer_amd.engine.replay import run
+  return run(args.model, args.dtype, args.out, args.max_tokens, page_size=args.page_size)
+
+
 def main(argv=None) -> int:
+  argv = list(sys.argv[1:] if argv is None else argv)
+  if argv and argv[0] == "bench":            # the benchmark parses its own options
+    from miniinfer_amd.benchmark import main as bench_main
+    return bench_main(argv[1:])
   ap = argparse.ArgumentParser(prog="python -m miniinfer_amd")
   sub = ap.add_subparsers(dest="cmd", required=True)
 
@@ -149,6 +166,16 @@ def main(argv=None) -> int:
   t.add_argument("--max-input-len", type=int, default=1024)
   t.add_argument("--max-output-len", type=int, default=1024)
   t.set_defaults(fn=cmd_throughput, max_num_seqs=256, max_model_len=4096)
+
+  rp = sub.add_parser("replay", help="feed a trace of token ids (JSON lines on stdin) through the model, write logits")
+  rp.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+  rp.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+  rp.add_argument("--out", required=True, help="folder for <step>.f32 files")
+  rp.add_argument("--max-tokens", type=int, required=True, help="tokens the cache pool is made for")
+  rp.add_argument("--page-size", type=int, default=16)
+  rp.set_defaults(fn=cmd_replay)
+
+  sub.add_parser("bench", add_help=False, help="decode and prefill throughput as one JSON line (`bench --help`)")
 
   args = ap.parse_args(argv)
   return args.fn(args)

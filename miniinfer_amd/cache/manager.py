@@ -81,8 +81,10 @@ class PagedGroup:
   need: PagedKV
   layers: List[int]
   pool: PagePool
-  k: Optional[torch.Tensor] = None     # [len(layers), num_pages + 1, nkv, page_size, d]
-  v: Optional[torch.Tensor] = None     # [len(layers), num_pages + 1, nkv, d, page_size] (transposed pages)
+  page_size: int                       # tokens per page of this group
+  dtype: torch.dtype
+  k: Optional[torch.Tensor] = None     # [len(layers), pages + 1, nkv, page_size, d]
+  v: Optional[torch.Tensor] = None     # [len(layers), pages + 1, nkv, d, page_size] (transposed pages)
   tables: Dict[Hashable, List[int]] = field(default_factory=dict)   # per request: page id per page index, 0 = given back
 
 
@@ -98,24 +100,34 @@ class LayerCache:
   """What one layer's mixer sees of the cache."""
   kind: str                              # "paged" | "state" | "none"
   group: int = -1
-  k: Optional[torch.Tensor] = None       # [num_pages + 1, nkv, page_size, d]
-  v: Optional[torch.Tensor] = None       # [num_pages + 1, nkv, d, page_size]
+  k: Optional[torch.Tensor] = None       # [pages + 1, nkv, page_size, d]
+  v: Optional[torch.Tensor] = None       # [pages + 1, nkv, d, page_size]
   state: Optional[torch.Tensor] = None   # [max_requests + 1, *shape]; row max_requests is scratch
   page_size: int = 0
   window: Optional[int] = None
 
 
+def _check_page_size(page_size: int) -> None:
+  if page_size <= 0 or page_size & (page_size - 1):
+    raise ValueError(f"page_size must be a power of two, got {page_size}")
+
+
 class CacheManager:
   def __init__(self, layer_needs: Sequence[object], page_size: int, num_pages: int, max_requests: int,
-               max_model_len: int, dtype: torch.dtype, device, allocate: bool = True):
-    """layer_needs[i] is the PagedKV / FixedState / None of layer i."""
-    if page_size <= 0 or page_size & (page_size - 1):
-      raise ValueError(f"page_size must be a power of two, got {page_size}")
+               max_model_len: int, dtype: torch.dtype, device, allocate: bool = True,
+               max_step_tokens: Optional[int] = None):
+    """layer_needs[i] is the PagedKV / FixedState / None of layer i.
+
+    page_size, dtype: of every group that names none of its own.  num_pages: pages of `page_size` tokens, i.e. a
+    group that keeps every key has room for num_pages * page_size tokens, whatever its own page size; a group
+    with a window has at most that, and no more than its requests can hold at once (`window_pool_pages`).
+    max_step_tokens: the most new tokens one step brings (default: max_model_len); it only bounds window pools."""
+    _check_page_size(page_size)
     self.page_size = page_size
     self.num_pages = num_pages
     self.max_requests = max_requests
     self.max_model_len = max_model_len
-    self.max_pages_per_request = -(-max_model_len // page_size)
+    self.max_step_tokens = max_step_tokens if max_step_tokens is not None else max_model_len
     self.dtype = dtype
     self.device = torch.device(device)
     self.paged: List[PagedGroup] = []
@@ -130,7 +142,11 @@ class CacheManager:
             break
         else:
           gi = len(self.paged)
-          self.paged.append(PagedGroup(need=need, layers=[], pool=PagePool(num_pages)))
+          P = need.page_size or page_size
+          _check_page_size(P)
+          pages = self.group_pages(need, page_size, num_pages, max_requests, self.max_step_tokens)
+          self.paged.append(PagedGroup(need=need, layers=[], pool=PagePool(pages), page_size=P,
+                                       dtype=need.dtype or dtype))
         self._layer_map.append(("paged", gi, len(self.paged[gi].layers)))
         self.paged[gi].layers.append(i)
       elif isinstance(need, FixedState):
@@ -144,6 +160,9 @@ class CacheManager:
         self.states[si].layers.append(i)
       else:
         raise TypeError(f"layer {i}: unknown cache need {need!r}")
+    # the finest page of any group: block tables are at most this many entries wide
+    self.min_page_size = min((g.page_size for g in self.paged), default=page_size)
+    self.max_pages_per_request = -(-max_model_len // self.min_page_size)
     self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
     # The state row that no request ever gets: padding entries of captured steps read and write it, as they
     # read and write page 0 of the paged groups.
@@ -153,19 +172,51 @@ class CacheManager:
     if allocate:
       self._allocate()
 
-  # ------------------------------------------------------------------ storage
+  # ------------------------------------------------------------------ sizes
+  @staticmethod
+  def window_pool_pages(window: int, page_size: int, max_requests: int, max_step_tokens: int) -> int:
+    """Pages that `max_requests` requests of a group with a window can hold at once.  Between steps a request
+    keeps the pages that its next token can still see, at most ceil(window / P) + 1; inside a step it also holds
+    the pages of the step's new tokens, ceil(n / P) + 1 more for n of them, and a step brings at most
+    `max_step_tokens` in all."""
+    per_request = -(-window // page_size) + 3
+    return max_requests * per_request + -(-max_step_tokens // page_size)
+
+  @classmethod
+  def group_pages(cls, need: PagedKV, page_size: int, num_pages: int, max_requests: int, max_step_tokens: int) -> int:
+    """Pages (of its own size) in the pool of the group with this need."""
+    P = need.page_size or page_size
+    pages = -(-num_pages * page_size // P)
+    if need.window is not None:
+      pages = min(pages, cls.window_pool_pages(need.window, P, max_requests, max_step_tokens))
+    return max(1, pages)
+
+  @classmethod
+  def storage_bytes(cls, layer_needs: Sequence[object], page_size: int, num_pages: int, max_requests: int,
+                    max_step_tokens: int, dtype: torch.dtype) -> int:
+    """Device bytes of the page pools for `num_pages` (scratch pages included)."""
+    total = 0
+    for n in layer_needs:
+      if isinstance(n, PagedKV):
+        P = n.page_size or page_size
+        esize = torch.empty((), dtype=n.dtype or dtype).element_size()
+        pages = cls.group_pages(n, page_size, num_pages, max_requests, max_step_tokens) + 1
+        total += 2 * n.num_kv_heads * n.head_dim * P * esize * pages
+    return total
+
   @staticmethod
   def bytes_per_page(layer_needs: Sequence[object], page_size: int, dtype: torch.dtype) -> int:
-    """Device bytes that one more page in every group costs."""
-    esize = torch.empty((), dtype=dtype).element_size()
-    return sum(2 * n.num_kv_heads * n.head_dim * page_size * esize for n in layer_needs if isinstance(n, PagedKV))
+    """Device bytes that room for `page_size` more tokens costs in every layer (window pools, which are bounded,
+    counted as if they grew too)."""
+    return sum(2 * n.num_kv_heads * n.head_dim * page_size * torch.empty((), dtype=n.dtype or dtype).element_size()
+               for n in layer_needs if isinstance(n, PagedKV))
 
   def _allocate(self) -> None:
     for g in self.paged:
-      n, h, d = len(g.layers), g.need.num_kv_heads, g.need.head_dim
+      n, h, d, P = len(g.layers), g.need.num_kv_heads, g.need.head_dim, g.page_size
       # keys [.., page_size, d]; values transposed [.., d, page_size]: the MFMA kernels read runs of keys per dim
-      g.k = torch.zeros((n, self.num_pages + 1, h, self.page_size, d), dtype=self.dtype, device=self.device)
-      g.v = torch.zeros((n, self.num_pages + 1, h, d, self.page_size), dtype=self.dtype, device=self.device)
+      g.k = torch.zeros((n, g.pool.num_pages + 1, h, P, d), dtype=g.dtype, device=self.device)
+      g.v = torch.zeros((n, g.pool.num_pages + 1, h, d, P), dtype=g.dtype, device=self.device)
     for s in self.states:
       shape = (len(s.layers), self.max_requests + 1) + tuple(s.need.shape)
       s.state = torch.zeros(shape, dtype=s.need.dtype or self.dtype, device=self.device)
@@ -175,7 +226,7 @@ class CacheManager:
     if kind == "paged":
       g = self.paged[gi]
       return LayerCache(kind="paged", group=gi, k=None if g.k is None else g.k[li], v=None if g.v is None else g.v[li],
-                        page_size=self.page_size, window=g.need.window)
+                        page_size=g.page_size, window=g.need.window)
     if kind == "state":
       s = self.states[gi]
       return LayerCache(kind="state", group=gi, state=None if s.state is None else s.state[li])
@@ -189,8 +240,11 @@ class CacheManager:
     return len(self._free_slots)
 
   def num_free_pages(self) -> int:
-    """Free pages of the tightest group."""
+    """Free pages of the tightest group (in pages of that group's own size)."""
     return min((g.pool.num_free for g in self.paged), default=self.num_pages)
+
+  def all_pages_free(self) -> bool:
+    return all(g.pool.num_free == g.pool.num_pages for g in self.paged)
 
   def length(self, req) -> int:
     return self._length[req]
@@ -219,22 +273,61 @@ class CacheManager:
     if g.need.window is None:
       return 0
     lo = max(0, next_pos - g.need.window + 1)
-    return lo // self.page_size
+    return lo // g.page_size
 
-  def held_pages(self, req) -> int:
-    """Page indices `req` has been given so far (0 for a request that is not admitted)."""
-    if not self.paged or req not in self.paged[0].tables:
+  def held_pages(self, req, group: int = 0) -> int:
+    """Page indices `req` has been given so far in a group (0 for a request that is not admitted)."""
+    if group >= len(self.paged) or req not in self.paged[group].tables:
       return 0
-    return len(self.paged[0].tables[req])
+    return len(self.paged[group].tables[req])
+
+  # ---- room: what the groups can still hand out.  A scheduler takes a copy (`room`), books its plan against it
+  # (`take`) and so never plans a step that `grow` would refuse; groups differ in page size, pool size and in when
+  # pages come back, so the books are kept per group.
+  def room(self) -> List[int]:
+    """Free pages per paged group (a copy to plan against)."""
+    return [g.pool.num_free for g in self.paged]
+
+  def _needs(self, req, new_len: int) -> List[int]:
+    return [max(0, -(-new_len // g.page_size) - len(g.tables.get(req, ()))) for g in self.paged]
+
+  def fits(self, room: Sequence[int], req, new_len: int, spare: int = 0) -> bool:
+    """Whether `req` (admitted or not) can grow to `new_len` tokens out of `room`, leaving `spare` pages in every group."""
+    return all(n + spare <= r for n, r in zip(self._needs(req, new_len), room))
+
+  def take(self, room: List[int], req, new_len: int) -> bool:
+    """Books growing `req` to `new_len` tokens against `room` (in place); False, and nothing booked, if it does not fit."""
+    needs = self._needs(req, new_len)
+    if any(n > r for n, r in zip(needs, room)):
+      return False
+    for i, n in enumerate(needs):
+      room[i] -= n
+    return True
+
+  def tokens_that_fit(self, room: Sequence[int], req) -> int:
+    """The longest `req` can become out of `room`."""
+    if not self.paged:
+      return self.max_model_len
+    return min((len(g.tables.get(req, ())) + r) * g.page_size for g, r in zip(self.paged, room))
+
+  def never_fits(self, num_tokens: int) -> Optional[str]:
+    """Why a request of `num_tokens` tokens could not be held even with every page free, or None if it could."""
+    for gi, g in enumerate(self.paged):
+      if g.need.window is None:
+        need = -(-num_tokens // g.page_size)
+      else:
+        need = min(-(-num_tokens // g.page_size), -(-g.need.window // g.page_size) + 2)
+      if need > g.pool.num_pages:
+        return (f"{num_tokens} tokens need {need} pages of {g.page_size} tokens in cache group {gi}, "
+                f"which has {g.pool.num_pages}")
+    return None
 
   def pages_needed(self, req, new_len: int) -> int:
-    """Pages each group must still hand out so that `req` can hold new_len tokens."""
-    if not self.paged:
-      return 0
-    return max(0, -(-new_len // self.page_size) - self.held_pages(req))
+    """The most pages any group must still hand out so that `req` can hold new_len tokens."""
+    return max(self._needs(req, new_len), default=0)
 
   def can_grow(self, req, new_len: int) -> bool:
-    return self.pages_needed(req, new_len) <= self.num_free_pages()
+    return self.fits(self.room(), req, new_len)
 
   def grow(self, req, new_len: int) -> None:
     """Make room for tokens up to position new_len - 1 in every group (all or nothing)."""
@@ -242,17 +335,19 @@ class CacheManager:
       raise CacheError(f"request {req!r}: {new_len} tokens exceed max_model_len={self.max_model_len}")
     if new_len < self._length[req]:
       raise CacheError(f"request {req!r} cannot shrink from {self._length[req]} to {new_len}")
-    need = self.pages_needed(req, new_len)
-    if need > self.num_free_pages():
-      raise OutOfPages(f"request {req!r} needs {need} more pages, {self.num_free_pages()} are free")
-    for g in self.paged:
-      g.tables[req].extend(g.pool.alloc(need))
+    needs = self._needs(req, new_len)
+    for gi, (g, n) in enumerate(zip(self.paged, needs)):
+      if n > g.pool.num_free:
+        raise OutOfPages(f"request {req!r} needs {n} more pages in cache group {gi}, {g.pool.num_free} are free")
+    for g, n in zip(self.paged, needs):
+      g.tables[req].extend(g.pool.alloc(n))
 
   def commit(self, req, new_len: int) -> None:
     """The step that wrote tokens up to new_len - 1 is done: record the length and give back
     the pages of window groups that no later token can see."""
-    if new_len > len(self.paged[0].tables[req]) * self.page_size if self.paged else False:
-      raise CacheError(f"request {req!r}: commit of {new_len} tokens beyond its pages")
+    for g in self.paged:
+      if new_len > len(g.tables[req]) * g.page_size:
+        raise CacheError(f"request {req!r}: commit of {new_len} tokens beyond its pages")
     self._length[req] = new_len
     for g in self.paged:
       if g.need.window is None:

@@ -40,6 +40,13 @@ class EngineConfig:
   tune_products: bool = True                  # time own and library kernels for the model's large products once
   eos: Optional[int] = None                   # None: from generation_config.json, else from config.json
   seed: int = 0
+  # "safetensors": the folder's *.safetensors files, by tensor name; "random": only config.json is read and the
+  # weights are drawn on the device from `seed` (N(0, initializer_range), norm weights 1 + N(0, 0.1))
+  load_format: str = "safetensors"
+  # False: products of few rows go where the rule sends them, never where a timing at start-up did, and a captured
+  # step is recorded one way only, so that a run's kernels (and with them its bfloat16 roundings) do not depend on
+  # timings; implies what `tune_products=False` does
+  timed_kernel_choices: bool = True
   device: str = "cuda:0"
 
   def __post_init__(self):
@@ -56,6 +63,8 @@ class EngineConfig:
       raise ValueError("max_num_batched_tokens must be positive")
     if self.max_model_len is not None and self.max_model_len <= 0:
       raise ValueError("max_model_len must be positive")
+    if self.load_format not in ("safetensors", "random"):
+      raise ValueError(f"load_format must be 'safetensors' or 'random', got {self.load_format!r}")
 
   # aliases the reference keeps (config.py:63-70)
   @property

@@ -602,6 +602,22 @@ __global__ __launch_bounds__(512) void norm_gemm_kernel(const float* __restrict_
   }
 }
 
+// Compute units of the current device (256 on an MI355X); every count of workgroups or waves that is meant to fill
+// the chip is derived from it.
+static int compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+  }
+  return cus;
+}
+
+// Wave slots of the chip: 16 on each compute unit.
+static int wave_slots() { return 16 * compute_units(); }
+
 // R [*, K] float32 residual, X [*, K] bfloat16 or null, R_out [M, K] float32 or null (written when given),
 // NW [K] float32 norm weight, rows [M] or null, W [N, K] (gate_up: [2 N, K]) bfloat16, C [M, N] bfloat16.
 MI_EXPORT int mi_norm_gemm_skinny(int gate_up, const float* R, const void* X, float* R_out, const float* NW,
@@ -617,7 +633,7 @@ MI_EXPORT int mi_norm_gemm_skinny(int gate_up, const float* R, const void* X, fl
   const int RB = gate_up ? 2 : (row_blocks >= 1024 ? 2 : 1);
   const int groups = gate_up ? row_blocks : (row_blocks + RB - 1) / RB;
   const int steps = (K + 31) / 32;
-  int waves = (4096 + groups - 1) / groups;
+  int waves = (wave_slots() + groups - 1) / groups;
   if (waves > 8) waves = 8;
   if (waves > steps / 2) waves = steps / 2;
   if (waves < 1) waves = 1;
@@ -652,17 +668,6 @@ static size_t skinny_lds_bytes(int waves, int RB, int MB, bool gate_up, int stag
 struct SkinnyGrid {
   int RB, rpg, groups;
 };
-
-static int compute_units() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-      cus = 256;
-  }
-  return cus;
-}
 
 static SkinnyGrid skinny_grid(bool gate_up, int N, int M) {
   const int row_blocks = (N + 15) / 16;
@@ -706,7 +711,7 @@ static SkinnyGrid skinny_grid(bool gate_up, int N, int M) {
 // Waves per workgroup: enough to fill the chip (where one would do, four: a launch of thousands of workgroups then
 // ends in smaller pieces; the output head takes 263 instead of 288 us); at least 2 steps of K per wave, at most 16.
 static int skinny_waves(int groups, int steps, int RB, int MB, bool gate_up) {
-  int waves = (4096 + groups - 1) / groups;
+  int waves = (wave_slots() + groups - 1) / groups;
   if (waves < 2) waves = 4;
   if (waves > 16) waves = 16;
   if (waves > steps / 2) waves = steps / 2;

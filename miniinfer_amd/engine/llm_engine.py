@@ -59,10 +59,15 @@ class RequestOutput:
 
 class LLMEngine:
   def __init__(self, model: str, model_config=None, random_weights_seed: Optional[int] = None, **kwargs):
-    """model: a folder with config.json and *.safetensors.  With `model_config` (a typed configuration)
-    and `random_weights_seed`, no folder is read and the weights are drawn on the device."""
+    """model: a folder with config.json and *.safetensors.  With the option `load_format="random"` only its
+    config.json is read and the weights are drawn on the device from the option `seed`.  `model_config` (a typed
+    configuration) stands in for the folder's config.json; `random_weights_seed` is `load_format="random"` with a
+    seed of its own for the weights."""
     kwargs.pop("use_multiprocess", None)   # the reference's examples pass it; there is one process here
+    if random_weights_seed is not None:
+      kwargs["load_format"] = "random"
     self.config = EngineConfig.from_kwargs(model, **kwargs)
+    t_start = time.perf_counter()
     if not torch.cuda.is_available():
       raise RuntimeError("miniinfer_amd needs a GPU: torch.cuda.is_available() is False and there is no CPU path")
     cfg = self.config
@@ -71,8 +76,8 @@ class LLMEngine:
     torch.cuda.set_device(self.device)
     self.model_config = model_config if model_config is not None else load_model_config(cfg.model_path)
     self.model = build_model(model_spec_of(self.model_config), self.dtype, self.device)
-    if random_weights_seed is not None:
-      fill_random(self.model, random_weights_seed)
+    if cfg.load_format == "random":
+      fill_random(self.model, random_weights_seed if random_weights_seed is not None else cfg.seed)
     else:
       load_weights(self.model, cfg.model_path)
     spec = self.model.spec
@@ -80,18 +85,23 @@ class LLMEngine:
     needs = self.model.cache_needs()
     self.num_pages = cfg.num_pages if cfg.num_pages is not None else self._pages_from_memory(needs)
     self.cache = CacheManager(needs, page_size=cfg.page_size, num_pages=self.num_pages, max_requests=cfg.max_num_seqs,
-                              max_model_len=self.max_model_len, dtype=self.dtype, device=self.device)
-    # the timed choices between own and library product kernels are process-wide and keyed by shape: an engine
-    # starts from none, so that it never inherits what an earlier engine in the process measured.  They are timed
-    # after the cache pools exist: where the pools come to lie in memory must not depend on what the timing
-    # allocated and gave back (decode attention over 48 requests' pages ran 11% slower in pools allocated after it).
-    ops.clear_product_choices()
-    if cfg.tune_products and self.dtype == torch.bfloat16:
+                              max_model_len=self.max_model_len, dtype=self.dtype, device=self.device,
+                              max_step_tokens=cfg.max_num_batched_tokens)
+    # Which kernel runs a product of few rows: this engine's own table (another engine in the process has its own).
+    # The products are timed after the cache pools exist: where the pools come to lie in memory must not depend on
+    # what the timing allocated and gave back (decode attention over 48 requests' pages ran 11% slower in pools
+    # allocated after it).
+    self.choices = ops.ProductChoices(rule_only=not cfg.timed_kernel_choices)
+    if cfg.tune_products and cfg.timed_kernel_choices and self.dtype == torch.bfloat16:
       try:
-        tune_products(self.model.products())
+        with self.choices:
+          tune_products(self.model.products())
       except (RuntimeError, torch.cuda.OutOfMemoryError) as e:      # the rule stands in for the measurement
+        self.choices.clear()
+        torch.cuda.empty_cache()
         warnings.warn(f"timing the product kernels failed ({e}); they are chosen by rule")
-    self.runner = ModelRunner(self.model, self.cache, use_graphs=not cfg.enforce_eager)
+    self.runner = ModelRunner(self.model, self.cache, use_graphs=not cfg.enforce_eager, choices=self.choices,
+                              compare_captures=cfg.timed_kernel_choices)
     eos = cfg.eos if cfg.eos is not None else self._eos_of_folder(cfg.model_path)
     if eos is None:
       eos = getattr(self.model_config, "eos_token_id", None)
@@ -108,6 +118,9 @@ class LLMEngine:
     self._pending = None
     self._token_bufs = [torch.zeros(max(1, cfg.max_num_seqs), dtype=torch.int32, pin_memory=True) for _ in range(2)]
     self._token_turn = 0
+    torch.cuda.synchronize(self.device)
+    self.startup_seconds = time.perf_counter() - t_start     # weights, cache pools, timing of the product kernels
+    self.warm_up_seconds = 0.0                                # spent in `warm_up` so far
 
   # ------------------------------------------------------------------ set-up helpers
   def _pages_from_memory(self, needs) -> int:
@@ -115,36 +128,60 @@ class LLMEngine:
     `gpu_memory_utilization` leaves alone and less what the largest step needs for its activations (the reference
     holds back a fifth of the free memory for them, whatever the model: utils/memory_utils.py:85-144; here the
     step's buffers are counted from the model's sizes and the token budget).  Never more pages than
-    `max_num_seqs` requests of `max_model_len` tokens can use."""
+    `max_num_seqs` requests of `max_model_len` tokens can use.  The pools' bytes are the cache manager's own count
+    (groups differ in page size, dtype and, with a window, in how many pages they can use at all)."""
     cfg = self.config
-    per_page = CacheManager.bytes_per_page(needs, cfg.page_size, self.dtype)
     cap = cfg.max_num_seqs * (-(-self.max_model_len // cfg.page_size))
-    if per_page == 0:
+
+    def pool_bytes(pages: int) -> int:
+      return CacheManager.storage_bytes(needs, cfg.page_size, pages, cfg.max_num_seqs, cfg.max_num_batched_tokens,
+                                        self.dtype)
+
+    if pool_bytes(cap) == 0:
       return max(1, cap)
     free, total = torch.cuda.mem_get_info(self.device)
     usable = free - int(total * (1.0 - cfg.gpu_memory_utilization)) - self.activation_bytes()
-    pages = usable // per_page - 1            # page 0 of every group is the scratch page
-    if pages < 2:
+    if pool_bytes(2) > usable:
       raise RuntimeError(f"not enough device memory for a cache: {free >> 20} MiB free, the largest step needs "
-                         f"{self.activation_bytes() >> 20} MiB, a page costs {per_page} bytes")
-    return int(min(pages, cap))
+                         f"{self.activation_bytes() >> 20} MiB, two pages cost {pool_bytes(2)} bytes")
+    lo, hi = 2, cap                      # the most pages whose pools fit: the bytes grow with the pages
+    while lo < hi:
+      mid = (lo + hi + 1) // 2
+      if pool_bytes(mid) <= usable:
+        lo = mid
+      else:
+        hi = mid - 1
+    return int(lo)
 
   def activation_bytes(self) -> int:
-    """An upper estimate of the device memory one step of the full token budget holds beside weights and cache:
-    per token two 32-bit residual rows and, in the activation dtype, the widest rows a block makes (each counted
-    twice, since the allocator keeps a freed buffer of one layer while the next layer's is made), the 32-bit logits
-    of `max_num_seqs` rows with the sampler's scratch, the pools of the captured decode steps, and 256 MiB of slack."""
+    """An upper estimate of the device memory that steps hold beside weights and cache.  One step of the full token
+    budget: per token two 32-bit residual rows and, in the activation dtype, the widest rows a block makes (each
+    counted twice, since the allocator keeps a freed buffer of one layer while the next layer's is made); while the
+    product kernels are timed at start-up, that timing's buffers instead if they are larger.  The 32-bit logits of
+    `max_num_seqs` rows with the sampler's scratch.  The captured decode steps: they share one pool for what they
+    hold while they run (counted once, for the widest of them) but each keeps its own logits, so one row of logits for
+    every row of every (batch, table width) bucket that this engine's limits allow.  And 256 MiB of slack (key-range
+    partials of the attention, the k-split products' partial results, the library's workspace)."""
     cfg, spec = self.config, self.model.spec
     esize = 2 if self.dtype == torch.bfloat16 else 4
     widest = spec.hidden_size
     for _, part, ps in self.model.named_params():
+      if part is self.model:            # the frame's own tables (embedding, head, positions) are no activations
+        continue
       if len(ps.shape) == 2:
-        widest = max(widest, ps.shape[0] if ps.shape[0] != spec.vocab_size else 0)
+        widest = max(widest, ps.shape[0])
     T = cfg.max_num_batched_tokens
     per_token = 2 * 4 * spec.hidden_size + 2 * esize * (2 * widest + 2 * spec.hidden_size)
+    step = T * per_token
+    if cfg.tune_products and cfg.timed_kernel_choices and self.dtype == torch.bfloat16:
+      step = max(step, 640 << 20)       # the timing's flush buffer, operands and partial results
     logits = 3 * 4 * spec.vocab_size * min(cfg.max_num_seqs, 256)
-    graphs = 0 if cfg.enforce_eager else 256 * (per_token + 4 * spec.vocab_size)
-    return int(T * per_token + logits + graphs + (256 << 20))
+    graphs = 0
+    if not cfg.enforce_eager:
+      from .runner import graph_bucket_rows
+      rows, widths = graph_bucket_rows(cfg.max_num_seqs, self.max_model_len, cfg.page_size)
+      graphs = 256 * per_token + rows * widths * 4 * spec.vocab_size
+    return int(step + logits + graphs + (256 << 20))
 
   @staticmethod
   def _eos_of_folder(path: str):
@@ -194,6 +231,9 @@ class LLMEngine:
 
   def add_request(self, prompt: Union[str, Sequence[int]], sampling_params: Optional[SamplingParams] = None,
                   request_id: Optional[str] = None) -> str:
+    """Queues a request and returns its id.  The step that books the request's last token hands the finished
+    request out in `StepOutput.finished` (`request_id`, `outputs`, `finish_reason`); the engine keeps no
+    reference to it after that (miniinfer/engine/llm_engine.py:1309-1339)."""
     params = sampling_params or SamplingParams()
     ids = self._encode(prompt)
     V = self.model.spec.vocab_size
@@ -211,7 +251,11 @@ class LLMEngine:
   def warm_up(self, max_num_seqs: Optional[int] = None, max_tokens: Optional[int] = None) -> int:
     """Captures the decode graphs ahead of their first use (every batch bucket up to `max_num_seqs`, every table
     width up to `max_tokens` tokens a request; defaults: the engine's limits).  Returns the number of graphs."""
-    return self.runner.capture_graphs(max_num_seqs or self.config.max_num_seqs, max_tokens or self.max_model_len)
+    t0 = time.perf_counter()
+    n = self.runner.capture_graphs(max_num_seqs or self.config.max_num_seqs, max_tokens or self.max_model_len)
+    torch.cuda.synchronize(self.device)
+    self.warm_up_seconds += time.perf_counter() - t0
+    return n
 
   def is_finished(self) -> bool:
     return self._pending is None and not self.scheduler.has_unfinished()
@@ -252,7 +296,10 @@ class LLMEngine:
     if sampling:
       event.synchronize()
       sampled = {r.number: t for r, t in zip(sampling, host.tolist())}
-    out.finished += self.scheduler.resolve(plan, sampled)
+    done = self.scheduler.resolve(plan, sampled)
+    for r in done:                      # the step's output hands a finished request out; the engine lets go of it
+      self._requests.pop(r.request_id, None)
+    out.finished += done
     out.num_prefill_tokens += plan.num_prefill_tokens
     out.num_decode_tokens += plan.num_decode_tokens
     out.num_preempted += len(plan.preempted)
@@ -289,6 +336,7 @@ class LLMEngine:
     if len(sampling_params) != len(prompts):
       raise ValueError("one SamplingParams for all prompts, or one per prompt")
     rids = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+    mine = [self._requests[rid] for rid in rids]
     t0 = time.time()
     decoded = 0
     last = t0
@@ -302,8 +350,7 @@ class LLMEngine:
     if use_tqdm:
       print(file=sys.stderr)
     results = []
-    for rid in rids:
-      r = self._requests.pop(rid)
+    for rid, r in zip(rids, mine):
       text = self.tokenizer.decode(r.outputs) if self.tokenizer is not None else ""
       results.append({"text": text, "token_ids": list(r.outputs), "request_id": rid, "finish_reason": r.finish_reason})
     return results
@@ -341,4 +388,3 @@ class LLMEngine:
         sent[rid] = ready
         if done:
           del live[rid]
-          self._requests.pop(rid, None)

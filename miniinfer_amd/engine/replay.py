@@ -34,7 +34,9 @@ TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 class Replayer:
   def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, max_requests: int = 16,
-               device: str = "cuda:0"):
+               device: str = "cuda:0", choices=None):
+    """max_tokens: the tokens the page pools are made for; max_requests: request slots; choices: the runner's table
+    of product-kernel choices (default: a new one, every product by rule)."""
     if not torch.cuda.is_available():
       raise RuntimeError("miniinfer_amd needs a GPU: torch.cuda.is_available() is False and there is no CPU path")
     dt = TORCH_DTYPES[normalize_dtype(dtype)]
@@ -45,7 +47,7 @@ class Replayer:
     self.cache = CacheManager(self.model.cache_needs(), page_size=page_size, num_pages=num_pages,
                               max_requests=max_requests, max_model_len=self.model.spec.max_positions,
                               dtype=dt, device=device)
-    self.runner = ModelRunner(self.model, self.cache)
+    self.runner = ModelRunner(self.model, self.cache, choices=choices)
 
   def step(self, record: dict) -> Optional[np.ndarray]:
     entries = []

@@ -14,6 +14,7 @@ index arrays are built on the host with numpy and reach the device in one copy.
 
 from __future__ import annotations
 
+import logging
 import warnings
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
@@ -24,6 +25,8 @@ import torch
 from ..cache.manager import CacheManager, LayerCache
 from ..kernels import ops
 from ..parts import DecoderModel
+
+log = logging.getLogger("miniinfer_amd")
 
 
 @dataclass
@@ -155,8 +158,8 @@ class _DecodeGraph:
     self.dev = torch.zeros(self.layout.total, dtype=torch.int32, device=runner.device)
     self.dev.copy_(self.stage)
     ctx = self.layout.context(self.dev, cache, runner.device)
-    ctx.q_lens, ctx.kv_lens = [1] * B, [W * cache.page_size] * B   # host-side sizes the kernels are tuned for
-    ctx.num_multi, ctx.max_q_len, ctx.max_kv_len = 0, 1, W * cache.page_size
+    ctx.q_lens, ctx.kv_lens = [1] * B, [W * cache.min_page_size] * B   # host-side sizes the kernels are tuned for
+    ctx.num_multi, ctx.max_q_len, ctx.max_kv_len = 0, 1, W * cache.min_page_size
     ctx.future_tokens = runner.future_tokens
     self.ctx = ctx
     # every entry is padding while warming up and capturing: it reads and writes the scratch page only
@@ -170,19 +173,23 @@ class _DecodeGraph:
     # product went to the library; or to the rule's choices, where the measurement chose otherwise (at 48 requests
     # of the Qwen3-8B shape by 4% of the step).  Such a step is captured those ways too and the quickest graph kept.
     others = []
-    if avoidable:
+    self.kept = "as chosen"
+    if avoidable and runner.compare_captures:
       with ops.own_products_only():
-        others.append(self._capture(runner, ctx) + ((after[0] - before[0]) > (after[1] - before[1]),))
-    if ops.off_rule_products_run() != off_rule:
+        others.append(self._capture(runner, ctx) + ((after[0] - before[0]) > (after[1] - before[1]), "own kernels only"))
+    if ops.off_rule_products_run() != off_rule and runner.compare_captures:
       mark = ops.library_products_run()
       with ops.rule_products_only():
-        others.append(self._capture(runner, ctx) + (ops.library_products_run()[0] != mark[0],))
+        others.append(self._capture(runner, ctx) + (ops.library_products_run()[0] != mark[0], "by rule"))
     if others:
       best = self._replay_ms(self.graph)
-      for graph, logits, uses_library in others:
+      timings = [f"as chosen {best * 1e3:.0f} us"]
+      for graph, logits, uses_library, how in others:
         ms = self._replay_ms(graph)
+        timings.append(f"{how} {ms * 1e3:.0f} us")
         if ms <= best:
-          best, self.graph, self.logits, library = ms, graph, logits, uses_library
+          best, self.graph, self.logits, library, self.kept = ms, graph, logits, uses_library, how
+      log.info("decode graph for %d entries, tables of %d pages: %s -> kept %s", B, W, ", ".join(timings), self.kept)
     if library and runner.check_graphs:
       # What a library records into a graph is its own affair (clears of a workspace have replayed wrongly): the
       # graph is replayed a few times, with eager work in between, against the eager result of the same (padding)
@@ -215,7 +222,9 @@ class _DecodeGraph:
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    # one memory pool for all captured steps of a runner: they never run side by side, so what one holds while it
+    # runs can be another's; only each graph's logits stay its own
+    with torch.cuda.graph(graph, pool=runner.graph_pool()):
       logits = runner.model.forward(ctx)
     return graph, logits
 
@@ -260,11 +269,28 @@ class _DecodeGraph:
 _GRAPH_BATCHES = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 
 
+def graph_bucket_rows(max_requests: int, max_tokens: int, page_size: int):
+  """(rows of all batch buckets that steps of up to `max_requests` single tokens can fall into, number of
+  table-width buckets up to `max_tokens` tokens a request): what the captured decode steps of an engine with these
+  limits keep alive at most, one row of logits per bucket row and width."""
+  top = next((b for b in _GRAPH_BATCHES if b >= max_requests), _GRAPH_BATCHES[-1])
+  rows = sum(b for b in _GRAPH_BATCHES if b <= top)
+  W = max(1, -(-max_tokens // page_size))
+  widths = max(1, (max(16, 1 << (W - 1).bit_length()) // 16).bit_length())
+  return rows, widths
+
+
 class ModelRunner:
-  def __init__(self, model: DecoderModel, cache: CacheManager, use_graphs: bool = False):
+  def __init__(self, model: DecoderModel, cache: CacheManager, use_graphs: bool = False,
+               choices: Optional[ops.ProductChoices] = None, compare_captures: bool = True):
     """use_graphs: replay steps that hold only single decoded tokens (at most 256 of them) from HIP graphs,
-    captured on demand per (batch bucket, block-table width bucket)."""
+    captured on demand per (batch bucket, block-table width bucket).  choices: the table that says which kernel
+    runs a product of few rows; it is this runner's own (a new, empty one by default: every product by rule) and is
+    the current one while the runner steps.  compare_captures: a step whose products could go more than one way
+    is captured each way and the quickest graph kept; off, it is captured once, as the table says."""
     self.model = model
+    self.choices = choices if choices is not None else ops.ProductChoices()
+    self.compare_captures = compare_captures
     self.cache = cache
     self.device = model.ctx.device
     self.vocab_size = model.spec.vocab_size
@@ -279,10 +305,16 @@ class ModelRunner:
     self._staging_turn = 0
     self._allow_future = False
     self._graphs: Dict[tuple, _DecodeGraph] = {}
+    self._graph_pool = None
     # Tokens of the last step's sampling output, by row.  A token id -(r + 1) in a step's entries stands for
     # future_tokens[r] as it is when the step's embedding kernel runs: whoever samples writes here, and may
     # launch the next step before reading the tokens back.
     self.future_tokens = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=self.device)
+
+  def graph_pool(self):
+    if self._graph_pool is None:
+      self._graph_pool = torch.cuda.graph_pool_handle()
+    return self._graph_pool
 
   # ------------------------------------------------------------------ host side of a step
   def _stage(self, n: int) -> torch.Tensor:
@@ -324,10 +356,12 @@ class ModelRunner:
     q_lens = [len(entries[i].tokens) for i in order]
     starts = [cache.length(entries[i].req) for i in order]
     kv_lens = [s + n for s, n in zip(starts, q_lens)]
-    need = sum(cache.pages_needed(entries[i].req, kv) for i, kv in zip(order, kv_lens))
-    if need > cache.num_free_pages():
-      from ..cache.manager import OutOfPages
-      raise OutOfPages(f"step needs {need} new pages, {cache.num_free_pages()} are free")
+    room = cache.room()
+    for i, kv in zip(order, kv_lens):
+      if not cache.take(room, entries[i].req, kv):
+        from ..cache.manager import OutOfPages
+        raise OutOfPages(f"the step's requests need more pages than are free (request {entries[i].req!r} growing to "
+                         f"{kv} tokens; free pages per cache group: {cache.room()})")
     for i, kv in zip(order, kv_lens):
       cache.grow(entries[i].req, kv)
     return order, q_lens, starts, kv_lens
@@ -336,7 +370,6 @@ class ModelRunner:
     """Writes the step's integer arrays into `host` (views of a flat buffer laid out by `lay`).  Only the first
     len(order) entries are written; a wider layout's tail belongs to the caller."""
     cache = self.cache
-    P = cache.page_size
     B, T, G, W = len(order), sum(q_lens), lay.G, lay.W
     cu = np.zeros(B + 1, dtype=np.int64)
     np.cumsum(q_lens, out=cu[1:])
@@ -353,6 +386,7 @@ class ModelRunner:
       host["req_slots"][b] = cache.slot(entries[i].req)
       for g in range(G):
         tab = cache.table(g, entries[i].req)
+        P = cache.paged[g].page_size
         n = min(len(tab), W)
         tables[g, b, :n] = tab[:n]
         tables[g, b, n:] = 0
@@ -368,7 +402,7 @@ class ModelRunner:
     first[1:] = np.cumsum(q_lens)[:-1]
     first_row = {i: int(first[b]) for b, i in enumerate(order)}
     rows = [first_row[i] + w for i, e in enumerate(entries) for w in e.want]
-    W = max(1, max(-(-kv // cache.page_size) for kv in kv_lens))
+    W = max(1, max(-(-kv // cache.min_page_size) for kv in kv_lens))
     lay = _Layout(T=T, B=B, R=len(rows), G=len(cache.paged), W=W)
     spare = 2 * (T // 4 + B + 1)           # room for a list of (entry, block of >= 4 query tokens)
     stage = self._stage(lay.total + spare)
@@ -396,16 +430,17 @@ class ModelRunner:
     device, in the order of the entries and of each entry's `want`.  With `allow_future`, a token id -(r + 1)
     is taken from `future_tokens[r]` on the device."""
     self._allow_future = allow_future
-    if self.use_graphs and len(entries) <= _GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries):
-      return self._step_from_graph(entries)
-    return self._step_eager(entries)
+    with self.choices:
+      if self.use_graphs and len(entries) <= _GRAPH_BATCHES[-1] and all(len(e.tokens) == 1 for e in entries):
+        return self._step_from_graph(entries)
+      return self._step_eager(entries)
 
   def graph_buckets(self, num_requests: int, num_tokens: int):
     """(batch bucket, block-table width bucket) of the graph that a step of `num_requests` single tokens replays
     when the longest of them holds `num_tokens` tokens."""
     cache = self.cache
     Bb = next(b for b in _GRAPH_BATCHES if b >= num_requests)
-    W = max(1, -(-num_tokens // cache.page_size))
+    W = max(1, -(-num_tokens // cache.min_page_size))
     Wb = max(16, 1 << (W - 1).bit_length())
     return Bb, min(Wb, max(cache.max_pages_per_request, W))
 
@@ -416,15 +451,16 @@ class ModelRunner:
     miniinfer/engine/llm_engine.py:281-313).  Returns how many graphs there are."""
     if not self.use_graphs:
       return 0
+    P = self.cache.min_page_size
     widths = sorted({self.graph_buckets(1, n)[1] for n in
-                     [self.cache.page_size * (16 << i) for i in range(32) if self.cache.page_size * (16 << i) < max_tokens]
-                     + [max_tokens]})
-    for b in _GRAPH_BATCHES:
-      if b > max(1, max_requests) and b != self.graph_buckets(max(1, max_requests), 1)[0]:
-        continue
-      for w in widths:
-        if (b, w) not in self._graphs:
-          self._graphs[(b, w)] = _DecodeGraph(self, b, w)
+                     [P * (16 << i) for i in range(32) if P * (16 << i) < max_tokens] + [max_tokens]})
+    with self.choices:
+      for b in _GRAPH_BATCHES:
+        if b > max(1, max_requests) and b != self.graph_buckets(max(1, max_requests), 1)[0]:
+          continue
+        for w in widths:
+          if (b, w) not in self._graphs:
+            self._graphs[(b, w)] = _DecodeGraph(self, b, w)
     return len(self._graphs)
 
   def _step_eager(self, entries: Sequence[StepEntry]) -> torch.Tensor:

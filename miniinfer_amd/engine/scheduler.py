@@ -150,10 +150,9 @@ class Scheduler:
       # the reference never checks this and would index past its table (kvcache/memory_pool.py:476-478)
       raise ValueError(f"prompt of {n} tokens plus max_tokens={req.params.max_tokens} exceeds "
                        f"max_model_len={self.max_model_len}")
-    P = self.cache.page_size
-    if -(-(n + req.params.max_tokens) // P) > self.cache.num_pages:
-      raise ValueError(f"request of up to {n + req.params.max_tokens} tokens can never fit the cache of "
-                       f"{self.cache.num_pages} pages of {P} tokens")
+    why = self.cache.never_fits(n + req.params.max_tokens)
+    if why is not None:
+      raise ValueError(f"request of up to {n + req.params.max_tokens} tokens can never fit the cache: {why}")
     if not self.enable_chunked_prefill and n + req.params.max_tokens > self.max_num_batched_tokens:
       raise ValueError(f"without chunked prefill a request of up to {n + req.params.max_tokens} tokens must fit the "
                        f"step budget of {self.max_num_batched_tokens}")
@@ -163,9 +162,6 @@ class Scheduler:
     return bool(self.waiting or self.running or self.num_unresolved)
 
   # ------------------------------------------------------------------ one step's plan
-  def _pages_for(self, req: Request, new_len: int) -> int:
-    return self.cache.pages_needed(req.number, new_len)
-
   def _preempt(self, req: Request) -> None:
     self.cache.release(req.number)
     self.running.remove(req)
@@ -178,37 +174,37 @@ class Scheduler:
     if not (self.waiting or self.running):
       return None
     budget = self.max_num_batched_tokens
-    free = self.cache.num_free_pages()
+    cache = self.cache
+    room = cache.room()            # free pages per cache group; the plan is booked against this copy
     entries: List[ScheduledEntry] = []
     preempted: List[Request] = []
 
+    def all_fit(reqs) -> bool:
+      trial = list(room)
+      return all(cache.take(trial, r.number, r.num_tokens) for r in reqs)
+
     # 1. decodes: one token for every running request whose known tokens are all but one in the cache
     decoding = [r for r in self.running if r.remaining == 1 and r.num_computed > 0]
-    while True:
-      need = sum(self._pages_for(r, r.num_tokens) for r in decoding)
-      if need <= free or not decoding:
-        break
+    while decoding and not all_fit(decoding):
       if self._draining:
         # Finished requests hold pages until their last token is written in, one call from now.  The decodes
         # that need a new page sit this step out (the most recently admitted first) rather than cost a running
         # request its whole cache.
-        short = need - free
         for r in reversed(list(decoding)):
-          if short <= 0:
+          if all_fit(decoding):
             break
-          n = self._pages_for(r, r.num_tokens)
-          if n > 0:
+          if cache.pages_needed(r.number, r.num_tokens) > 0:
             decoding.remove(r)
-            short -= n
         break
       victim = self.running[-1]
       self._preempt(victim)
       preempted.append(victim)
       decoding = [r for r in decoding if r is not victim]
-      free = self.cache.num_free_pages()
+      room = cache.room()
     for r in decoding[:budget]:
+      if not cache.take(room, r.number, r.num_tokens):
+        continue
       entries.append(ScheduledEntry(r, r.num_computed, 1, True))
-      free -= self._pages_for(r, r.num_tokens)
       budget -= 1
     scheduled = {id(e.request) for e in entries}
 
@@ -218,29 +214,27 @@ class Scheduler:
         break
       if id(r) in scheduled or r.remaining <= 0 or (r.remaining == 1 and r.num_computed > 0):
         continue
-      n = self._portion(r, budget, free)
-      if n <= 0:
+      n = self._portion(r, budget, room)
+      if n <= 0 or not cache.take(room, r.number, r.num_computed + n):
         continue
       entries.append(ScheduledEntry(r, r.num_computed, n, r.num_computed + n == r.num_tokens))
-      free -= self._pages_for(r, r.num_computed + n)
       budget -= n
 
     # 3. admissions, in arrival order; none while a request had to be preempted in this step
     while self.waiting and budget > 0 and not preempted and len(self.running) < self.max_num_seqs \
-        and self.cache.num_free_slots() > 0:
+        and cache.num_free_slots() > 0:
       r = self.waiting[0]
       # watermark: its whole known sequence must fit, with one spare page for each request already running,
       # so that an admission does not at once force a preemption
-      if self._pages_for(r, r.num_tokens) + len(self.running) > free:
+      if not cache.fits(room, r.number, r.num_tokens, spare=len(self.running)):
         break
-      n = self._portion(r, budget, free)
-      if n <= 0:
+      n = self._portion(r, budget, room)
+      if n <= 0 or not cache.take(room, r.number, n):
         break
       self.waiting.popleft()
-      self.cache.admit(r.number)
+      cache.admit(r.number)
       self.running.append(r)
       entries.append(ScheduledEntry(r, 0, n, n == r.num_tokens))
-      free -= self._pages_for(r, n)
       budget -= n
 
     if not entries:
@@ -256,11 +250,10 @@ class Scheduler:
       return None
     return ScheduledStep(entries, preempted)
 
-  def _portion(self, r: Request, budget: int, free_pages: int) -> int:
+  def _portion(self, r: Request, budget: int, room) -> int:
     """How many of r's remaining tokens run in this step: bounded by the budget and by the tokens that fit
-    the pages r holds plus the free ones.  Without chunked prefill it is all of them or none."""
-    P = self.cache.page_size
-    capacity = (self.cache.held_pages(r.number) + free_pages) * P
+    the pages r holds plus what `room` still has.  Without chunked prefill it is all of them or none."""
+    capacity = self.cache.tokens_that_fit(room, r.number)
     n = min(r.remaining, budget, capacity - r.num_computed)
     if not self.enable_chunked_prefill and n < r.remaining:
       return 0

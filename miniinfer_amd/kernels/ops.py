@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_int64, c_void_p
-from typing import Dict, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
@@ -364,7 +364,6 @@ LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_
 BOTH_STAGED_MAX_ROWS = 16
 BOTH_STAGED_ANY_ELEMENTS = 16 << 20  # without a measurement: both operands are staged for matrices of this size,
 BOTH_STAGED_MIN_K = 2048             # or with rows of at least this many columns where no activation follows
-_PRODUCT_CHOICE: Dict[tuple, int] = {}
 KSPLIT_MIN_ROWS = 17                 # without a measurement: k is split for more than 16 rows
 KSPLIT_MIN_K = 2048                  # of at least this many columns (the left operand is then 64 KB and more)
 KSPLIT_OVER_LIBRARY_K = 16384        # and for large matrices too, instead of the library, when the rows are this long
@@ -374,17 +373,95 @@ LINES_MIN_ELEMENTS = 40 << 20        # without a measurement: the weights come i
 LINES_MIN_K = 16384                  # with rows of at least this many columns (a multiple of 64)
 
 
+class ProductChoices:
+  """Where products of few rows go: a table of timed choices, keyed by (rows point, matrix rows, k, gate|up), over a
+  rule, with switches that set the table aside.  An engine owns one and makes it the current one around its steps
+  (`with choices:`), so two engines in a process never share timings; code that runs outside any engine (tests,
+  tools) uses the module's default table, which starts empty, i.e. by rule.
+
+  force: None, or LIBRARY / an OWN_... constant that every product goes to which can (for tests and measurements);
+  rule_only: the table is never consulted; own_only: nothing goes to the library."""
+
+  def __init__(self, rule_only: bool = False):
+    self.table: Dict[tuple, int] = {}
+    self.rule_only = bool(rule_only)
+    self.own_only = False
+    self.force: Optional[int] = None
+    self.library_products = [0, 0]     # (all, avoidable) products that went to the library
+    self.off_rule = 0                  # products sent, by measurement, elsewhere than the rule would have
+    self._outer: List["ProductChoices"] = []
+
+  def __enter__(self):
+    self._outer.append(_CURRENT[0])
+    _CURRENT[0] = self
+    return self
+
+  def __exit__(self, *exc):
+    _CURRENT[0] = self._outer.pop()
+    return False
+
+  def set(self, rows_point: int, matrix_rows: int, k: int, gate_up: bool, choice) -> None:
+    self.table[(rows_point, matrix_rows, k, bool(gate_up))] = int(choice)
+
+  def known(self, matrix_rows: int, k: int, gate_up: bool) -> bool:
+    return all((p, matrix_rows, k, bool(gate_up)) in self.table for p in TUNE_ROWS)
+
+  def clear(self) -> None:
+    self.table.clear()
+
+  def measured(self, num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> Optional[int]:
+    if self.force is not None:
+      can_split = not (gate_up and (matrix_rows // 2) % 4)
+      if self.force == OWN_KSPLIT and not can_split:
+        return OWN_ROWS
+      if self.force == OWN_ROWS_BOTH_STAGED and not (num_rows <= BOTH_STAGED_MAX_ROWS and k % 32 == 0):
+        return OWN_ROWS
+      if self.force in (OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES) and k % 64:
+        return OWN_ROWS
+      return self.force
+    if self.table and not self.rule_only:
+      for p in TUNE_ROWS:
+        if p >= num_rows:
+          return self.table.get((p, matrix_rows, k, bool(gate_up)))
+    return None
+
+
+_DEFAULT_CHOICES = ProductChoices()
+_CURRENT: List[ProductChoices] = [_DEFAULT_CHOICES]
+
+
+def current_choices() -> ProductChoices:
+  return _CURRENT[0]
+
+
 def set_product_choice(rows_point: int, matrix_rows: int, k: int, gate_up: bool, choice) -> None:
-  """choice: LIBRARY or one of the OWN_... constants (False and True stand for LIBRARY and OWN_ROWS)."""
-  _PRODUCT_CHOICE[(rows_point, matrix_rows, k, bool(gate_up))] = int(choice)
+  """In the current table.  choice: LIBRARY or one of the OWN_... constants (False and True stand for LIBRARY and
+  OWN_ROWS)."""
+  _CURRENT[0].set(rows_point, matrix_rows, k, gate_up, choice)
 
 
 def product_choice_known(matrix_rows: int, k: int, gate_up: bool) -> bool:
-  return all((p, matrix_rows, k, bool(gate_up)) in _PRODUCT_CHOICE for p in TUNE_ROWS)
+  return _CURRENT[0].known(matrix_rows, k, gate_up)
 
 
 def clear_product_choices() -> None:
-  _PRODUCT_CHOICE.clear()
+  _CURRENT[0].clear()
+
+
+_COMPUTE_UNITS: Dict[int, int] = {}
+
+
+def compute_units(device=None) -> int:
+  """Compute units of the device (256 on an MI355X, which is also what is assumed where there is no GPU to ask, as in
+  host-only tests of the launch rules).  The launch rules derive from it how many workgroups or waves fill the chip."""
+  if not torch.cuda.is_available():
+    return 256
+  index = torch.device(device).index if device is not None else None
+  if index is None:
+    index = torch.cuda.current_device()
+  if index not in _COMPUTE_UNITS:
+    _COMPUTE_UNITS[index] = int(torch.cuda.get_device_properties(index).multi_processor_count) or 256
+  return _COMPUTE_UNITS[index]
 
 
 _SIDE_STREAMS: Dict[int, "torch.cuda.Stream"] = {}
@@ -402,53 +479,49 @@ def side_stream(device=None) -> "torch.cuda.Stream":
   return _SIDE_STREAMS[index]
 
 
-_OWN_ONLY = [False]
-_LIBRARY_PRODUCTS = [0, 0]
-
-
 class own_products_only:
   """While active, `skinny_preferred` sends every product of up to SKINNY_MAX_ROWS rows to this library's kernel."""
 
   def __enter__(self):
-    self.was, _OWN_ONLY[0] = _OWN_ONLY[0], True
+    self.table = _CURRENT[0]
+    self.was, self.table.own_only = self.table.own_only, True
     return self
 
   def __exit__(self, *exc):
-    _OWN_ONLY[0] = self.was
+    self.table.own_only = self.was
     return False
-
-
-_RULE_ONLY = [False]
-_OFF_RULE = [0]
 
 
 class rule_products_only:
   """While active, measurements are set aside: every product of few rows goes where the rule sends it."""
 
   def __enter__(self):
-    self.was, _RULE_ONLY[0] = _RULE_ONLY[0], True
+    self.table = _CURRENT[0]
+    self.was, self.table.rule_only = self.table.rule_only, True
     return self
 
   def __exit__(self, *exc):
-    _RULE_ONLY[0] = self.was
+    self.table.rule_only = self.was
     return False
 
 
 def off_rule_products_run() -> int:
   """How many products have so far been sent, by measurement, elsewhere than the rule would have sent them."""
-  return _OFF_RULE[0]
+  return _CURRENT[0].off_rule
 
 
 def library_products_run() -> Tuple[int, int]:
   """(all, avoidable): how many products have gone to the library so far, and how many of them this library's
   weight-streaming kernel could have run instead (`linear` counts them with `note_library_product`)."""
-  return _LIBRARY_PRODUCTS[0], _LIBRARY_PRODUCTS[1]
+  c = _CURRENT[0]
+  return c.library_products[0], c.library_products[1]
 
 
 def note_library_product(avoidable: bool = False) -> None:
-  _LIBRARY_PRODUCTS[0] += 1
+  c = _CURRENT[0]
+  c.library_products[0] += 1
   if avoidable:
-    _LIBRARY_PRODUCTS[1] += 1
+    c.library_products[1] += 1
 
 
 def skinny_preferred(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> bool:
@@ -460,23 +533,20 @@ def skinny_preferred(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fa
   outweighs the norm and activation kernels that fusing saved."""
   if num_rows > SKINNY_MAX_ROWS:
     return False
-  if _OWN_ONLY[0]:
+  cur = _CURRENT[0]
+  if cur.own_only:
     return True
-  c = _measured_choice(num_rows, matrix_rows, k, gate_up)
+  c = cur.measured(num_rows, matrix_rows, k, gate_up)
   rule = rule_choice(num_rows, matrix_rows, k, gate_up)
   if c is not None:
     if c != rule:
-      _OFF_RULE[0] += 1
+      cur.off_rule += 1
     return c != LIBRARY
   return rule != LIBRARY
 
 
 def _measured_choice(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> Optional[int]:
-  if _PRODUCT_CHOICE and not _RULE_ONLY[0]:
-    for p in TUNE_ROWS:
-      if p >= num_rows:
-        return _PRODUCT_CHOICE.get((p, matrix_rows, k, bool(gate_up)))
-  return None
+  return _CURRENT[0].measured(num_rows, matrix_rows, k, gate_up)
 
 
 def skinny_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> int:
@@ -804,7 +874,7 @@ def attn_prefill_tokens_per_block(nq: int, nkv: int, d: int, wide: bool = False)
   return lib.mi_attn_prefill_tokens_per_block_wide(nq, nkv) if wide else lib.mi_attn_prefill_tokens_per_block(nq, nkv)
 
 
-PREFILL_WIDE_MIN_WORKGROUPS = 1024     # from here on (four for every compute unit) the "wide" prefill variant pays
+PREFILL_WIDE_WORKGROUPS_PER_UNIT = 4   # from this many workgroups for every compute unit on, the "wide" prefill variant pays
 
 
 def attn_prefill_wide_pays(q_lens, nq: int, nkv: int, d: int) -> int:
@@ -814,7 +884,7 @@ def attn_prefill_wide_pays(q_lens, nq: int, nkv: int, d: int) -> int:
   if tpb <= 0:
     return 0
   items = sum(-(-n // tpb) for n in q_lens if n > 1)
-  return tpb if items * nkv >= PREFILL_WIDE_MIN_WORKGROUPS else 0
+  return tpb if items * nkv >= PREFILL_WIDE_WORKGROUPS_PER_UNIT * compute_units() else 0
 
 
 def attn_decode_geometry(d: int):
@@ -970,5 +1040,6 @@ def measured_peaks(device=None, stream_bytes: int = 1 << 31) -> Tuple[float, flo
     ms = best_ms(lambda: _check(lib, lib.mi_probe_mfma(cus * 8, 4096, _ptr(sink), ctypes.byref(flops), _stream())), 3)
     tflops = flops.value / ms / 1e9
   del buf
+  torch.cuda.empty_cache()      # the read buffer goes back to the driver: a cache sized from free memory must see it
   _MEASURED_PEAKS[index] = (gbs, tflops)
   return _MEASURED_PEAKS[index]

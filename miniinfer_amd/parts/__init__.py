@@ -3,4 +3,4 @@ from .base import (BLOCKS, FEED_FORWARDS, FRAMES, MIXERS, NORMS, POSITIONS, Buil
                    register_position)
 from . import norm, position, attention, mlp, block   # registers the built-in kinds
 from .model import DecoderModel
-from .norm import DeferredNorm
+from .norm import DeferredNorm, Norm

@@ -34,6 +34,10 @@ class PagedAttention(Part):
     self.position = POSITIONS.build(spec.position, ctx)
     self.q_norm = NORMS.build(spec.qk_norm, ctx) if spec.qk_norm is not None else None
     self.k_norm = NORMS.build(spec.qk_norm, ctx) if spec.qk_norm is not None else None
+    # The attention kernels norm the heads themselves, restating a weight-only RMS norm from `weight` and `eps`.
+    # A head norm of another kind (one that does not say `fusable_rms`) is evaluated by its own `forward` on the
+    # heads as rows [tokens * heads, head_dim], and the kernels are then given no norm to do.
+    self.heads_norm_fused = self.q_norm is None or bool(getattr(self.q_norm, "fusable_rms", False))
     self.shares_kv = bool(getattr(spec, "shares_kv", False))
     self.qkv_weight: Optional[torch.Tensor] = None   # q rows only when the keys and values are borrowed
     self.o_weight: Optional[torch.Tensor] = None
@@ -82,33 +86,47 @@ class PagedAttention(Part):
     T = x.shape[0]
     qkv = linear(x, self.qkv_weight, bias=self.qkv_bias)
     table = self.position.rotary_table()
-    eps = self.q_norm.eps if self.q_norm is not None else 0.0
-    if ctx.num_multi == 0 and not self.shares_kv and (table is None or table.shape[1] == self.d) and \
+    q_weight = k_weight = None
+    eps = 0.0
+    if self.q_norm is not None and self.heads_norm_fused:
+      q_weight, eps = self.q_norm.weight, self.q_norm.eps
+      k_weight = self.k_norm.weight if not self.shares_kv else None
+    elif self.q_norm is not None:
+      self._norm_heads(qkv)
+    if ctx.num_multi == 0 and self.heads_norm_fused and not self.shares_kv and (table is None or table.shape[1] == self.d) and \
         ops.mfma_attention_supported(qkv.dtype, self.nq, self.nkv, self.d, cache.page_size):
       # a step of decoded tokens only: the attention kernel norms, rotates and caches by itself
       out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
-      self._attend_decode(qkv, out, ctx, cache, 0, ctx.num_requests, front=(table, eps))
+      self._attend_decode(qkv, out, ctx, cache, 0, ctx.num_requests, front=(table, eps, q_weight, k_weight))
       return PendingLinear(out, self.o_weight, self.o_bias)
     if self.shares_kv:
       # only queries of its own: they are normed and rotated; the borrowed pages are read, never written
-      ops.qk_norm_rope_cache(qkv, self.nq, 0, self.d, self.q_norm.weight if self.q_norm is not None else None, None,
-                             eps, table, ctx.positions, None, None, None, cache.page_size)
+      ops.qk_norm_rope_cache(qkv, self.nq, 0, self.d, q_weight, None, eps, table, ctx.positions, None, None, None,
+                             cache.page_size)
     else:
-      ops.qk_norm_rope_cache(
-        qkv, self.nq, self.nkv, self.d,
-        self.q_norm.weight if self.q_norm is not None else None,
-        self.k_norm.weight if self.k_norm is not None else None,
-        eps, table, ctx.positions, cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
+      ops.qk_norm_rope_cache(qkv, self.nq, self.nkv, self.d, q_weight, k_weight, eps, table, ctx.positions,
+                             cache.k, cache.v, ctx.slots[cache.group], cache.page_size)
     out = torch.empty((T, self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
     self._attend(qkv, out, ctx, cache)
     return PendingLinear(out, self.o_weight, self.o_bias)
+
+  def _norm_heads(self, qkv: torch.Tensor) -> None:
+    """The head norms by the norm parts' own `forward`, in place on the q and k columns of the fused projection."""
+    T = qkv.shape[0]
+    nq, nkv, d = self.nq, self.nkv, self.d
+    q = qkv[:, :nq * d]
+    q.copy_(self.q_norm.forward(q.reshape(T * nq, d)).view(T, nq * d))
+    if not self.shares_kv:
+      k = qkv[:, nq * d:(nq + nkv) * d]
+      k.copy_(self.k_norm.forward(k.reshape(T * nkv, d)).view(T, nkv * d))
 
   def _attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx, cache) -> None:
     nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0
     table = ctx.block_tables[cache.group]
     if not ops.mfma_attention_supported(qkv.dtype, nq, nkv, d, cache.page_size):
       T = qkv.shape[0]
-      splits = plain_splits(T * nq, min(ctx.max_kv_len, window) if window else ctx.max_kv_len)
+      splits = plain_splits(T * nq, min(ctx.max_kv_len, window) if window else ctx.max_kv_len,
+                            16 * ops.compute_units())
       part_o = part_ml = None
       if splits > 1:
         part_o = ctx.scratch("attn_part_o", T * nq * splits * d, torch.float32)
@@ -127,12 +145,13 @@ class PagedAttention(Part):
       self._attend_decode(qkv, out, ctx, cache, ctx.num_multi, n_single)
 
   def _attend_decode(self, qkv, out, ctx, cache, first: int, count: int, front=None) -> None:
-    """Entries first .. first + count - 1, one token each.  With `front` = (rotation table, eps) the projection is
-    still raw and the kernel does the head norms, the rotation and the cache write too."""
+    """Entries first .. first + count - 1, one token each.  With `front` = (rotation table, eps, q norm weight, k norm
+    weight) the projection is still raw and the kernel does the head norms, the rotation and the cache write too."""
     nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0
     table = ctx.block_tables[cache.group]
     tile_keys, waves = ops.attn_decode_geometry(d)
-    splits = decode_splits(count * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len, tile_keys, waves)
+    splits = decode_splits(count * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len, tile_keys, waves,
+                           2 * ops.compute_units())
     need = count * nq * splits
     part_o = ctx.scratch("attn_part_o", need * d, torch.float32)
     part_ml = ctx.scratch("attn_part_ml", need * 2, torch.float32)
@@ -141,17 +160,15 @@ class PagedAttention(Part):
                       part_o, part_ml, self.scale, window)
     else:
       ops.attn_decode_front(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, first, count, splits,
-                            part_o, part_ml, self.scale, window,
-                            self.q_norm.weight if self.q_norm is not None else None,
-                            self.k_norm.weight if self.k_norm is not None else None,
-                            front[1], front[0], ctx.positions, ctx.slots[cache.group])
+                            part_o, part_ml, self.scale, window, front[2], front[3], front[1], front[0],
+                            ctx.positions, ctx.slots[cache.group])
 
 
 def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, waves: int = 4,
                   resident_workgroups: int = 512) -> int:
   """Into how many key ranges (workgroups of `waves` waves, each taking macro tiles of `tile_keys` keys in turn) a
   decoding request is cut.  `resident_workgroups` run on the chip at once (two per compute unit, whatever the head
-  size): the ranges are as many as still fit in one such round, since a second round that is nearly empty costs as
+  size; the default is an MI355X's 2 x 256, the attention part passes its device's): the ranges are as many as still fit in one such round, since a second round that is nearly empty costs as
   much as a full one (96 kv-head entries: 5 ranges take 27 us, 6 take 32); when one range per entry would leave
   more than a fifth of the round empty, two are used (384 entries: 77 against 82 us).  At most 32, which the merge
   kernel still combines in one pass over memory (one request of 32,768 keys: 34 us with 32 ranges, 47 with 64),
@@ -166,7 +183,7 @@ def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, wav
 
 def plain_splits(num_head_tokens: int, max_keys: int, resident_waves: int = 4096) -> int:
   """Into how many key ranges the one-wave-per-(token, head) kernel cuts each token's keys: as many as fill the
-  chip's wave slots (16 on each of 256 compute units) once, each range at least two tiles of 64 keys, at most 64
+  chip's wave slots (16 on each compute unit; the default is an MI355X's 16 x 256) once, each range at least two tiles of 64 keys, at most 64
   ranges.  Prompt portions have waves enough and stay whole."""
   want = resident_waves // max(1, num_head_tokens)
   tiles = -(-max_keys // 64)

@@ -66,10 +66,15 @@ class ParamSpec:
 
 @dataclass(frozen=True)
 class PagedKV:
-  """Keys and values of every past token (or of the last `window` tokens) in pages."""
+  """Keys and values of every past token (or of the last `window` tokens) in pages.  Layers whose needs are equal
+  in every field share a group: one pool of pages, one free list, one block table per request.
+  page_size: tokens per page of this group (a power of two), None = the engine's; dtype: of the pages, None = the
+  engine's.  A group with a window is given only as many pages as its requests can hold at once."""
   num_kv_heads: int
   head_dim: int
   window: Optional[int] = None
+  page_size: Optional[int] = None
+  dtype: Optional[torch.dtype] = None
 
 
 @dataclass(frozen=True)

@@ -60,6 +60,8 @@ def _fuse_norm_around_library(d, weight: torch.Tensor) -> Optional[torch.Tensor]
   M = d.residual.shape[0]
   p = d.x
   inter = weight.shape[0] // 2
+  if not getattr(d.norm, "fusable_rms", False):
+    return None
   if not (isinstance(p, PendingLinear) and p.value is None and p.bias is None and M <= ops.SKINNY_MAX_ROWS
           and inter % 4 == 0 and weight.dtype == torch.bfloat16 and weight.shape[1] == d.residual.shape[1]
           and weight.is_contiguous()):
@@ -77,9 +79,11 @@ def _fuse_norm_around_library(d, weight: torch.Tensor) -> Optional[torch.Tensor]
 
 
 def _fuse_norm(d, weight: torch.Tensor, gate_up: bool) -> Optional[torch.Tensor]:
-  """The product of a deferred norm with `weight` without a kernel for the norm, when the shapes allow it."""
+  """The product of a deferred norm with `weight` without a kernel for the norm, when the shapes allow it and the
+  norm says that it is a weight-only RMS norm (`fusable_rms`): the kernels used here restate that formula from the
+  norm's `weight` and `eps`, so a norm of any other kind is left to evaluate itself."""
   M = d.residual.shape[0]
-  if d.consumed or d.dtype != torch.bfloat16:
+  if d.consumed or d.dtype != torch.bfloat16 or not getattr(d.norm, "fusable_rms", False):
     return None
   if not ops.skinny_preferred(M, weight.shape[0], weight.shape[1], gate_up):
     return _fuse_norm_around_library(d, weight) if gate_up else None

@@ -16,7 +16,7 @@ class DeferredNorm:
   do, for few rows); any other calls `materialize()`.  After either, `residual` is the updated residual stream (it
   may be a new buffer, or the old one updated in place)."""
 
-  def __init__(self, norm: "RMSNorm", x: Optional[torch.Tensor], residual: torch.Tensor):
+  def __init__(self, norm, x: Optional[torch.Tensor], residual: torch.Tensor):
     self.norm = norm
     self.x = x
     self.residual = residual
@@ -51,7 +51,27 @@ class DeferredNorm:
     self.consumed = True
 
 
-class RMSNorm(Part):
+class Norm(Part):
+  """Base of norm kinds: `forward(x) -> y` (x [M, size] in the activation dtype or float32, y in the activation
+  dtype) and `forward_residual(x, residual, rows=None) -> y` (residual += x in place, 32-bit, x may be None, then
+  the norm of the residual; with `rows`, only those rows are normed and the residual is left as it is) are the
+  kind's own; `defer` hands the pieces to the consumer, who either evaluates them through those two methods or,
+  for a kind that says `fusable_rms`, folds them into its own kernel."""
+
+  fusable_rms = False
+
+  def defer(self, x, residual: torch.Tensor) -> DeferredNorm:
+    return DeferredNorm(self, x, residual)
+
+
+class RMSNorm(Norm):
+  # What this norm computes is exactly y = x * rsqrt(mean(x^2) + eps) * weight, with a float32 `weight` [size] and
+  # `eps`: a consumer may then fold it into a kernel of its own that restates this formula (the products' kernels
+  # take its two halves, the attention kernels norm heads with it).  A norm kind that computes anything else
+  # (a mean taken off, a bias, 1 + weight) leaves this False, which is the default: it is then always evaluated by
+  # its own `forward` / `forward_residual`, never by another part's kernel.
+  fusable_rms = True
+
   def __init__(self, spec, ctx: BuildContext):
     self.size = spec.size
     self.eps = spec.eps
@@ -65,9 +85,6 @@ class RMSNorm(Part):
     """norm(x); x [M, size] in the activation dtype or float32; result in the activation dtype."""
     out = torch.empty(x.shape, dtype=self.ctx.dtype, device=x.device)
     return ops.add_rmsnorm(x, None, self.weight, self.eps, out)
-
-  def defer(self, x: Optional[torch.Tensor], residual: torch.Tensor) -> DeferredNorm:
-    return DeferredNorm(self, x, residual)
 
   def forward_residual(self, x: Optional[torch.Tensor], residual: torch.Tensor,
                        rows: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -1,0 +1,282 @@
+"""The whole engine at the sequence lengths and batch widths that the measurements quote, against the plain
+implementation: one request of 9,001 tokens (whole, in budget-sized portions, with its last tokens decoded one by
+one, and generated from through the entry point with captured steps whose block tables are a thousand pages wide),
+and a hundred live requests decoding side by side (through the replay and through the entry point).
+
+What these lengths and widths switch on that shorter tests never reach: the prefill attention's instances chosen
+by the rule from the number of workgroups ("wide" for a whole 9,001-token prompt, "dense" for portions of 4,096,
+"two_tiles" for small ones), causal tile skipping over a hundred macro tiles, decode attention over hundreds of
+pages with many key ranges, block tables wider than 512 pages in captured steps; and for wide batches products of
+more than 64 rows (the library's), of 17 to 64 rows (k split across workgroups, by rule, and forced), decode
+attention without key ranges, sampling of a hundred rows.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import tiny_models as tm
+import trace_tools as tt
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-4
+
+# 16 query heads so that a whole prompt of 9,001 tokens makes the thousand workgroups from which on the rule picks
+# the "wide" instance; everything else small, so that the plain implementation takes seconds
+LONG = dict(
+  architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=300, hidden_size=64, intermediate_size=96,
+  num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=8, head_dim=16, hidden_act="silu",
+  max_position_embeddings=33000, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=True,
+  attention_bias=False, rope_scaling=None)
+LONG_TOKENS = 9001
+# factor on the per-head norm weights of q and k: in 32-bit, attention that picks few keys among thousands shows a
+# key that is missed or seen twice; in bfloat16 the rounding of queries and keys would grow with the scores
+SHARPEN = {"float32": 2.5, "bfloat16": 1.0}
+
+
+@pytest.fixture(scope="module")
+def long_model(tmp_path_factory):
+  base = tm.random_weights(LONG, seed=21, dtype=torch.bfloat16, std=0.05)
+  tokens = tm.random_tokens(LONG, LONG_TOKENS, seed=77)
+  out = dict(tokens=tokens, weights={}, want={}, folders={})
+  for name, dt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+    w = dict(base)
+    for k in w:
+      if k.endswith("q_norm.weight") or k.endswith("k_norm.weight"):
+        w[k] = (w[k].float() * SHARPEN[name]).to(torch.bfloat16)
+    wf = {k: v.float() for k, v in w.items()}
+    out["weights"][name] = wf
+    print(f"plain implementation, {LONG_TOKENS} tokens, weights for {name} ...", flush=True)
+    out["want"][name] = plain.qwen3_logits(tokens, wf, dict(LONG)).numpy()
+    out["folders"][name] = str(tmp_path_factory.mktemp("long") / name)
+    tm.write_model(out["folders"][name], LONG, {k: v.to(dt) for k, v in w.items()})
+  return out
+
+
+def _cut(tokens, sizes, rid="r"):
+  steps, i = [], 0
+  for s, n in enumerate(sizes):
+    n = min(n, len(tokens) - i)
+    steps.append({"step": s, "entries": [{"id": rid, "tokens": tokens[i:i + n], "want": list(range(n))}], "end": []})
+    i += n
+  assert i == len(tokens)
+  steps[-1]["end"] = [rid]
+  return steps
+
+
+# seen on an MI355X in bfloat16: max 0.9%, mean 0.12% of the largest logit; the bounds are about twice that
+BF16_MAX, BF16_MEAN = 0.02, 0.003
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_request_of_9001_tokens_under_every_way_of_cutting(long_model, dtype, monkeypatch):
+  from miniinfer_amd.engine.replay import Replayer
+  from miniinfer_amd.kernels import ops
+  tokens, want = long_model["tokens"], long_model["want"][dtype]
+  requests = {"r": tokens}
+  seen = []
+  real = ops.attn_prefill
+  nkv = LONG["num_key_value_heads"]
+
+  def spy(*a, **k):
+    work = a[8]
+    seen.append((k.get("variant", "auto"), work.shape[0] * nkv))
+    return real(*a, **k)
+
+  monkeypatch.setattr(ops, "attn_prefill", spy)
+  plans = {
+    "whole": tt.whole(requests),
+    "budget_portions": _cut(tokens, [4096, 300, 4096, 509]),
+    "tail_decoded": tt.tail_decoded(requests, 32),
+  }
+  worst = {}
+  for name, steps in plans.items():
+    print(f"9,001 tokens {dtype} {name}: {len(steps)} steps", flush=True)
+    rp = Replayer(long_model["folders"][dtype], dtype, tt.peak_tokens(steps, requests), page_size=16)
+    outs = []
+    for st in steps:
+      outs.append(rp.step(st))
+    rp.cache.check()
+    assert rp.cache.all_pages_free() and not rp.cache.live_requests()
+    got = tt.gather(steps, outs, requests, LONG["vocab_size"])["r"]
+    assert not np.isnan(got).any()
+    err = np.abs(got - want)
+    scale = np.abs(want).max()
+    worst[name] = (float(err.max() / scale), float(err.mean() / scale), int(err.max(-1).argmax()))
+    if dtype == "float32":
+      assert err.max() <= FP32_TOL, f"{name}: max abs err {err.max():.3g} at position {err.max(-1).argmax()}"
+    else:
+      assert err.max() <= BF16_MAX * scale, f"{name}: max err {err.max():.4g} of scale {scale:.4g}"
+      assert err.mean() <= BF16_MEAN * scale, f"{name}: mean err {err.mean():.4g} of scale {scale:.4g}"
+  print(f"9,001 tokens {dtype}: (max, mean) error / largest logit, worst position: {worst}", flush=True)
+  if dtype == "bfloat16":
+    # the rule itself chose all three instances of the prefill kernel
+    units = ops.compute_units()
+    assert any(v == "wide" for v, _ in seen), seen
+    assert any(v == "auto" and wg > 2 * units for v, wg in seen), seen       # "dense"
+    assert any(v == "auto" and wg <= 2 * units for v, wg in seen), seen      # "two_tiles"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_generating_after_9001_tokens_from_captured_steps_a_thousand_pages_wide(long_model, dtype):
+  from miniinfer_amd import LLMEngine, SamplingParams
+  tokens, w = long_model["tokens"], long_model["weights"][dtype]
+  n_new = 6
+  with LLMEngine(model=long_model["folders"][dtype], dtype=dtype, page_size=16, num_pages=640, max_num_seqs=2,
+                 max_model_len=10000, max_num_batched_tokens=4096) as eng:
+    out = eng.generate([tokens], SamplingParams(temperature=0.0, max_tokens=n_new, ignore_eos=True), use_tqdm=False)[0]
+    widths = {wd for b, wd in eng.runner._graphs if b == 1}
+    assert eng.runner.use_graphs and max(widths) >= 512 and all(g.ok for g in eng.runner._graphs.values()), widths
+    assert eng.cache.all_pages_free()
+  got = out["token_ids"]
+  assert len(got) == n_new
+  # one plain pass over the prompt and what was generated: every generated token is the plain implementation's
+  # choice at its place given the same history (32-bit), or all but ties for it (bfloat16)
+  lg = plain.qwen3_logits(tokens + got, w, dict(LONG))
+  for i, tok in enumerate(got):
+    row = lg[len(tokens) - 1 + i]
+    if dtype == "float32":
+      assert int(row.argmax()) == tok, f"token {i}: {tok}, plain {int(row.argmax())}"
+    else:
+      assert row[tok] >= row.max() - BF16_MAX * row.abs().max(), f"token {i} ({tok}) is not near the plain top"
+
+
+# --------------------------------------------------------------------------- a hundred live requests
+
+# the benchmark's layer sizes (so that the products are the shapes whose kernels are chosen by rows: rows of 1,024,
+# 2,048 and 3,072 columns) with a small vocabulary and two layers
+WIDE = dict(
+  architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=2048, hidden_size=1024, intermediate_size=3072,
+  num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=8, head_dim=128, hidden_act="silu",
+  max_position_embeddings=4096, rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False,
+  attention_bias=False, rope_scaling=None)
+NUM_LIVE = 100
+DECODED = 5
+
+
+@pytest.fixture(scope="module")
+def wide_model(tmp_path_factory):
+  import random
+  rng = random.Random(5)
+  base = tm.random_weights(WIDE, seed=4, dtype=torch.bfloat16, std=0.03)
+  requests = {f"r{i}": tm.random_tokens(WIDE, rng.randint(12, 48), seed=900 + i) for i in range(NUM_LIVE)}
+  wf = {k: v.float() for k, v in base.items()}
+  out = dict(requests=requests, weights=wf, folders={})
+  print(f"plain implementation, {NUM_LIVE} requests ...", flush=True)
+  out["want"] = {rid: plain.qwen3_logits(t, wf, dict(WIDE)).numpy() for rid, t in requests.items()}
+  for name, dt in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+    out["folders"][name] = str(tmp_path_factory.mktemp("wide") / name)
+    tm.write_model(out["folders"][name], WIDE, {k: v.to(dt) for k, v in base.items()})
+  return out
+
+
+def _wide_steps(requests, live_counts):
+  """Prompts but for their last DECODED tokens, ten requests a step; then DECODED steps in which the first
+  live_counts[i] requests bring one token each."""
+  ids = list(requests)
+  steps = []
+  for s0 in range(0, len(ids), 10):
+    steps.append({"step": len(steps), "end": [],
+                  "entries": [{"id": r, "tokens": requests[r][:-DECODED], "want": list(range(len(requests[r]) - DECODED))}
+                              for r in ids[s0:s0 + 10]]})
+  done = {r: len(requests[r]) - DECODED for r in ids}
+  for n in live_counts:
+    entries = []
+    for r in ids[:n]:
+      entries.append({"id": r, "tokens": [requests[r][done[r]]], "want": [0]})
+      done[r] += 1
+    steps.append({"step": len(steps), "entries": entries, "end": []})
+  steps[-1]["end"] = ids
+  return steps, done
+
+
+# seen in bfloat16: max 0.5%, mean 0.07% of the largest logit
+WIDE_BF16_MAX, WIDE_BF16_MEAN = 0.012, 0.002
+
+
+@pytest.mark.parametrize("products", ["by_rule", "k_split", "library", "own_rows"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_hundred_requests_decode_side_by_side(wide_model, dtype, products, monkeypatch):
+  """Steps of 100, 100, 64, 40 and 17 single tokens (the last three are the widths at which a product of few rows
+  may go to this library's kernels): by the rule, and with every product forced to the k-split kernel, to the
+  library, or to the kernel that owns whole rows."""
+  from miniinfer_amd.engine.replay import Replayer
+  from miniinfer_amd.kernels import ops
+  if dtype == "float32" and products != "by_rule":
+    pytest.skip("the 32-bit mode has one product kernel")
+  requests, want = wide_model["requests"], wide_model["want"]
+  steps, done = _wide_steps(requests, [100, 100, 64, 40, 17])
+  choices = ops.ProductChoices()
+  choices.force = {"by_rule": None, "k_split": ops.OWN_KSPLIT, "library": ops.LIBRARY, "own_rows": ops.OWN_ROWS}[products]
+  rp = Replayer(wide_model["folders"][dtype], dtype, tt.peak_tokens(steps, requests), page_size=16,
+                max_requests=NUM_LIVE, choices=choices)
+  seen_variants = []
+  real = ops._skinny_call
+
+  def spy(lib, variant, *a, **k):
+    seen_variants.append((variant, a[6]))        # (variant, rows of the left operand)
+    return real(lib, variant, *a, **k)
+
+  monkeypatch.setattr(ops, "_skinny_call", spy)
+  outs = [rp.step(st) for st in steps]
+  rp.cache.check()
+  assert rp.cache.all_pages_free()
+  if dtype == "bfloat16":
+    wide_rows = {v for v, m in seen_variants if 17 <= m <= 64}
+    if products in ("by_rule", "k_split"):
+      assert 1 in wide_rows, f"no product of 17 to 64 rows had its k split: {sorted(set(seen_variants))}"
+    if products == "library":
+      assert choices.library_products[0] > 0 and not wide_rows
+    if products == "own_rows":
+      assert wide_rows == {0}
+  got = tt.gather(steps, outs, {r: t[:done[r]] for r, t in requests.items()}, WIDE["vocab_size"])
+  worst = (0.0, 0.0)
+  for rid in requests:
+    n = done[rid]
+    assert not np.isnan(got[rid]).any()
+    err = np.abs(got[rid] - want[rid][:n])
+    scale = np.abs(want[rid]).max()
+    worst = max(worst, (float(err.max() / scale), float(err.mean() / scale)))
+    if dtype == "float32":
+      assert err.max() <= FP32_TOL, f"request {rid}: max abs err {err.max():.3g}"
+    else:
+      assert err.max() <= WIDE_BF16_MAX * scale, f"request {rid}: max err {err.max():.4g} of scale {scale:.4g}"
+      assert err.mean() <= WIDE_BF16_MEAN * scale, f"request {rid}: mean err {err.mean():.4g} of scale {scale:.4g}"
+  print(f"100 live requests {dtype} {products}: largest (max, mean) error / largest logit {worst}", flush=True)
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_hundred_requests_generate_through_the_entry_point(wide_model, dtype, graphs):
+  """100 requests at once through `LLMEngine`: steps of 100 sampled rows, decode steps from the captured graphs of
+  the 128- and (once some requests have ended) 96-entry buckets and below; every token is checked against one plain
+  pass over the request's own history."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  requests, w = wide_model["requests"], wide_model["weights"]
+  prompts = [t[:max(4, len(t) - 20)] for t in requests.values()]
+  # requests end at different times, so that the decode steps walk down through the batch buckets
+  params = [SamplingParams(temperature=0.0, max_tokens=3 + (i % 4) * 2 + (6 if i < 70 else 0), ignore_eos=True)
+            for i in range(len(prompts))]
+  with LLMEngine(model=wide_model["folders"][dtype], dtype=dtype, page_size=16, num_pages=600, max_num_seqs=128,
+                 max_model_len=256, max_num_batched_tokens=2048, enforce_eager=not graphs) as eng:
+    outs = eng.generate(prompts, params, use_tqdm=False)
+    if graphs:
+      buckets = {b for b, _ in eng.runner._graphs}
+      assert 128 in buckets and 96 in buckets, buckets
+      assert all(g.ok for g in eng.runner._graphs.values())
+    assert eng.cache.all_pages_free() and not eng._requests
+  near = 0
+  for p, sp, o in zip(prompts, params, outs):
+    got = o["token_ids"]
+    assert len(got) == sp.max_tokens
+    lg = plain.qwen3_logits(p + got, w, dict(WIDE))
+    for i, tok in enumerate(got):
+      row = lg[len(p) - 1 + i]
+      if dtype == "float32":
+        assert int(row.argmax()) == tok
+      else:
+        assert row[tok] >= row.max() - 0.02 * row.abs().max(), f"token {i} ({tok}) is not near the plain top"
+        near += int(row.argmax()) != tok
+  print(f"100 requests through the entry point, {dtype}, graphs {graphs}: {near} tokens were near ties", flush=True)

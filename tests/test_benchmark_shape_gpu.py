@@ -80,7 +80,7 @@ def test_benchmark_shape_under_every_way_of_cutting(shape_model, dtype):
     for st in steps:
       outs.append(rp.step(st))
       rp.cache.check()
-    assert rp.cache.num_free_pages() == rp.cache.num_pages and not rp.cache.live_requests()
+    assert rp.cache.all_pages_free() and not rp.cache.live_requests()
     got = tt.gather(steps, outs, requests, SHAPE["vocab_size"])
     for rid in requests:
       assert not np.isnan(got[rid]).any()
@@ -110,7 +110,7 @@ def test_benchmark_shape_generates_through_the_entry_point(shape_model, dtype):
     assert eng.runner.use_graphs and eng.config.enable_overlap and eng.config.tune_products
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=n_new, ignore_eos=True), use_tqdm=False)
     assert len(eng.runner._graphs) > 0, "decode steps were meant to come from captured graphs"
-    assert eng.cache.num_free_pages() == eng.cache.num_pages
+    assert eng.cache.all_pages_free()
   for p, o in zip(prompts, outs):
     if dtype == "float32":
       assert o["token_ids"] == plain.greedy_generate(p, n_new, w, cfg)

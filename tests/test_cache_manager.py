@@ -126,3 +126,96 @@ def test_random_orders_keep_the_books(seed):
     m.release(r)
   m.check()
   assert m.num_free_pages() == 24 and m.num_free_slots() == 5
+
+
+def test_groups_may_have_page_sizes_dtypes_and_pool_sizes_of_their_own():
+  """A group names its own page size and dtype; a group with a window gets only the pages its requests can hold at
+  once; a group that keeps every key has room for num_pages * page_size tokens whatever its own page size."""
+  full, coarse = PagedKV(2, 8), PagedKV(1, 16, page_size=32, dtype=torch.float32)
+  win = PagedKV(2, 8, window=20, page_size=4)
+  m = CacheManager([full, coarse, win, full], page_size=8, num_pages=64, max_requests=3, max_model_len=512,
+                   dtype=torch.bfloat16, device="cpu", max_step_tokens=40)
+  assert [g.page_size for g in m.paged] == [8, 32, 4] and [g.layers for g in m.paged] == [[0, 3], [1], [2]]
+  assert m.paged[0].pool.num_pages == 64 and m.paged[1].pool.num_pages == 16      # 512 tokens each
+  # window 20 in pages of 4: (5 + 3) pages a request, 10 pages for a step's 40 new tokens
+  assert m.paged[2].pool.num_pages == CacheManager.window_pool_pages(20, 4, 3, 40) == 3 * 8 + 10
+  assert m.paged[0].k.shape == (2, 65, 2, 8, 8) and m.paged[0].k.dtype == torch.bfloat16
+  assert m.paged[1].v.shape == (1, 17, 1, 16, 32) and m.paged[1].k.dtype == torch.float32
+  assert m.paged[2].k.shape == (1, 35, 2, 4, 8)
+  assert m.layer_cache(1).page_size == 32 and m.layer_cache(2).page_size == 4 and m.layer_cache(0).page_size == 8
+  assert m.min_page_size == 4 and m.max_pages_per_request == 128
+  want = 2 * 2 * 2 * 8 * 8 * 2 * 65 + 2 * 1 * 16 * 32 * 4 * 17 + 2 * 2 * 8 * 4 * 2 * 35
+  assert CacheManager.storage_bytes([full, coarse, win, full], 8, 64, 3, 40, torch.bfloat16) == want
+  assert sum(t.numel() * t.element_size() for g in m.paged for t in (g.k, g.v)) == want
+  m.admit("a")
+  m.grow("a", 33); m.commit("a", 33)
+  assert [len(m.table(g, "a")) for g in range(3)] == [5, 2, 9]
+  # the next token, at 33, sees keys 14..33: the window group's pages 0..2 (keys 0..11) are gone
+  assert m.table(2, "a")[:3] == [0, 0, 0] and all(p > 0 for p in m.table(2, "a")[3:])
+  m.check()
+  m.release("a")
+  assert m.all_pages_free()
+
+
+def test_room_is_booked_per_group():
+  full, coarse = PagedKV(1, 8), PagedKV(1, 8, page_size=16)
+  m = CacheManager([full, coarse], page_size=4, num_pages=16, max_requests=4, max_model_len=64, dtype=torch.float32,
+                   device="cpu")
+  assert m.room() == [16, 4]
+  m.admit("a"); m.admit("b")
+  m.grow("a", 17); m.commit("a", 17)                 # 5 fine pages, 2 coarse ones
+  room = m.room()
+  assert room == [11, 2]
+  assert m.tokens_that_fit(room, "a") == min((5 + 11) * 4, (2 + 2) * 16) == 64
+  assert m.tokens_that_fit(room, "b") == 32           # the coarse group is the tighter one for a new request
+  assert m.fits(room, "b", 32) and not m.fits(room, "b", 33) and not m.fits(room, "b", 32, spare=1)
+  assert m.take(room, "b", 20) and room == [6, 0]
+  assert m.take(room, "a", 24) and room == [5, 0]     # one more fine page, no coarse one
+  assert not m.take(room, "a", 33) and room == [5, 0]   # refused: nothing booked
+  assert m.room() == [11, 2]                          # the manager's own books are untouched by a plan
+  assert m.pages_needed("b", 20) == 5 and m.can_grow("b", 32) and not m.can_grow("b", 33)
+  with pytest.raises(OutOfPages):
+    m.grow("b", 33)
+  assert m.held_pages("b") == 0                       # all or nothing
+  assert m.never_fits(64) is None and "group 0" in m.never_fits(65)
+  w = CacheManager([PagedKV(1, 8, window=8)], page_size=4, num_pages=6, max_requests=1, max_model_len=4096,
+                   dtype=torch.float32, device="cpu")
+  assert w.never_fits(4000) is None                   # a window needs the pages of its window only
+  assert CacheManager([PagedKV(1, 8, window=64)], page_size=4, num_pages=6, max_requests=1, max_model_len=4096,
+                      dtype=torch.float32, device="cpu").never_fits(4000) is not None
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_orders_keep_the_books_of_unlike_groups(seed):
+  rnd = random.Random(100 + seed)
+  needs = [PagedKV(1, 8), PagedKV(1, 8, page_size=16), PagedKV(1, 8, window=24, page_size=4), PagedKV(2, 8, window=9)]
+  m = CacheManager(needs, page_size=8, num_pages=24, max_requests=5, max_model_len=400, dtype=torch.float32,
+                   device="cpu", max_step_tokens=30)
+  live = {}
+  next_id = 0
+  for _ in range(800):
+    op = rnd.random()
+    if op < 0.25 and m.num_free_slots() > 0:
+      m.admit(next_id); live[next_id] = 0; next_id += 1
+    elif op < 0.85 and live:
+      # one step: several requests grow together, planned against one copy of the room, within the step's tokens
+      room, plan, left = m.room(), [], 30
+      for r in rnd.sample(list(live), k=min(len(live), rnd.choice([1, 2, 3]))):
+        n = min(left, rnd.choice([1, 1, 1, 2, 7, 30]), 400 - live[r])
+        if n > 0 and m.take(room, r, live[r] + n):
+          plan.append((r, live[r] + n))
+          left -= n
+      for r, new_len in plan:
+        m.grow(r, new_len)                              # never refused: the plan was booked
+      for r, new_len in plan:
+        m.commit(r, new_len); live[r] = new_len
+    elif live:
+      r = rnd.choice(list(live))
+      m.release(r); del live[r]
+    m.check()
+    for r, n in live.items():
+      assert m.length(r) == n and [m.held_pages(r, g) for g in range(4)] == [-(-n // 8), -(-n // 16), -(-n // 4), -(-n // 8)]
+  for r in list(live):
+    m.release(r)
+  m.check()
+  assert m.all_pages_free() and m.num_free_slots() == 5

@@ -27,7 +27,7 @@ def test_greedy_config_a(tmp_path):
   assert [o["token_ids"] for o in outs] == want
   assert all(o["finish_reason"] == "max_tokens" for o in outs)
   eng.cache.check()
-  assert eng.cache.num_free_pages() == eng.cache.num_pages
+  assert eng.cache.all_pages_free()
 
 
 def test_greedy_config_b_chunked_budget_32(tmp_path):
@@ -40,7 +40,7 @@ def test_greedy_config_b_chunked_budget_32(tmp_path):
                  max_num_batched_tokens=32) as eng:
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True), use_tqdm=False)
   assert [o["token_ids"] for o in outs] == want
-  assert eng.cache.num_free_pages() == eng.cache.num_pages
+  assert eng.cache.all_pages_free()
 
 
 def test_greedy_survives_preemption(tmp_path):
@@ -54,7 +54,7 @@ def test_greedy_survives_preemption(tmp_path):
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True), use_tqdm=False)
     assert eng.scheduler.num_preemptions > 0, "the test is meant to run out of pages"
   assert [o["token_ids"] for o in outs] == want
-  assert eng.cache.num_free_pages() == eng.cache.num_pages
+  assert eng.cache.all_pages_free()
 
 
 def test_greedy_bfloat16_follows_plain(tmp_path):
@@ -157,7 +157,7 @@ def test_launching_ahead_of_the_tokens_changes_no_token(tmp_path, dtype):
         eng.scheduler.eos_token_id = eng.eos_token_id = probe[3]
       outs = eng.generate(prompts, params, use_tqdm=False)
       results[overlap] = [(o["token_ids"], o["finish_reason"]) for o in outs]
-      assert eng.cache.num_free_pages() == eng.cache.num_pages and eng.is_finished()
+      assert eng.cache.all_pages_free() and eng.is_finished()
       eng.cache.check()
       if overlap:
         assert eng.scheduler.num_preemptions > 0, "the test is meant to run out of pages"
@@ -185,7 +185,7 @@ def test_stream_generate_yields_every_token_once_and_in_order(tmp_path):
           ended[out.request_id] = out.finish_reason
       assert [seen[r] for r in sorted(seen, key=lambda r: int(r.split("-")[1]))] == [o["token_ids"] for o in whole]
       assert list(ended.values()) == ["max_tokens"] * 3 and eng.is_finished()
-      assert eng.cache.num_free_pages() == eng.cache.num_pages
+      assert eng.cache.all_pages_free()
 
 
 def test_eos_comes_from_generation_config_json(tmp_path):
@@ -277,13 +277,13 @@ def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, produ
   prompts = [tm.random_tokens(cfg, n, seed=90 + n) for n in (7, 60, 33)]
   with LLMEngine(model=str(tmp_path / "m"), dtype="bfloat16", page_size=8, num_pages=64, max_num_seqs=4,
                  tune_products=False, max_num_batched_tokens=48) as eng:
-    before = ops.library_products_run()[0]
+    before = eng.choices.library_products[0]
     scaled_activations = []
     real = ops.silu_mul_scaled
     monkeypatch.setattr(ops, "silu_mul_scaled", lambda *a, **k: (scaled_activations.append(1), real(*a, **k))[1])
     if products == "own":
-      with ops.own_products_only():
-        outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
+      eng.choices.own_only = True
+      outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
     else:
       choice = {"own_ksplit": ops.OWN_KSPLIT, "own_staged": ops.OWN_ROWS_STAGED,
                 "own_staged_lines": ops.OWN_ROWS_STAGED_LINES, "own_both_staged": ops.OWN_ROWS_BOTH_STAGED,
@@ -293,12 +293,10 @@ def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, produ
           # (library_gate_up: only the gate|up product goes to the library; the product before it keeps the norm's
           # first half in its ending, and the activation kernel applies the norm's row factor)
           mine = choice if products != "library_gate_up" or m[1] else ops.OWN_ROWS
-          ops.set_product_choice(rows, m[0].shape[0], m[0].shape[1], m[1], mine)
-      try:
-        outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
-      finally:
-        ops.clear_product_choices()
-    ran_library = ops.library_products_run()[0] - before
+          eng.choices.set(rows, m[0].shape[0], m[0].shape[1], m[1], mine)      # the engine's own table
+      outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True), use_tqdm=False)
+    assert not ops.current_choices().table                    # and nobody else's
+    ran_library = eng.choices.library_products[0] - before
     assert (ran_library > 0) == (products in ("library", "library_gate_up"))
     assert (len(scaled_activations) > 0) == (products == "library_gate_up")
   for p, o in zip(prompts, outs):
@@ -307,3 +305,59 @@ def test_bfloat16_tokens_follow_plain_with_either_product_kernel(tmp_path, produ
       lg = plain.qwen3_logits(hist, w, dict(cfg))[-1]
       assert lg[tok] >= lg.max() - 0.03 * lg.abs().max(), f"token {tok} is not near the plain top"
       hist.append(tok)
+
+
+def test_add_request_and_step_loop_hands_finished_requests_out_and_keeps_none(tmp_path):
+  """The documented loop of `add_request` and `step` (no `generate`): every finished request comes out of exactly
+  one `StepOutput.finished`, with its tokens, and the engine keeps no reference to it."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "A")
+  prompts = [tm.random_tokens(cfg, n, seed=60 + n) for n in (5, 17, 33, 9)]
+  want = {f"req-{i}": plain.greedy_generate(p, 6 + i, w, dict(cfg)) for i, p in enumerate(prompts)}
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=16, num_pages=32, max_num_seqs=4) as eng:
+    for rounds in range(2):                     # the second round reuses the ids' numbers' successors
+      ids = [eng.add_request(p, SamplingParams(temperature=0.0, max_tokens=6 + i, ignore_eos=True))
+             for i, p in enumerate(prompts)]
+      got = {}
+      while not eng.is_finished():
+        for r in eng.step().finished:
+          assert r.request_id not in got
+          got[r.request_id] = (list(r.outputs), r.finish_reason)
+      assert sorted(got) == sorted(ids) and not eng._requests
+      for i, rid in enumerate(ids):
+        assert got[rid] == (want[f"req-{i}"], "max_tokens")
+    assert eng.cache.all_pages_free()
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_overlapped_loop_lets_a_decode_sit_out_while_others_overwrite_the_device_tokens(tmp_path, graphs):
+  """The overlapped loop with so few pages that a decode must wait: request a reaches max_tokens while its last
+  token is still on the device, so its pages come back one call later; b's next token needs a new page and none is
+  free, so b sits a step out (it is not preempted) while c decodes and its sampled token overwrites the device
+  buffer from which b's own placeholder was to be read.  b must come back with its real token: every request's
+  tokens are the plain implementation's."""
+  from miniinfer_amd import LLMEngine, SamplingParams
+  cfg, w = _model(tmp_path, "B")
+  P = 8
+  spec = [(8, 2), (15, 4), (24, 6)]             # (prompt tokens, max_tokens) of a, b, c
+  prompts = [tm.random_tokens(cfg, n, seed=70 + n) for n, _ in spec]
+  want = [plain.greedy_generate(p, m, w, dict(cfg)) for p, (_, m) in zip(prompts, spec)]
+  with LLMEngine(model=str(tmp_path / "m"), dtype="float32", page_size=P, num_pages=8, max_num_seqs=3,
+                 max_num_batched_tokens=64, enable_overlap=True, enforce_eager=not graphs) as eng:
+    sat_out = []
+    real = eng.scheduler.schedule
+
+    def schedule():
+      plan = real()
+      decoding = [r for r in eng.scheduler.running if r.remaining == 1 and r.num_computed > 0]
+      inside = {id(e.request) for e in plan.entries} if plan is not None else set()
+      sat_out.extend(r.request_id for r in decoding if id(r) not in inside)
+      return plan
+
+    eng.scheduler.schedule = schedule
+    outs = eng.generate(prompts, [SamplingParams(temperature=0.0, max_tokens=m, ignore_eos=True) for _, m in spec],
+                        use_tqdm=False)
+    assert eng.scheduler.num_preemptions == 0
+    assert "req-1" in sat_out, "the test is meant to leave b's decode out of a step"
+    assert eng.cache.all_pages_free()
+  assert [o["token_ids"] for o in outs] == want

@@ -136,11 +136,11 @@ def test_a_step_whose_products_could_go_either_way_is_captured_both_ways(tmp_pat
       rn.cache.admit(r)
       rn.step([StepEntry(r, tm.random_tokens(cfg, 2 + r % 11, seed=r), [])])
       live.append(r)
-    before = ops.library_products_run()
+    before = tuple(rn.choices.library_products)
     for t in range(5):
       outs[k].append(rn.step([StepEntry(q, [(5 * q + t) % cfg["vocab_size"]], [0]) for q in live]).float().cpu())
       torch.cuda.synchronize()
-    after = ops.library_products_run()
+    after = tuple(rn.choices.library_products)
     counted.append((after[0] - before[0], after[1] - before[1]))
   assert counted[0][1] > 0, "the eager steps of 24 rows sent no avoidable product to the library"
   assert {b for b, _ in runners[1]._graphs} == {24}

@@ -42,7 +42,7 @@ def _replay(folder, dtype, steps, requests, page_size, max_tokens):
   for st in steps:
     outs.append(rp.step(st))
     rp.cache.check()
-  assert rp.cache.num_free_pages() == rp.cache.num_pages, "pages were not all given back"
+  assert rp.cache.all_pages_free(), "pages were not all given back"
   assert not rp.cache.live_requests()
   return outs
 
@@ -101,7 +101,7 @@ def test_prefill_variant_for_long_prompts_through_the_engine(tmp_path, name, mon
   """The prefill attention's instance with two blocks of query columns per wave is chosen for steps with thousands of
   workgroups; with the threshold lowered to one, the tiny configurations run through it, whole and mixed."""
   from miniinfer_amd.kernels import ops
-  monkeypatch.setattr(ops, "PREFILL_WIDE_MIN_WORKGROUPS", 1)
+  monkeypatch.setattr(ops, "PREFILL_WIDE_WORKGROUPS_PER_UNIT", 0)
   seen = []
   real = ops.attn_prefill
   monkeypatch.setattr(ops, "attn_prefill", lambda *a, **k: (seen.append(k.get("variant")), real(*a, **k))[1])

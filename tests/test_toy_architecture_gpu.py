@@ -255,7 +255,7 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
     for st in steps:
       outs.append(rp.step(st))
       rp.cache.check()
-    assert rp.cache.num_free_pages() == rp.cache.num_pages
+    assert rp.cache.all_pages_free()
     got = tt.gather(steps, outs, requests, 300)
     for r in requests:
       err = np.abs(got[r] - want[r]).max()
@@ -287,7 +287,7 @@ def test_toy_architecture_generates_through_the_entry_point_and_survives_preempt
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True), use_tqdm=False)
     assert eng.scheduler.num_preemptions > 0, "the test is meant to run out of pages"
     eng.cache.check()
-    assert eng.cache.num_free_pages() == eng.cache.num_pages and eng.cache.num_free_slots() == 3
+    assert eng.cache.all_pages_free() and eng.cache.num_free_slots() == 3
   assert [o["token_ids"] for o in outs] == want
 
 
@@ -336,5 +336,5 @@ def test_recordable_toy_architecture_generates_from_graphs(tmp_path):
     assert eng.runner.use_graphs
     outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True), use_tqdm=False)
     assert eng.scheduler.num_preemptions > 0 and len(eng.runner._graphs) > 0
-    assert eng.cache.num_free_pages() == eng.cache.num_pages
+    assert eng.cache.all_pages_free()
   assert [o["token_ids"] for o in outs] == want

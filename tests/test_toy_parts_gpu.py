@@ -270,7 +270,7 @@ def test_routed_feed_forward_and_other_position_encodings_are_registered_built_a
     for st in steps:
       outs.append(rp.step(st))
       rp.cache.check()
-    assert rp.cache.num_free_pages() == rp.cache.num_pages
+    assert rp.cache.all_pages_free()
     got = tt.gather(steps, outs, requests, 200)
     for r in requests:
       err = np.abs(got[r] - want[r]).max()
