@@ -10,47 +10,59 @@
 // miniinfer/layers/attention.py:112-128; query head h reads kv head h / (nq / nkv)
 // (miniinfer/layers/attention.py:131-191); softmax(scale * q.k) v.
 //
-// One wave per (token, query head).  A tile is 64 keys: each lane scores one key (the query
-// is broadcast from LDS), the wave reduces max and sum for the running softmax, then the lanes
-// switch to output columns and add the tile's probability-weighted value rows.  With few tokens
-// and many keys the key range of each (token, head) is cut into num_splits parts of whole tiles, one
-// wave each, which leave an unnormalised sum with its running maximum and denominator in scratch
+// One wave per (token, query heads of one kv head).  A tile is 64 keys: each lane scores one key against the
+// wave's queries (broadcast from LDS; the key row is loaded once for all of them), the wave reduces max and sum
+// for each head's running softmax, then the lanes switch to output columns and add the tile's probability-weighted
+// value rows.  With few tokens and many keys the key range of each token is cut into num_splits parts of whole
+// tiles, one wave each, which leave an unnormalised sum with its running maximum and denominator in scratch
 // memory; a second kernel combines them (the parts' order of summation is the only difference).
 // Key pages are [num_pages, nkv, P, d]; value pages are stored transposed, [num_pages, nkv, d, P].
 #include "common.h"
 
-template <typename T, int VEC>
-__device__ __forceinline__ float dot_row(const float* __restrict__ qs, const T* __restrict__ row, int d);
+// scores of one key row against REP queries (qs [REP][d] in LDS): every element of the row is loaded once; each
+// query's sum is one chain of fused multiply-adds over the dims in ascending order
+template <typename T, int REP>
+__device__ __forceinline__ void dot_rows(const float* __restrict__ qs, const T* __restrict__ row, int d, float (&s)[REP]);
 
-template <>
-__device__ __forceinline__ float dot_row<float, 4>(const float* __restrict__ qs, const float* __restrict__ row, int d) {
-  float acc = 0.f;
-  for (int e = 0; e < d; e += 4) {
-    const float4 kv = *reinterpret_cast<const float4*>(row + e);
-    acc = fmaf(qs[e], kv.x, acc);
-    acc = fmaf(qs[e + 1], kv.y, acc);
-    acc = fmaf(qs[e + 2], kv.z, acc);
-    acc = fmaf(qs[e + 3], kv.w, acc);
-  }
-  return acc;
-}
-
-template <>
-__device__ __forceinline__ float dot_row<bf16, 8>(const float* __restrict__ qs, const bf16* __restrict__ row, int d) {
-  float acc = 0.f;
-  for (int e = 0; e < d; e += 8) {
-    const uint4 raw = *reinterpret_cast<const uint4*>(row + e);
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+template <int REP>
+__device__ __forceinline__ void dot_rows_f32(const float* __restrict__ qs, const float* __restrict__ row, int d, float (&s)[REP]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      acc = fmaf(qs[e + 2 * i], __uint_as_float(w[i] << 16), acc);
-      acc = fmaf(qs[e + 2 * i + 1], __uint_as_float(w[i] & 0xffff0000u), acc);
-    }
+  for (int x = 0; x < REP; ++x) s[x] = 0.f;
+#pragma unroll 4
+  for (int e = 0; e < d; e += 4) {
+    float kv[4];
+    load4(row + e, kv);
+#pragma unroll
+    for (int x = 0; x < REP; ++x)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[x] = fmaf(qs[x * d + e + i], kv[i], s[x]);
   }
-  return acc;
 }
 
-template <typename T, int VEC>
+template <int REP>
+__device__ __forceinline__ void dot_rows_bf16(const float* __restrict__ qs, const bf16* __restrict__ row, int d, float (&s)[REP]) {
+#pragma unroll
+  for (int x = 0; x < REP; ++x) s[x] = 0.f;
+#pragma unroll 2
+  for (int e = 0; e < d; e += 8) {
+    float kv[8];
+    load4(row + e, *reinterpret_cast<float(*)[4]>(&kv[0]));
+    load4(row + e + 4, *reinterpret_cast<float(*)[4]>(&kv[4]));
+#pragma unroll
+    for (int x = 0; x < REP; ++x)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s[x] = fmaf(qs[x * d + e + i], kv[i], s[x]);
+  }
+}
+
+template <int REP>
+__device__ __forceinline__ void dot_rows_any(const float* qs, const float* row, int d, float (&s)[REP]) { dot_rows_f32<REP>(qs, row, d, s); }
+template <int REP>
+__device__ __forceinline__ void dot_rows_any(const float* qs, const bf16* row, int d, float (&s)[REP]) { dot_rows_bf16<REP>(qs, row, d, s); }
+
+// One wave per (token, group of REP query heads, key range).  REP = the query heads of a kv head when that is 1, 2, 4
+// or 8 (the keys and values are then read once for all of them), else 1 (a wave per query head).
+template <typename T, int REP>
 __global__ __launch_bounds__(256) void paged_attention_kernel(
     const T* __restrict__ q, int64_t q_row_stride, T* __restrict__ out, int64_t out_row_stride,
     const T* __restrict__ k_pages, const T* __restrict__ v_pages, const int* __restrict__ block_table, int table_width,
@@ -60,17 +72,18 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   extern __shared__ float smem[];
   const int lane = threadIdx.x & (MI_WAVE - 1);
   const int wave = threadIdx.x / MI_WAVE;
-  float* qs = smem + wave * d;
+  float* qs = smem + wave * REP * d;
+  const int groups = nq / REP;               // head groups per token
   const int64_t wid = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + wave;
-  const bool live = wid < (int64_t)num_tokens * nq * num_splits;
-  int t = 0, h = 0, split = 0;
+  const bool live = wid < (int64_t)num_tokens * groups * num_splits;
+  int t = 0, h0 = 0, split = 0;
   if (live) {
-    const int64_t th = wid / num_splits;
-    split = (int)(wid - th * num_splits);
-    t = (int)(th / nq);
-    h = (int)(th - (int64_t)t * nq);
-    const T* qr = q + (int64_t)t * q_row_stride + (int64_t)h * d;
-    for (int e = lane; e < d; e += MI_WAVE) qs[e] = to_float(qr[e]);
+    const int64_t tg = wid / num_splits;
+    split = (int)(wid - tg * num_splits);
+    t = (int)(tg / groups);
+    h0 = (int)(tg - (int64_t)t * groups) * REP;
+    const T* qr = q + (int64_t)t * q_row_stride + (int64_t)h0 * d;
+    for (int e = lane; e < REP * d; e += MI_WAVE) qs[e] = to_float(qr[e]);
   }
   __syncthreads();
   if (!live) return;
@@ -80,101 +93,173 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   const int q_len = cu_q[b + 1] - q_begin;
   const int pos = kv_len[b] - q_len + (t - q_begin);
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int g = h / (nq / nkv);
+  const int g = h0 / (nq / nkv);
   const int P = 1 << page_shift;
   const int* bt = block_table + (int64_t)b * table_width;
 
-  // this wave's part of the tiles of lo .. pos (the first part is never empty)
+  // this wave's part of the tiles of lo .. pos: the tiles are shared out evenly, the parts differ by one tile at
+  // most (with fewer tiles than parts some parts are empty; they leave m = -inf, l = 0)
   const int tiles = (pos - lo) / MI_WAVE + 1;
-  const int tiles_per_split = (tiles + num_splits - 1) / num_splits;
-  const int j_begin = lo + split * tiles_per_split * MI_WAVE;
-  const int j_stop = (split + 1 == num_splits) ? pos + 1 : min(pos + 1, j_begin + tiles_per_split * MI_WAVE);
+  const int j_begin = lo + (int)((int64_t)split * tiles / num_splits) * MI_WAVE;
+  const int j_stop = (split + 1 == num_splits) ? pos + 1 : lo + (int)((int64_t)(split + 1) * tiles / num_splits) * MI_WAVE;
 
-  float m = -INFINITY, l = 0.f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float m[REP], l[REP], acc[REP][4];
+#pragma unroll
+  for (int x = 0; x < REP; ++x) {
+    m[x] = -INFINITY;
+    l[x] = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[x][c] = 0.f;
+  }
 
   for (int j0 = j_begin; j0 < j_stop; j0 += MI_WAVE) {
     const int j = j0 + lane;
-    float s = -INFINITY;
+    float s[REP], p[REP];
+#pragma unroll
+    for (int x = 0; x < REP; ++x) s[x] = -INFINITY;
     if (j <= pos) {
       const int64_t page = bt[j >> page_shift];
       const T* row = k_pages + ((page * nkv + g) * P + (j & (P - 1))) * d;
-      s = dot_row<T, VEC>(qs, row, d) * scale;
-    }
-    const float m_new = fmaxf(m, wave_max(s));   // the tile's first key is visible, so m_new is finite
-    const float p = (j <= pos) ? expf(s - m_new) : 0.f;
-    const float alpha = expf(m - m_new);         // 0 on the first tile (m = -inf)
-    l = l * alpha + wave_sum(p);
-    m = m_new;
+      dot_rows_any<REP>(qs, row, d, s);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] *= alpha;
+      for (int x = 0; x < REP; ++x) s[x] *= scale;
+    }
+#pragma unroll
+    for (int x = 0; x < REP; ++x) {
+      const float m_new = fmaxf(m[x], wave_max(s[x]));   // the tile's first key is visible, so m_new is finite
+      p[x] = (j <= pos) ? expf(s[x] - m_new) : 0.f;
+      const float alpha = expf(m[x] - m_new);            // 0 on the first tile (m = -inf)
+      l[x] = l[x] * alpha + wave_sum(p[x]);
+      m[x] = m_new;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[x][c] *= alpha;
+    }
+    // The tile's value rows, page by page: in the transposed pages [d][P] the keys of a page lie side by side for
+    // every dim, so a lane reads runs of 4 keys of its dims at once (where the page and the run allow it) and looks
+    // the page up once.  The products are added key by key in ascending order either way.
     const int n = (pos - j0 + 1 < MI_WAVE) ? pos - j0 + 1 : MI_WAVE;
-    for (int i = 0; i < n; ++i) {
-      const float pi = __shfl(p, i, MI_WAVE);
+    for (int i = 0; i < n;) {
       const int jj = j0 + i;
+      const int in_page = jj & (P - 1);
+      const int run = min(n - i, P - in_page);
       const int64_t page = bt[jj >> page_shift];
-      const T* vcol = v_pages + (page * nkv + g) * (int64_t)d * P + (jj & (P - 1));   // value pages are [d][P]
+      const T* vbase = v_pages + (page * nkv + g) * (int64_t)d * P + in_page;
+      for (int u = 0; u < run;) {
+        if (P >= 4 && ((in_page + u) & 3) == 0 && u + 4 <= run) {
+          float pk[REP][4];
+#pragma unroll
+          for (int x = 0; x < REP; ++x)
+#pragma unroll
+            for (int y = 0; y < 4; ++y) pk[x][y] = __shfl(p[x], i + u + y, MI_WAVE);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int e = lane + c * MI_WAVE;
+            if (e < d) {
+              float v4[4];
+              load4(vbase + (int64_t)e * P + u, v4);
+#pragma unroll
+              for (int x = 0; x < REP; ++x)
+#pragma unroll
+                for (int y = 0; y < 4; ++y) acc[x][c] = fmaf(pk[x][y], v4[y], acc[x][c]);
+            }
+          }
+          u += 4;
+        } else {
+          float pi[REP];
+#pragma unroll
+          for (int x = 0; x < REP; ++x) pi[x] = __shfl(p[x], i + u, MI_WAVE);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int e = lane + c * MI_WAVE;
+            if (e < d) {
+              const float vv = to_float(vbase[(int64_t)e * P + u]);
+#pragma unroll
+              for (int x = 0; x < REP; ++x) acc[x][c] = fmaf(pi[x], vv, acc[x][c]);
+            }
+          }
+          u += 1;
+        }
+      }
+      i += run;
+    }
+  }
+#pragma unroll
+  for (int x = 0; x < REP; ++x) {
+    const int h = h0 + x;
+    if (num_splits > 1) {
+      const int64_t item = ((int64_t)t * nq + h) * num_splits + split;
+      float* po = part_o + item * d;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const int e = lane + c * MI_WAVE;
-        if (e < d) acc[c] = fmaf(pi, to_float(vcol[(int64_t)e * P]), acc[c]);
+        if (e < d) po[e] = acc[x][c];
+      }
+      if (lane == 0) {
+        part_ml[item * 2] = m[x];
+        part_ml[item * 2 + 1] = l[x];
+      }
+    } else {
+      T* o = out + (int64_t)t * out_row_stride + (int64_t)h * d;
+      const float inv = 1.f / l[x];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int e = lane + c * MI_WAVE;
+        if (e < d) o[e] = from_float<T>(acc[x][c] * inv);
       }
     }
   }
-  if (num_splits > 1) {
-    float* po = part_o + wid * d;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int e = lane + c * MI_WAVE;
-      if (e < d) po[e] = acc[c];
-    }
-    if (lane == 0) {
-      part_ml[wid * 2] = m;
-      part_ml[wid * 2 + 1] = l;
-    }
-    return;
-  }
-  T* o = out + (int64_t)t * out_row_stride + (int64_t)h * d;
-  const float inv = 1.f / l;
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const int e = lane + c * MI_WAVE;
-    if (e < d) o[e] = from_float<T>(acc[c] * inv);
-  }
 }
 
-// One wave per (token, head): out = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s with M = max_s m_s.
-// An empty part has m = -inf and l = 0 and adds nothing; the first part is never empty, so M is finite.
+// One workgroup per (token, head): out = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s with M = max_s m_s.
+// An empty part has m = -inf and l = 0 and adds nothing; the last part is never empty, so M is finite.
+// The parts' weights are made once, by the lanes side by side, and kept in LDS; then thread (group, dim) adds the
+// parts group, group + G, ... of its dim (G = 256 / the head size rounded up to a power of two), whose loads do not
+// depend on one another, and the groups' sums are added in order.
+#define MERGE_THREADS 256
 template <typename T>
-__global__ __launch_bounds__(256) void paged_attention_merge_kernel(
+__global__ __launch_bounds__(MERGE_THREADS) void paged_attention_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, T* __restrict__ out, int64_t out_row_stride,
-    int num_tokens, int nq, int d, int num_splits) {
-  const int lane = threadIdx.x & (MI_WAVE - 1);
-  const int64_t th = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + threadIdx.x / MI_WAVE;
-  if (th >= (int64_t)num_tokens * nq) return;
+    int num_tokens, int nq, int d, int dpad, int num_splits) {
+  extern __shared__ float msm[];             // [num_splits] weights, [MERGE_THREADS] partial sums, [4] the waves' l
+  float* wts = msm;
+  float* red = msm + num_splits;
+  float* lsum = red + MERGE_THREADS;
+  const int tid = threadIdx.x, lane = tid & (MI_WAVE - 1), wave = tid / MI_WAVE;
+  const int64_t th = blockIdx.x;
   const float* ml = part_ml + th * num_splits * 2;
   float M = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, ml[2 * s]);
+  for (int s = tid; s < num_splits; s += MERGE_THREADS) M = fmaxf(M, ml[2 * s]);
+  M = wave_max(M);
+  if (lane == 0) lsum[wave] = M;
+  __syncthreads();
+  M = fmaxf(fmaxf(lsum[0], lsum[1]), fmaxf(lsum[2], lsum[3]));
+  __syncthreads();
   float l = 0.f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < num_splits; ++s) {
+  for (int s = tid; s < num_splits; s += MERGE_THREADS) {
     const float w = expf(ml[2 * s] - M);
+    wts[s] = w;
     l = fmaf(w, ml[2 * s + 1], l);
-    const float* po = part_o + (th * num_splits + s) * d;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int e = lane + c * MI_WAVE;
-      if (e < d) acc[c] = fmaf(w, po[e], acc[c]);
-    }
   }
-  const int t = (int)(th / nq);
-  const int h = (int)(th - (int64_t)t * nq);
-  T* o = out + (int64_t)t * out_row_stride + (int64_t)h * d;
-  const float inv = 1.f / l;
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const int e = lane + c * MI_WAVE;
-    if (e < d) o[e] = from_float<T>(acc[c] * inv);
+  l = wave_sum(l);
+  if (lane == 0) lsum[wave] = l;
+  __syncthreads();
+  l = (lsum[0] + lsum[1]) + (lsum[2] + lsum[3]);
+  const int G = MERGE_THREADS / dpad;
+  const int grp = tid / dpad, e = tid % dpad;
+  float acc = 0.f;
+  if (e < d) {
+    const float* po = part_o + th * num_splits * d + e;
+#pragma unroll 8
+    for (int s = grp; s < num_splits; s += G) acc = fmaf(wts[s], po[(int64_t)s * d], acc);
+  }
+  red[tid] = acc;
+  __syncthreads();
+  if (grp == 0 && e < d) {
+    float v = red[e];
+    for (int g2 = 1; g2 < G; ++g2) v += red[g2 * dpad + e];
+    const int t = (int)(th / nq);
+    const int h = (int)(th - (int64_t)t * nq);
+    out[(int64_t)t * out_row_stride + (int64_t)h * d + e] = from_float<T>(v / l);
   }
 }
 
@@ -198,31 +283,41 @@ MI_EXPORT int mi_paged_attention(int dtype, const void* q, int64_t q_row_stride,
   int shift = 0;
   while ((1 << shift) < page_size) ++shift;
   const int waves_per_block = 4;
-  const int64_t waves = (int64_t)num_tokens * nq * num_splits;
+  const int per_kv = nq / nkv;
+  const int rep = (per_kv == 2 || per_kv == 4 || per_kv == 8) ? per_kv : 1;
+  const int64_t waves = (int64_t)num_tokens * (nq / rep) * num_splits;
   MI_REQUIRE(waves / waves_per_block < (int64_t)INT32_MAX, "paged_attention: too many (token, head, part) items");
   const int blocks = (int)((waves + waves_per_block - 1) / waves_per_block);
-  const size_t lds = (size_t)waves_per_block * d * sizeof(float);
-  if (dtype == MI_DTYPE_F32)
-    paged_attention_kernel<float, 4><<<blocks, waves_per_block * MI_WAVE, lds, stream>>>(
-        (const float*)q, q_row_stride, (float*)out, out_row_stride, (const float*)k_pages, (const float*)v_pages,
-        block_table, table_width, token_req, cu_q, kv_len, num_tokens, nq, nkv, d, shift, scale, window, num_splits,
-        part_o, part_ml);
-  else if (dtype == MI_DTYPE_BF16)
-    paged_attention_kernel<bf16, 8><<<blocks, waves_per_block * MI_WAVE, lds, stream>>>(
-        (const bf16*)q, q_row_stride, (bf16*)out, out_row_stride, (const bf16*)k_pages, (const bf16*)v_pages,
-        block_table, table_width, token_req, cu_q, kv_len, num_tokens, nq, nkv, d, shift, scale, window, num_splits,
-        part_o, part_ml);
-  else
+  const size_t lds = (size_t)waves_per_block * rep * d * sizeof(float);
+#define ATTN_GO(T, REP)                                                                                              \
+  paged_attention_kernel<T, REP><<<blocks, waves_per_block * MI_WAVE, lds, stream>>>(                               \
+      (const T*)q, q_row_stride, (T*)out, out_row_stride, (const T*)k_pages, (const T*)v_pages, block_table,        \
+      table_width, token_req, cu_q, kv_len, num_tokens, nq, nkv, d, shift, scale, window, num_splits, part_o, part_ml)
+#define ATTN_REP(T)                                                                                                 \
+  if (rep == 8) ATTN_GO(T, 8);                                                                                      \
+  else if (rep == 4) ATTN_GO(T, 4);                                                                                 \
+  else if (rep == 2) ATTN_GO(T, 2);                                                                                 \
+  else ATTN_GO(T, 1)
+  if (dtype == MI_DTYPE_F32) {
+    ATTN_REP(float);
+  } else if (dtype == MI_DTYPE_BF16) {
+    ATTN_REP(bf16);
+  } else
     MI_FAIL("paged_attention: unknown dtype %d", dtype);
+#undef ATTN_REP
+#undef ATTN_GO
   MI_CHECK_LAUNCH("paged_attention");
   if (num_splits > 1) {
-    const int merge_blocks = (int)(((int64_t)num_tokens * nq + waves_per_block - 1) / waves_per_block);
+    int dpad = 8;
+    while (dpad < d) dpad *= 2;
+    const int merge_blocks = num_tokens * nq;
+    const size_t mlds = ((size_t)num_splits + MERGE_THREADS + 4) * sizeof(float);
     if (dtype == MI_DTYPE_F32)
-      paged_attention_merge_kernel<float><<<merge_blocks, waves_per_block * MI_WAVE, 0, stream>>>(
-          part_o, part_ml, (float*)out, out_row_stride, num_tokens, nq, d, num_splits);
+      paged_attention_merge_kernel<float><<<merge_blocks, MERGE_THREADS, mlds, stream>>>(
+          part_o, part_ml, (float*)out, out_row_stride, num_tokens, nq, d, dpad, num_splits);
     else
-      paged_attention_merge_kernel<bf16><<<merge_blocks, waves_per_block * MI_WAVE, 0, stream>>>(
-          part_o, part_ml, (bf16*)out, out_row_stride, num_tokens, nq, d, num_splits);
+      paged_attention_merge_kernel<bf16><<<merge_blocks, MERGE_THREADS, mlds, stream>>>(
+          part_o, part_ml, (bf16*)out, out_row_stride, num_tokens, nq, d, dpad, num_splits);
     MI_CHECK_LAUNCH("paged_attention_merge");
   }
   return 0;

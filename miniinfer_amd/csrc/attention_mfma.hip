@@ -1133,14 +1133,16 @@ MI_EXPORT int mi_attn_decode_static(const void* q, int64_t q_row_stride, void* o
                                     hipStream_t stream) {
   MI_REQUIRE(num_entries >= 0 && num_splits >= 1 && nq > 0, "attn_decode_static: bad entry range or splits");
   const int64_t need = (int64_t)num_entries * nq * num_splits;        // partials: D floats of output, 2 of (max, sum)
-  MI_REQUIRE(num_splits == 1 || need * (D + 2) <= (int64_t)MI_ATTN_STATIC_SCRATCH_FLOATS,
+  // part_o first, part_ml behind it on the next 64-byte boundary (need * D is a multiple of 16 floats as long as the
+  // head size is one; the rounding keeps the alignment whatever a later head size may be)
+  const int64_t ml_offset = (need * D + 15) / 16 * 16;
+  MI_REQUIRE(num_splits == 1 || ml_offset + 2 * need <= (int64_t)MI_ATTN_STATIC_SCRATCH_FLOATS,
              "attn_decode_static: %d entries x %d heads x %d splits need %lld floats of partial results; the static "
              "scratch holds %d (use fewer splits, or mi_attn_decode with a workspace of your own)",
-             num_entries, nq, num_splits, (long long)(need * (D + 2)), MI_ATTN_STATIC_SCRATCH_FLOATS);
+             num_entries, nq, num_splits, (long long)(ml_offset + 2 * need), MI_ATTN_STATIC_SCRATCH_FLOATS);
   float* base = nullptr;
   if (static_scratch(&base)) return 1;
-  // part_o first (need * D floats: a multiple of 16 floats, so part_ml behind it stays 64-byte aligned)
   return mi_attn_decode(q, q_row_stride, out, out_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len,
-                        first_entry, num_entries, num_splits, base, base + need * D, nq, nkv, page_size, scale, window,
+                        first_entry, num_entries, num_splits, base, base + ml_offset, nq, nkv, page_size, scale, window,
                         stream);
 }

@@ -1,13 +1,17 @@
 // C[M, N] = A[M, K] * W[N, K]^T  (x @ W^T, the linear layer of miniinfer/layers/linear.py:4-33)
 // with 32-bit FMA accumulation and no reduced-precision matrix instruction: this is the matrix
 // product of the true 32-bit path, and the any-shape fallback of the bfloat16 path.
-// The sum over K runs in one fixed order for every output element, whatever M is, so a row's
-// result does not depend on what else is in the batch.
+//
+// One order of summation for every result element, whatever M is and whichever kernel runs it: k is cut into
+// chunks of 64; a chunk's products are added by one chain of fused multiply-adds, k ascending, from zero; the
+// chunks' sums are added one after the other, first chunk first.  So a row's result does not depend on what else
+// is in the batch, bit for bit, and the chunks are what the kernel for few rows works on side by side.
 #include "common.h"
 
 #define BM 64
 #define BN 64
 #define BK 16
+#define CHUNK_K 64        // k per chunk of the order of summation (a multiple of BK)
 
 template <typename TA, typename TC>
 __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, int64_t lda,
@@ -23,11 +27,11 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
   const int lr = tid >> 2;        // 0..63: tile row this thread loads
   const int lk = (tid & 3) * 4;   // 0,4,8,12: first k it loads
 
-  float acc[4][4];
+  float acc[4][4], tot[4][4];     // the running chunk's chain, and the sum of the chunks before it
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = tot[i][j] = 0.f;
 
   for (int k0 = 0; k0 < K; k0 += BK) {
     {
@@ -53,6 +57,15 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
     }
+    if ((k0 + BK) % CHUNK_K == 0 || k0 + BK >= K) {      // a chunk ends here
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          tot[i][j] += acc[i][j];
+          acc[i][j] = 0.f;
+        }
+    }
     __syncthreads();
   }
 #pragma unroll
@@ -62,53 +75,170 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const TA* __restrict__ A, 
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
-      if (n < N) C[(int64_t)m * ldc + n] = from_float<TC>(acc[i][j]);
+      if (n < N) C[(int64_t)m * ldc + n] = from_float<TC>(tot[i][j]);
     }
   }
 }
 
-// The same product for up to 16 rows of A (a decode step of the 32-bit path), where the 64 x 64 tiles above would
-// leave the chip idle: a workgroup takes 16 rows of W and all rows of A, one result element per thread, chunks of
-// 64 k through LDS with the next chunk's loads in flight.  Every element is summed over k in the same order, with
-// the same fused multiply-adds, as in the kernel above: a row's result is bit for bit what it is there.
-#define FK 64
-template <typename TA, typename TC>
-__global__ __launch_bounds__(256) void gemm_nt_few_rows_kernel(const TA* __restrict__ A, int64_t lda,
-                                                               const TA* __restrict__ W, int64_t ldw,
-                                                               TC* __restrict__ C, int64_t ldc, int M, int N, int K) {
-  __shared__ float As[16][FK + 1];
-  __shared__ float Ws[16][FK + 1];
-  const int tid = threadIdx.x;
-  const int m = tid >> 4;          // the thread's row of A (and the row of A it loads)
-  const int nl = tid & 15;         // its row of W within the workgroup's 16
-  const int n0 = blockIdx.x * 16;
-  const int lk = (tid & 15) * 4;   // first k of the chunk that it loads: rows tid / 16 of A and of W
-  const bool a_ok = m < M, w_ok = n0 + m < N;
-  const TA* arow = A + (int64_t)(a_ok ? m : 0) * lda;
-  const TA* wrow = W + (int64_t)(w_ok ? n0 + m : 0) * ldw;
-  float ar[4], wr[4];
-#define FEW_FETCH(K0)                                                                          \
-  _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                              \
-    const int k = (K0) + lk + j;                                                               \
-    ar[j] = (a_ok && k < K) ? to_float(arow[k]) : 0.f;                                         \
-    wr[j] = (w_ok && k < K) ? to_float(wrow[k]) : 0.f;                                         \
-  }
-  FEW_FETCH(0)
-  float acc = 0.f;
-  for (int k0 = 0; k0 < K; k0 += FK) {
+// The same product for up to 16 rows of A (a decode step of the 32-bit path), where the time is the time to stream
+// W and the 64 x 64 tiles above would leave most of the chip idle.  A workgroup owns R rows of W (4, 8 or 16) and has
+// R x SCH threads: thread (r, c) takes chunk c of a block
+// of SCH chunks of row r, fetches its 64 weights itself (16 loads of 16 bytes, all on their way at once, no branch
+// between them), and multiplies them with that chunk of every row of A, which the workgroup has staged in LDS once
+// per block (a chunk's 64 values every 68 floats, so that the chunks' reads fall into different banks).  A thread's
+// MT chains (one per row of A) are the order of summation's chunk chains; the chunks' sums go through LDS to one
+// thread per result element, which adds them in order.  MT = 4, 8 or 16 rows of A are held; SCH = 16, 32 or 48 chunks
+// (1,024 to 3,072 k) a block, as many as k has where the staged rows fit LDS; VEC: k, the row strides and the bases allow 16-byte
+// accesses (else one element at a time).
+#define SPAD 68           // floats from one staged chunk of a row of A to the next
+
+// v = p[k .. k + 3], zeros where the row or k is outside; no branch: an address that is outside is replaced by the
+// row's first element, which is always there.
+template <typename TA, bool VEC>
+__device__ __forceinline__ void fetch4(const TA* p, int k, int K, bool row_ok, float (&v)[4]) {
+  if (VEC) {
+    const bool ok = row_ok && k < K;         // K is a multiple of 4 here
+    load4(p + (ok ? k : 0), v);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      As[m][lk + j] = ar[j];
-      Ws[m][lk + j] = wr[j];
+    for (int i = 0; i < 4; ++i) v[i] = ok ? v[i] : 0.f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = row_ok && k + i < K;
+      const float x = to_float(p[ok ? k + i : 0]);
+      v[i] = ok ? x : 0.f;
+    }
+  }
+}
+
+template <typename TA, typename TC, int MT, int SCH, bool VEC>
+__global__ __launch_bounds__(512) void gemm_nt_stream_kernel(const TA* __restrict__ A, int64_t lda,
+                                                             const TA* __restrict__ W, int64_t ldw,
+                                                             TC* __restrict__ C, int64_t ldc, int M, int N, int K,
+                                                             int R) {
+  extern __shared__ float lds[];
+  float* As = lds;                            // [MT][SCH][SPAD]
+  float* part = lds + MT * SCH * SPAD;        // [SCH][R][MT]: the chunks' sums of the running block
+  const int tid = threadIdx.x;
+  const int c = tid % SCH, r = tid / SCH;
+  const int n = blockIdx.x * R + r;
+  const bool n_ok = n < N;
+  const TA* wrow = W + (int64_t)(n_ok ? n : 0) * ldw;
+  // the result element that this thread finishes (threads 0 .. R * MT - 1)
+  static_assert(MT <= SCH, "R * MT result elements over R * SCH threads");
+  const int fr = tid / MT, fm = tid % MT;
+  const bool finisher = tid < R * MT;
+  float tot = 0.f;
+  for (int kb = 0; kb < K; kb += SCH * CHUNK_K) {
+    // this thread's weights of the block: all loads on their way before anything waits
+    float wv[CHUNK_K / 4][4];
+#pragma unroll
+    for (int q = 0; q < CHUNK_K / 4; ++q) fetch4<TA, VEC>(wrow, kb + c * CHUNK_K + 4 * q, K, n_ok, wv[q]);
+    // the block of A into LDS, rows beyond M as zeros: 8 loads of 16 bytes of a thread on their way at a time
+    constexpr int ITEMS = MT * SCH * (CHUNK_K / 4);
+    for (int base = tid; base < ITEMS; base += 8 * blockDim.x) {
+      float v[8][4];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int idx = base + u * blockDim.x;
+        const int idc = idx < ITEMS ? idx : 0;
+        const int m = idc / (SCH * (CHUNK_K / 4)), q = idc % (SCH * (CHUNK_K / 4));
+        fetch4<TA, VEC>(A + (int64_t)(m < M ? m : 0) * lda, kb + 4 * q, K, m < M, v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int idx = base + u * blockDim.x;
+        if (idx < ITEMS) {
+          const int m = idx / (SCH * (CHUNK_K / 4)), q = idx % (SCH * (CHUNK_K / 4));
+          store4(As + (m * SCH + q / (CHUNK_K / 4)) * SPAD + 4 * (q % (CHUNK_K / 4)), v[u]);
+        }
+      }
     }
     __syncthreads();
-    if (k0 + FK < K) FEW_FETCH(k0 + FK)
+    float acc[MT];
 #pragma unroll
-    for (int kk = 0; kk < FK; ++kk) acc = fmaf(As[m][kk], Ws[nl][kk], acc);
+    for (int m = 0; m < MT; ++m) acc[m] = 0.f;
+#pragma unroll
+    for (int q = 0; q < CHUNK_K / 4; ++q) {
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        float a[4];
+        load4(As + (m * SCH + c) * SPAD + 4 * q, a);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[m] = fmaf(a[i], wv[q][i], acc[m]);
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) part[(c * R + r) * MT + m] = acc[m];
     __syncthreads();
+    if (finisher) {
+      const int chunks = min(SCH, (K - kb + CHUNK_K - 1) / CHUNK_K);
+      for (int cc = 0; cc < chunks; ++cc) tot += part[(cc * R + fr) * MT + fm];
+    }
+    // (the next block's first barrier keeps its writes to `part` behind these reads)
   }
-#undef FEW_FETCH
-  if (m < M && n0 + nl < N) C[(int64_t)m * ldc + n0 + nl] = from_float<TC>(acc);
+  const int fn = blockIdx.x * R + fr;
+  if (finisher && fm < M && fn < N) C[(int64_t)fm * ldc + fn] = from_float<TC>(tot);
+}
+
+static int gemm_compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+  }
+  return cus;
+}
+
+template <typename TA, typename TC, int MT, int SCH, bool VEC>
+static int launch_stream_instance(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
+                                  int N, int K, int R, hipStream_t stream) {
+  const size_t lds = ((size_t)MT * SCH * SPAD + (size_t)SCH * R * MT) * sizeof(float);
+  static bool raised = false;       // per instantiation: more dynamic LDS than the default allotment
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_stream_kernel<TA, TC, MT, SCH, VEC>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    MI_REQUIRE(e == hipSuccess, "gemm_nt: cannot raise the LDS allotment: %s", hipGetErrorString(e));
+    raised = true;
+  }
+  gemm_nt_stream_kernel<TA, TC, MT, SCH, VEC><<<ceil_div(N, R), R * SCH, lds, stream>>>(
+      (const TA*)A, lda, (const TA*)W, ldw, (TC*)C, ldc, M, N, K, R);
+  return 0;
+}
+
+template <typename TA, typename TC>
+static int launch_stream(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
+                         hipStream_t stream) {
+  // Chunks a workgroup works on side by side: all of k at once where the staged rows of A fit LDS (every load of the
+  // product is then on its way together, which is what its time comes to when W is small), in steps of 16 chunks.
+  // Rows of W per workgroup: 16 where that still makes a workgroup for every compute unit, else 8 where that makes
+  // one for every other unit, else 4 (every workgroup stages the rows of A once, so more rows mean fewer reads of
+  // A; what fills the machine is the bytes on their way, 256 of them a thread), and never more than 512 threads.
+  const int cus = gemm_compute_units();
+  const int mt = M <= 4 ? 4 : (M <= 8 ? 8 : 16);
+  const int chunks = ceil_div(K, CHUNK_K);
+  int sch = chunks <= 16 ? 16 : (chunks <= 32 || mt == 16 ? 32 : 48);
+  int R = N / 16 >= cus ? 16 : (N / 8 >= cus / 2 ? 8 : 4);
+  while (R > 1 && (R * sch > 512 || ((size_t)mt * sch * SPAD + (size_t)sch * R * mt) * sizeof(float) > 160 * 1024)) R /= 2;
+  const bool vec = K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0;
+#define GO(MT, SCH)                                                                                                  \
+  return vec ? launch_stream_instance<TA, TC, MT, SCH, true>(A, lda, W, ldw, C, ldc, M, N, K, R, stream)            \
+             : launch_stream_instance<TA, TC, MT, SCH, false>(A, lda, W, ldw, C, ldc, M, N, K, R, stream)
+  if (mt == 4) {
+    if (sch == 16) GO(4, 16);
+    if (sch == 32) GO(4, 32);
+    GO(4, 48);
+  }
+  if (mt == 8) {
+    if (sch == 16) GO(8, 16);
+    if (sch == 32) GO(8, 32);
+    GO(8, 48);
+  }
+  if (sch == 16) GO(16, 16);
+  GO(16, 32);
+#undef GO
 }
 
 // in_dtype: dtype of A and W; out_dtype: dtype of C.
@@ -119,13 +249,13 @@ MI_EXPORT int mi_gemm_nt(int in_dtype, int out_dtype, const void* A, int64_t lda
              (long long)lda, (long long)ldw, (long long)ldc, K, N);
   if (M == 0) return 0;
   const bool few = M <= 16;
-  dim3 grid(few ? ceil_div(N, 16) : ceil_div(N, BN), few ? 1 : ceil_div(M, BM));
+  dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
   MI_REQUIRE(grid.y <= 65535, "gemm_nt: M=%d too large for one launch", M);
 #define LAUNCH(TA, TC)                                                                                              \
-  if (few)                                                                                                          \
-    gemm_nt_few_rows_kernel<TA, TC><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TA*)W, ldw, (TC*)C, ldc, M, \
-                                                              N, K);                                               \
-  else                                                                                                              \
+  if (few) {                                                                                                        \
+    const int rc = launch_stream<TA, TC>(A, lda, W, ldw, C, ldc, M, N, K, stream);                                  \
+    if (rc) return rc;                                                                                              \
+  } else                                                                                                            \
     gemm_nt_kernel<TA, TC><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TA*)W, ldw, (TC*)C, ldc, M, N, K)
   if (in_dtype == MI_DTYPE_F32 && out_dtype == MI_DTYPE_F32) {
     LAUNCH(float, float);

@@ -125,7 +125,9 @@ class PagedAttention(Part):
     table = ctx.block_tables[cache.group]
     if not ops.mfma_attention_supported(qkv.dtype, nq, nkv, d, cache.page_size):
       T = qkv.shape[0]
-      splits = plain_splits(T * nq, min(ctx.max_kv_len, window) if window else ctx.max_kv_len,
+      per_kv = nq // nkv
+      waves = T * (nkv if per_kv in (2, 4, 8) else nq)      # the kernel takes such a group's heads in one wave
+      splits = plain_splits(waves, min(ctx.max_kv_len, window) if window else ctx.max_kv_len,
                             16 * ops.compute_units())
       part_o = part_ml = None
       if splits > 1:
@@ -181,13 +183,14 @@ def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, wav
   return int(max(1, min(want, max(1, tiles // waves), 32)))
 
 
-def plain_splits(num_head_tokens: int, max_keys: int, resident_waves: int = 4096) -> int:
-  """Into how many key ranges the one-wave-per-(token, head) kernel cuts each token's keys: as many as fill the
-  chip's wave slots (16 on each compute unit; the default is an MI355X's 16 x 256) once, each range at least two tiles of 64 keys, at most 64
-  ranges.  Prompt portions have waves enough and stay whole."""
-  want = resident_waves // max(1, num_head_tokens)
+def plain_splits(num_waves: int, max_keys: int, resident_waves: int = 4096) -> int:
+  """Into how many key ranges the plain kernel (one wave per token and group of query heads) cuts each token's keys:
+  as many as fill the chip's wave slots (16 on each compute unit; the default is an MI355X's 16 x 256) once, each
+  range at least one tile of 64 keys, at most 64 ranges: a wave takes its tiles one after the other, so few tokens
+  over many keys are as quick as their longest range.  Prompt portions have waves enough and stay whole."""
+  want = resident_waves // max(1, num_waves)
   tiles = -(-max_keys // 64)
-  return int(max(1, min(want, tiles // 2, 64)))
+  return int(max(1, min(want, tiles, 64)))
 
 
 register_mixer("paged_attention", PagedAttention)

@@ -196,8 +196,8 @@ def test_plain_attention_key_ranges():
   over many keys, never shorter than two tiles, never more than 64."""
   from miniinfer_amd.parts.attention import plain_splits
   assert plain_splits(2048 * 16, 2048) == 1
-  assert plain_splits(8 * 16, 100) == 1
-  assert plain_splits(8 * 16, 2048) == 16
-  assert plain_splits(1, 700) == 5
+  assert plain_splits(8 * 16, 100) == 2
+  assert plain_splits(8 * 16, 2048) == 32 and plain_splits(8 * 8, 2048) == 32
+  assert plain_splits(1, 700) == 11
   assert plain_splits(1, 1 << 20) == 64
   assert plain_splits(4096, 1 << 20) == 1
