@@ -931,6 +931,84 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
   }
 }
 
+// The same for more than 32 splits (one long request: the key ranges then outnumber what a wave's loads cover at
+// once): a workgroup of 4 waves per (entry, head).  The threads share out the splits for the maximum and the weights,
+// which are kept in LDS; then thread (group, 4 dims) adds the splits group, group + G, ... of its dims, whose loads do
+// not depend on one another, and the groups' sums are added in order.
+__global__ __launch_bounds__(256) void decode_merge_many_kernel(const float* __restrict__ part_o,
+                                                               const float* __restrict__ part_ml,
+                                                               uint16_t* __restrict__ out, int64_t out_row_stride,
+                                                               const int* __restrict__ cu_q, int first_entry, int nq,
+                                                               int num_splits) {
+  __shared__ float wts[1024];
+  __shared__ float red4[4];
+  __shared__ f32x4 accs[256];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int e = blockIdx.x / nq, head = blockIdx.x % nq;
+  const int64_t base = ((int64_t)e * nq + head) * num_splits;
+  float M = -INFINITY;
+  for (int s = tid; s < num_splits; s += 256) M = fmaxf(M, part_ml[(base + s) * 2]);
+  M = wave_max(M);
+  if (lane == 0) red4[wave] = M;
+  __syncthreads();
+  M = fmaxf(fmaxf(red4[0], red4[1]), fmaxf(red4[2], red4[3]));
+  __syncthreads();
+  float L = 0.f;
+  for (int s = tid; s < num_splits; s += 256) {
+    const float2 ml = *reinterpret_cast<const float2*>(part_ml + (base + s) * 2);
+    const float w = ml.x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml.x - M);
+    wts[s] = w;
+    L += w * ml.y;
+  }
+  L = wave_sum(L);
+  if (lane == 0) red4[wave] = L;
+  __syncthreads();
+  L = (red4[0] + red4[1]) + (red4[2] + red4[3]);
+  constexpr int DL = D / 4 <= 4 ? 4 : (D / 4 <= 8 ? 8 : (D / 4 <= 16 ? 16 : (D / 4 <= 32 ? 32 : 64)));
+  constexpr int G = 256 / DL;
+  const int grp = tid / DL, dl = tid % DL;
+  const bool live = 4 * dl < D;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    const float* po = part_o + base * D + 4 * dl;
+#pragma unroll 8
+    for (int s = grp; s < num_splits; s += G) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(po + (int64_t)s * D);
+      const float w = wts[s];
+      acc[0] += w * v[0];
+      acc[1] += w * v[1];
+      acc[2] += w * v[2];
+      acc[3] += w * v[3];
+    }
+  }
+  accs[tid] = acc;
+  __syncthreads();
+  if (grp == 0 && live) {
+    f32x4 t = accs[dl];
+    for (int g2 = 1; g2 < G; ++g2) {
+      const f32x4 v = accs[g2 * DL + dl];
+      t[0] += v[0];
+      t[1] += v[1];
+      t[2] += v[2];
+      t[3] += v[3];
+    }
+    const float inv = 1.f / L;
+    uint16_t* o = out + (int64_t)cu_q[first_entry + e] * out_row_stride + (int64_t)head * D;
+    *reinterpret_cast<s16x4*>(o + 4 * dl) = pack_bf16x4(t[0] * inv, t[1] * inv, t[2] * inv, t[3] * inv);
+  }
+}
+
+static void launch_decode_merge(const float* part_o, const float* part_ml, uint16_t* out, int64_t out_row_stride,
+                                const int* cu_q, int first_entry, int num_entries, int nq, int num_splits,
+                                hipStream_t stream) {
+  if (num_splits > 32)
+    decode_merge_many_kernel<<<num_entries * nq, 256, 0, stream>>>(part_o, part_ml, out, out_row_stride, cu_q,
+                                                                  first_entry, nq, num_splits);
+  else
+    decode_merge_kernel<<<num_entries * nq, 64, 0, stream>>>(part_o, part_ml, out, out_row_stride, cu_q, first_entry,
+                                                             nq, num_splits);
+}
+
 // ---------------------------------------------------------------- entry points
 static int check_common(const char* what, int nq, int nkv, int page_size, int64_t q_row_stride, int64_t out_row_stride,
                         int table_width) {
@@ -1050,8 +1128,8 @@ MI_EXPORT int mi_attn_decode(const void* q, int64_t q_row_stride, void* out, int
       log2_of(page_size), scale, window, DecodeFront{});
   MI_CHECK_LAUNCH("attn_decode");
   if (num_splits > 1) {
-    decode_merge_kernel<<<num_entries * nq, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q,
-                                                             first_entry, nq, num_splits);
+    launch_decode_merge(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q, first_entry, num_entries, nq, num_splits,
+                        stream);
     MI_CHECK_LAUNCH("attn_decode merge");
   }
   return 0;
@@ -1089,8 +1167,8 @@ MI_EXPORT int mi_attn_decode_front(const void* qkv, int64_t qkv_row_stride, void
       log2_of(page_size), scale, window, front);
   MI_CHECK_LAUNCH("attn_decode_front");
   if (num_splits > 1) {
-    decode_merge_kernel<<<num_entries * nq, 64, 0, stream>>>(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q,
-                                                             first_entry, nq, num_splits);
+    launch_decode_merge(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q, first_entry, num_entries, nq, num_splits,
+                        stream);
     MI_CHECK_LAUNCH("attn_decode_front merge");
   }
   return 0;

@@ -49,6 +49,7 @@ struct NormHalves {
   const float* norm_weight; // [N]
   uint16_t* a_out;          // [M, N] bfloat16, leading dimension N
   float* ss_out;            // [gridDim.x][SS_ROW(M)]
+  int ss_stride;            // floats from one part's row of row_ss / ss_out to the next: SS_ROW(M)
 };
 
 // MODE 0 takes every shape.  MODES 1 to 5 are the same product for K a multiple of 32 and operands below 4 GB: the
@@ -71,6 +72,13 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
                                                            void* __restrict__ C, int64_t ldc, int M, int N, int K,
                                                            int rpg, NormHalves nh) {
   extern __shared__ float red[];   // [(waves + 1) / 2][RB * MB][256], then (norm halves) [OB * 256] squares, [waves][64] sums
+  // A launch whose grid has a second dimension shares out the rows of A as well: workgroup (x, y) takes rows
+  // 16 MB y .. of A (and of the result) against its rows of W, so that few rows of W still make workgroups enough;
+  // the workgroups of one x read the same rows of W, and they are neighbours modulo 8 in launch order whenever the
+  // grid's first dimension is a multiple of 8, that is on one XCD, whose L2 then holds those rows.
+  const int m_base = 16 * MB * blockIdx.y;
+  A += (int64_t)m_base * lda;
+  M = min(M - m_base, 16 * MB);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in every lane: said so
   const int nw = blockDim.x >> 6;
@@ -131,7 +139,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       for (int p = tid / SS; p < nh.ss_parts; p += 4 * stride) {                                                     \
         float v[4];                                                                                                  \
         _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                                \
-          v[j] = p + j * stride < nh.ss_parts ? nh.row_ss[(int64_t)(p + j * stride) * SS + m] : 0.f;                 \
+          v[j] = p + j * stride < nh.ss_parts ? nh.row_ss[(int64_t)(p + j * stride) * nh.ss_stride + m_base + m] : 0.f; \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) my_ss += v[j];                                                 \
       }                                                                                                              \
     }                                                                                                                \
@@ -143,7 +151,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         const int n = n0 + rpg * (blk / MB) + r;                                                                     \
         const int m = 16 * (blk % MB) + (ln & 15);                                                                   \
         if (e < OBLK * 256 && r < rpg && n < n_end && m < M) {                                                       \
-          r_pre[j] = nh.residual[(int64_t)m * N + n];                                                                \
+          r_pre[j] = nh.residual[(int64_t)(m_base + m) * N + n];                                                     \
           w_pre[j] = nh.norm_weight[n];                                                                              \
         }                                                                                                            \
       }                                                                                                              \
@@ -461,16 +469,16 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       float rv = 0.f;
       if (live) {
         const int j = (e - (int)threadIdx.x) / (int)blockDim.x;
-        const float r_old = j == 0 ? r_pre[0] : (j == 1 ? r_pre[1] : nh.residual[(int64_t)m * N + n]);
+        const float r_old = j == 0 ? r_pre[0] : (j == 1 ? r_pre[1] : nh.residual[(int64_t)(m_base + m) * N + n]);
         const float w_n = j == 0 ? w_pre[0] : (j == 1 ? w_pre[1] : nh.norm_weight[n]);
         rv = r_old + v;
-        nh.residual[(int64_t)m * N + n] = rv;
-        nh.a_out[(int64_t)m * N + n] = float_to_bf16_bits(rv * w_n);
+        nh.residual[(int64_t)(m_base + m) * N + n] = rv;
+        nh.a_out[(int64_t)(m_base + m) * N + n] = float_to_bf16_bits(rv * w_n);
       }
       sq[e] = rv * rv;
     } else if (live) {
-      if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n] = v;
-      else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n] = float_to_bf16_bits(v);
+      if (OUT_F32) reinterpret_cast<float*>(C)[(int64_t)(m_base + m) * ldc + n] = v;
+      else reinterpret_cast<uint16_t*>(C)[(int64_t)(m_base + m) * ldc + n] = float_to_bf16_bits(v);
     }
   }
   if (nh.residual) {
@@ -481,7 +489,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       for (int rb = 0; rb < (GATE_UP ? 1 : RB); ++rb)
         for (int q = 0; q < 4; ++q)
           for (int i = 0; i < 4; ++i) total += sq[(rb * MB + (m >> 4)) * 256 + 4 * ((m & 15) + 16 * q) + i];
-      nh.ss_out[(int64_t)blockIdx.x * SS + m] = total;
+      nh.ss_out[(int64_t)blockIdx.x * nh.ss_stride + m_base + m] = total;
     }
   }
 }
@@ -749,11 +757,13 @@ static void launch_instance(dim3 grid, dim3 block, size_t lds, hipStream_t strea
 
 template <int MB, int RB>
 static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
-                  int64_t ldc, int M, int N, int K, int waves, const SkinnyGrid& sg, const NormHalves& nh,
-                  int want, hipStream_t stream) {
-  const dim3 grid(sg.groups);
+                  int64_t ldc, int M_all, int N, int K, int waves, const SkinnyGrid& sg, const NormHalves& nh,
+                  int want, int grid_y, hipStream_t stream) {
+  // grid_y > 1: the rows of A are shared out too, 16 MB to a workgroup (the kernel takes its share of M_all)
+  const dim3 grid(sg.groups, grid_y);
+  const int M = grid_y > 1 ? 16 * MB : M_all;        // rows of A a workgroup stages
   const int64_t w_rows = gate_up ? 2 * (int64_t)N : N;
-  const bool lean = K % 32 == 0 && w_rows * ldw * 2 < ((int64_t)1 << 32) && (int64_t)M * lda * 2 < ((int64_t)1 << 32) &&
+  const bool lean = K % 32 == 0 && w_rows * ldw * 2 < ((int64_t)1 << 32) && (int64_t)M_all * lda * 2 < ((int64_t)1 << 32) &&
                     (((uintptr_t)A | (uintptr_t)W) & 15) == 0;
   // want: the kernel's mode the caller asks for (1 .. 5); it is taken as far as the shape allows
   int mode = 0;
@@ -774,12 +784,12 @@ static int launch(bool out_f32, bool gate_up, const void* A, int64_t lda, const 
   {                                                                                                                  \
     if (mode == 5) {                                                                                                 \
       if constexpr (MB == 1)                                                                                         \
-        launch_instance<MB, RB, F32, GU, 5>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh);  \
-    } else if (mode == 4) launch_instance<MB, RB, F32, GU, 4>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
-    else if (mode == 3) launch_instance<MB, RB, F32, GU, 3>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
-    else if (mode == 2) launch_instance<MB, RB, F32, GU, 2>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
-    else if (mode == 1) launch_instance<MB, RB, F32, GU, 1>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh); \
-    else launch_instance<MB, RB, F32, GU, 0>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, sg.rpg, nh);  \
+        launch_instance<MB, RB, F32, GU, 5>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M_all, N, K, sg.rpg, nh);  \
+    } else if (mode == 4) launch_instance<MB, RB, F32, GU, 4>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M_all, N, K, sg.rpg, nh); \
+    else if (mode == 3) launch_instance<MB, RB, F32, GU, 3>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M_all, N, K, sg.rpg, nh); \
+    else if (mode == 2) launch_instance<MB, RB, F32, GU, 2>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M_all, N, K, sg.rpg, nh); \
+    else if (mode == 1) launch_instance<MB, RB, F32, GU, 1>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M_all, N, K, sg.rpg, nh); \
+    else launch_instance<MB, RB, F32, GU, 0>(grid, block, lds, stream, A, lda, W, ldw, C, ldc, M_all, N, K, sg.rpg, nh);  \
   }
   if (gate_up) {
     if constexpr (RB == 2) {
@@ -834,10 +844,21 @@ static int skinny_rows(int out_f32, int gate_up, const void* A, int64_t lda, con
   const int steps = (K + 31) / 32;
   const int MB = (M + 15) / 16;
   const int waves = skinny_waves(groups, steps, RB, MB, gate_up != 0);
-  const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
+  const NormHalves nh{row_ss, ss_parts, eps, residual, norm_weight, (uint16_t*)a_out, ss_out, SS_ROW(M)};
+  if (want == 6 && M > 16) {
+    // the rows of A shared out as well: blocks of 16 rows along the grid's second dimension, every workgroup the
+    // kernel for up to 16 rows with both operands staged (or what of that the shape allows)
+    const int gy = MB;
+    const int w6 = skinny_waves(groups * gy, steps, RB, 1, gate_up != 0);
+    if (RB == 1) launch<1, 1>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, w6, sg, nh, 5, gy, stream);
+    else launch<1, 2>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, w6, sg, nh, 5, gy, stream);
+    MI_CHECK_LAUNCH("gemm_skinny");
+    return 0;
+  }
+  if (want == 6) want = 5;
 #define CASE(mb, rb)                                                                                          \
   if (MB == mb && RB == rb) {                                                                                 \
-    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, want, stream);    \
+    launch<mb, rb>(out_f32 != 0, gate_up != 0, A, lda, W, ldw, C, ldc, M, N, K, waves, sg, nh, want, 1, stream); \
     MI_CHECK_LAUNCH("gemm_skinny");                                                                           \
     return 0;                                                                                                 \
   }
@@ -1129,7 +1150,7 @@ static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
 // is the first half of a norm (`ss_parts`), and the floats of scratch it needs (0 for every variant but 1).
 MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K, int* ss_parts, int64_t* scratch_floats) {
   MI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_plan: M=%d N=%d K=%d", M, N, K);
-  MI_REQUIRE(variant >= 0 && variant <= 5, "gemm_skinny_plan: variant %d", variant);
+  MI_REQUIRE(variant >= 0 && variant <= 6, "gemm_skinny_plan: variant %d", variant);
   if (variant != 1) {
     if (ss_parts) *ss_parts = skinny_grid(gate_up != 0, N, M).groups;
     if (scratch_floats) *scratch_floats = 0;
@@ -1146,13 +1167,14 @@ MI_EXPORT int mi_gemm_skinny_plan(int variant, int gate_up, int M, int N, int K,
 // added in the order of the splits by a second kernel that also does the endings; variant 2 = variant 0 with the left
 // operand staged through LDS; variants 3 and 4 = variants 0 and 2 with the weights fetched in whole memory lines;
 // variant 5 = both operands staged through LDS, for up to 16 rows (each where the shape allows it; else the nearest
-// that it does).  Variants 0, 2 and 5 add the same products in the same order: their results are equal bit for
-// bit, and so are those of 3 and 4.
+// that it does); variant 6 = for more than 16 rows, the rows of A shared out across workgroups as well, 16 to each,
+// every workgroup as in variant 5 (for up to 16 rows it is variant 5).  Variants 0, 2 and 5 add the same products in
+// the same order: their results are equal bit for bit, and so are those of 3 and 4.
 MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void* A, int64_t lda, const void* W,
                                int64_t ldw, void* C, int64_t ldc, int M, int N, int K, const float* row_ss,
                                int ss_parts, float eps, float* residual, const float* norm_weight, void* a_out,
                                float* ss_out, float* scratch, int64_t scratch_floats, hipStream_t stream) {
-  if (variant != 1 && variant >= 0 && variant <= 5)
+  if (variant != 1 && variant >= 0 && variant <= 6)
     return skinny_rows(out_f32, gate_up, A, lda, W, ldw, C, ldc, M, N, K, row_ss, ss_parts, eps, residual, norm_weight,
                        a_out, ss_out, variant == 0 ? 1 : variant, stream);
   MI_REQUIRE(variant == 1, "gemm_skinny: variant %d", variant);

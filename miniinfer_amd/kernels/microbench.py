@@ -59,6 +59,10 @@ def cmd_product(args) -> int:
     ops.gemm_skinny(a, ws[turn[0] % copies], out, gate_up=args.gate_up, variant=5)
     turn[0] += 1
 
+  def ours_rows_shared_out():
+    ops.gemm_skinny(a, ws[turn[0] % copies], out, gate_up=args.gate_up, variant=6)
+    turn[0] += 1
+
   def library():
     torch.matmul(a, ws[turn[0] % copies].t())
     turn[0] += 1
@@ -67,7 +71,9 @@ def cmd_product(args) -> int:
   for name, fn in (("gemm_skinny", ours), ("gemm_skinny with the left operand staged", ours_staged),
                    ("gemm_skinny with the left operand staged and the weights in whole lines", ours_staged_lines),
                    ("gemm_skinny with both operands staged", ours_both_staged),
-                   ("gemm_skinny with k split", ours_ksplit), ("library", library)):
+                   ("gemm_skinny with k split", ours_ksplit),
+                   ("gemm_skinny with the rows of the left operand shared out", ours_rows_shared_out),
+                   ("library", library)):
     t = graph_time_us(fn, calls)
     print(f"{name}: rows {args.rows}, weights [{rows_w}, {args.k}] {nbytes / 1e6:.1f} MB: {t:.1f} us, "
           f"{nbytes / t / 1e6:.2f} TB/s" + (" (without the activation)" if name == "library" and args.gate_up else ""))

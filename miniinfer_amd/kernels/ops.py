@@ -358,9 +358,11 @@ TUNE_ROWS = (1, 4, 8, 16, 32, 48, 64)   # row counts at which `tuning.tune_produ
 # (rows point, matrix rows, k, gate|up) -> the quickest: LIBRARY, or this library's kernel in which every workgroup
 # owns whole rows of the result (OWN_ROWS; OWN_ROWS_STAGED: with the left operand staged through LDS; OWN_ROWS_LINES,
 # OWN_ROWS_STAGED_LINES: the same two with the weights fetched in whole memory lines; OWN_ROWS_BOTH_STAGED: both
-# operands through LDS, for up to 16 rows), or the one that splits k across workgroups (OWN_KSPLIT).  An own kernel's
-# choice is its variant number + 1.
-LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES, OWN_ROWS_BOTH_STAGED = range(7)
+# operands through LDS, for up to 16 rows; OWN_ROWS_SHARED_OUT: for more than 16 rows, the rows of the left operand
+# shared out across workgroups too, 16 to each, both operands staged), or the one that splits k across workgroups
+# (OWN_KSPLIT).  An own kernel's choice is its variant number + 1.
+(LIBRARY, OWN_ROWS, OWN_KSPLIT, OWN_ROWS_STAGED, OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES, OWN_ROWS_BOTH_STAGED,
+ OWN_ROWS_SHARED_OUT) = range(8)
 BOTH_STAGED_MAX_ROWS = 16
 BOTH_STAGED_ANY_ELEMENTS = 16 << 20  # without a measurement: both operands are staged for matrices of this size,
 BOTH_STAGED_MIN_K = 2048             # or with rows of at least this many columns where no activation follows
@@ -415,6 +417,8 @@ class ProductChoices:
       if self.force == OWN_KSPLIT and not can_split:
         return OWN_ROWS
       if self.force == OWN_ROWS_BOTH_STAGED and not (num_rows <= BOTH_STAGED_MAX_ROWS and k % 32 == 0):
+        return OWN_ROWS
+      if self.force == OWN_ROWS_SHARED_OUT and k % 32:
         return OWN_ROWS
       if self.force in (OWN_ROWS_LINES, OWN_ROWS_STAGED_LINES) and k % 64:
         return OWN_ROWS
@@ -557,7 +561,8 @@ def skinny_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fals
   whole memory lines too (two steps of k at a time, put in place by an exchange between lanes: large matrices
   stream faster that way); 5 = both operands staged through LDS, every request for whole lines (up to 16 rows;
   the same sums as 0 bit for bit); 1 = k is split across workgroups, which read a slice of the left operand each and
-  leave 32-bit partial results that a second kernel adds in a fixed order.
+  leave 32-bit partial results that a second kernel adds in a fixed order; 6 = for more than 16 rows, the rows of the
+  left operand are shared out across workgroups too, 16 to each (see `shared_out_offered`).
   Measured where `tuning.tune_products` has been; else by rule."""
   c = _measured_choice(num_rows, matrix_rows, k, gate_up)
   can_split = not (gate_up and (matrix_rows // 2) % 4)
@@ -566,8 +571,27 @@ def skinny_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool = Fals
   return _rule_variant(num_rows, matrix_rows, k, gate_up)
 
 
+SHARED_OUT_MAX_WORKGROUPS_PER_UNIT = 1.5   # without a measurement: the rows of the left operand are shared out while
+                                           # (row blocks of the matrix) x (blocks of 16 rows) stay within this
+
+
+def shared_out_offered(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> bool:
+  """Whether the form that shares out the rows of the left operand too is a candidate: more than 16 rows, and so few
+  rows of the matrix that whole blocks of 16 of them leave compute units idle (a [1024, 2048] matrix at 64 rows: 64
+  workgroups otherwise; 5.0 us this way against 7.9 with the left operand staged, 8.4 with k split and 8.3 in the
+  library; [1024, 3072]: 5.9 against 10.4, 9.5 and 10.0).  Every workgroup reads its rows of the matrix once per
+  block of 16 rows, out of its XCD's L2, so matrices of many rows gain nothing ([4096, 1024] at 64 rows: 6.5 against
+  6.4) and a gate|up matrix loses (9.8 against 7.9)."""
+  if num_rows <= 16 or k % 32 or gate_up:
+    return False
+  groups = -(-matrix_rows // 16) * -(-num_rows // 16)
+  return groups <= SHARED_OUT_MAX_WORKGROUPS_PER_UNIT * compute_units()
+
+
 def _rule_variant(num_rows: int, matrix_rows: int, k: int, gate_up: bool) -> int:
   can_split = not (gate_up and (matrix_rows // 2) % 4)
+  if shared_out_offered(num_rows, matrix_rows, k, gate_up):
+    return 6
   if can_split and num_rows >= KSPLIT_MIN_ROWS and k >= KSPLIT_MIN_K:
     return 1
   large = matrix_rows * k >= LINES_MIN_ELEMENTS

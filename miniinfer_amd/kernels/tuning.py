@@ -110,6 +110,8 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
         forms[c] = graph_time_us(own(c - 1), calls, flush)
       if ops.both_staged_offered(M, rows_w, K, gate_up):
         forms[ops.OWN_ROWS_BOTH_STAGED] = graph_time_us(own(5), calls, flush)
+      if M > 16 and K % 32 == 0 and not gate_up and -(-rows_w // 16) * -(-M // 16) <= 4 * ops.compute_units():
+        forms[ops.OWN_ROWS_SHARED_OUT] = graph_time_us(own(6), calls, flush)
       rows_choice = min(forms, key=forms.get)
       t_rows = forms[rows_choice]
       # k is split from 16 rows up only: below, the left operand is too small for its re-reads to matter, and the
@@ -138,7 +140,8 @@ def tune_products(products: Iterable[Tuple[torch.Tensor, bool]], log: Optional[C
         names = {ops.LIBRARY: "library", ops.OWN_ROWS: "own", ops.OWN_KSPLIT: "own with k split",
                  ops.OWN_ROWS_STAGED: "own, left operand staged", ops.OWN_ROWS_LINES: "own, weights in whole lines",
                  ops.OWN_ROWS_STAGED_LINES: "own, left operand staged, weights in whole lines",
-                 ops.OWN_ROWS_BOTH_STAGED: "own, both operands staged"}
+                 ops.OWN_ROWS_BOTH_STAGED: "own, both operands staged",
+                 ops.OWN_ROWS_SHARED_OUT: "own, rows of the left operand shared out"}
         log(f"product [{rows_w}, {K}]{' gate|up' if gate_up else ''} x {M} rows: "
             + ", ".join(f"{names[c]} {t:.1f} us" for c, t in forms.items())
             + f", own with k split {t_split:.1f} us, library {t_lib:.1f} us with its extra kernels -> {names[choice]}")

@@ -172,15 +172,15 @@ def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, wav
   decoding request is cut.  `resident_workgroups` run on the chip at once (two per compute unit, whatever the head
   size; the default is an MI355X's 2 x 256, the attention part passes its device's): the ranges are as many as still fit in one such round, since a second round that is nearly empty costs as
   much as a full one (96 kv-head entries: 5 ranges take 27 us, 6 take 32); when one range per entry would leave
-  more than a fifth of the round empty, two are used (384 entries: 77 against 82 us).  At most 32, which the merge
-  kernel still combines in one pass over memory (one request of 32,768 keys: 34 us with 32 ranges, 47 with 64),
-  and at least one macro tile per wave."""
+  more than a fifth of the round empty, two are used (384 entries: 77 against 82 us).  At most 64 (one request of
+  32,768 keys: 34.4 us with 32 ranges, 32.2 with 64, 34.0 with 128; beyond 32 ranges the merge is a kernel of four
+  waves per head, whose loads are all on their way at once), and at least one macro tile per wave."""
   tiles = -(-max_keys // tile_keys)
   n = max(1, num_head_entries)
   want = max(1, resident_workgroups // n)
   if want == 1 and n < resident_workgroups and 5 * n <= 4 * resident_workgroups:
     want = 2
-  return int(max(1, min(want, max(1, tiles // waves), 32)))
+  return int(max(1, min(want, max(1, tiles // waves), 64)))
 
 
 def plain_splits(num_waves: int, max_keys: int, resident_waves: int = 4096) -> int:

@@ -7,8 +7,9 @@ What these lengths and widths switch on that shorter tests never reach: the pref
 by the rule from the number of workgroups ("wide" for a whole 9,001-token prompt, "dense" for portions of 4,096,
 "two_tiles" for small ones), causal tile skipping over a hundred macro tiles, decode attention over hundreds of
 pages with many key ranges, block tables wider than 512 pages in captured steps; and for wide batches products of
-more than 64 rows (the library's), of 17 to 64 rows (k split across workgroups, by rule, and forced), decode
-attention without key ranges, sampling of a hundred rows.
+more than 64 rows (the library's), of 17 to 64 rows (by rule, and forced to each form: k split across workgroups, the
+left operand's rows shared out, whole rows, the library), decode attention without key ranges, sampling of a hundred
+rows.
 """
 
 import numpy as np
@@ -198,7 +199,7 @@ def _wide_steps(requests, live_counts):
 WIDE_BF16_MAX, WIDE_BF16_MEAN = 0.025, 0.0035
 
 
-@pytest.mark.parametrize("products", ["by_rule", "k_split", "library", "own_rows"])
+@pytest.mark.parametrize("products", ["by_rule", "k_split", "library", "own_rows", "rows_shared_out"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_hundred_requests_decode_side_by_side(wide_model, dtype, products, monkeypatch):
   """Steps of 100, 100, 64, 40 and 17 single tokens (the last three are the widths at which a product of few rows
@@ -211,7 +212,8 @@ def test_a_hundred_requests_decode_side_by_side(wide_model, dtype, products, mon
   requests, want = wide_model["requests"], wide_model["want"]
   steps, done = _wide_steps(requests, [100, 100, 64, 40, 17])
   choices = ops.ProductChoices()
-  choices.force = {"by_rule": None, "k_split": ops.OWN_KSPLIT, "library": ops.LIBRARY, "own_rows": ops.OWN_ROWS}[products]
+  choices.force = {"by_rule": None, "k_split": ops.OWN_KSPLIT, "library": ops.LIBRARY, "own_rows": ops.OWN_ROWS,
+                   "rows_shared_out": ops.OWN_ROWS_SHARED_OUT}[products]
   rp = Replayer(wide_model["folders"][dtype], dtype, tt.peak_tokens(steps, requests), page_size=16,
                 max_requests=NUM_LIVE, choices=choices)
   seen_variants = []
@@ -227,12 +229,16 @@ def test_a_hundred_requests_decode_side_by_side(wide_model, dtype, products, mon
   assert rp.cache.all_pages_free()
   if dtype == "bfloat16":
     wide_rows = {v for v, m in seen_variants if 17 <= m <= 64}
-    if products in ("by_rule", "k_split"):
+    if products == "by_rule":      # rows of 2,048 and 3,072 columns of a matrix of 1,024 rows: the left operand's rows shared out
+      assert 6 in wide_rows, f"no product of 17 to 64 rows by the rule's form for few matrix rows: {sorted(set(seen_variants))}"
+    if products == "k_split":
       assert 1 in wide_rows, f"no product of 17 to 64 rows had its k split: {sorted(set(seen_variants))}"
     if products == "library":
       assert choices.library_products[0] > 0 and not wide_rows
     if products == "own_rows":
       assert wide_rows == {0}
+    if products == "rows_shared_out":
+      assert wide_rows == {6}
   got = tt.gather(steps, outs, {r: t[:done[r]] for r, t in requests.items()}, WIDE["vocab_size"])
   worst = (0.0, 0.0)
   for rid in requests:

@@ -382,8 +382,9 @@ def test_mfma_attention_finds_a_far_key_and_respects_the_window_edge():
 
 
 # whole rows of the result per workgroup / k split across workgroups / whole rows, left operand staged through LDS /
-# whole rows, weights fetched in whole memory lines / both / both operands staged through LDS
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
+# whole rows, weights fetched in whole memory lines / both / both operands staged through LDS / the rows of the left
+# operand shared out across workgroups too
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M,N,K", [(1, 1024, 1024), (8, 4096, 1024), (16, 1024, 3072), (17, 500, 80), (64, 6144, 1024),
                                    (3, 151936, 256), (33, 48, 2048), (5, 130, 88), (64, 1000, 40), (7, 2050, 64),
@@ -435,7 +436,7 @@ def test_gemm_skinny_drawn_shapes():
     if gate_up:
       want = torch.nn.functional.silu(want[:, :N]) * want[:, N:]
     outs = {}
-    for variant in (0, 1, 2, 3, 4, 5):
+    for variant in (0, 1, 2, 3, 4, 5, 6):
       if variant == 1 and gate_up and N % 4:
         continue
       out = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
@@ -449,7 +450,7 @@ def test_gemm_skinny_drawn_shapes():
       assert torch.equal(outs[5], outs[0]), (M, N, K)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 112, 80), (40, 160, 96), (64, 100, 256), (33, 1028, 2200),
                                    (8, 1536, 4096), (16, 516, 2048), (48, 260, 1024), (3, 200, 5120), (20, 36, 448)])
 def test_gemm_skinny_gate_up_activation(M, I, K, variant):
@@ -566,7 +567,7 @@ def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, win
                                                (40, 136, 264, 200, True), (64, 1024, 2048, 3072, False), (5, 88, 40, 24, False),
                                                (12, 2056, 96, 160, True), (64, 1024, 3072, 4096, False),
                                                (33, 520, 2304, 132, True)])
-@pytest.mark.parametrize("variants", [(0, 0), (1, 0), (0, 1), (1, 1), (2, 2), (2, 1), (4, 3), (3, 4), (5, 5)])
+@pytest.mark.parametrize("variants", [(0, 0), (1, 0), (0, 1), (1, 1), (2, 2), (2, 1), (4, 3), (3, 4), (5, 5), (6, 6), (6, 1)])
 def test_norm_split_between_two_products(M, N, K, N2, gate_up, variants):
   """residual += a W1^T; y = rmsnorm(residual) * w; out = y W2^T (or the gated activation of it), the add and the
   norm done half in the first product's kernel and half in the second's.  Against 64-bit arithmetic with the

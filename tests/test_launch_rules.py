@@ -3,7 +3,7 @@
 import pytest
 
 
-def test_decode_key_ranges_fill_one_round_and_stay_mergeable_in_one_pass():
+def test_decode_key_ranges_fill_one_round_and_stay_few():
   from miniinfer_amd.parts.attention import decode_splits
   for waves, tile in ((4, 64), (2, 32)):
     for entries in (1, 2, 4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 256):
@@ -12,13 +12,14 @@ def test_decode_key_ranges_fill_one_round_and_stay_mergeable_in_one_pass():
           n = entries * kv_heads
           s = decode_splits(n, keys, tile, waves)
           tiles = -(-keys // tile)
-          assert 1 <= s <= 32
+          assert 1 <= s <= 64
           assert s == 1 or s * waves <= tiles                 # a wave of every range has a tile
           assert s <= 2 or n * s <= 512                        # more than two ranges only while they fit one round
   # the cases the rule was measured on
   assert decode_splits(8 * 8, 2048) == 8 and decode_splits(12 * 8, 2048) == 5 and decode_splits(24 * 8, 2048) == 2
   assert decode_splits(48 * 8, 2048) == 2 and decode_splits(64 * 8, 2048) == 1
-  assert decode_splits(8, 8192) == 32 and decode_splits(8, 32768) == 32 and decode_splits(8, 2048) == 8
+  assert decode_splits(8, 8192) == 32 and decode_splits(8, 32768) == 64 and decode_splits(8, 2048) == 8
+  assert decode_splits(16, 32768) == 32 and decode_splits(1, 1 << 20) == 64
   assert decode_splits(8 * 4, 2048, 32, 2) == 16 and decode_splits(64 * 4, 2048, 32, 2) == 2
 
 
@@ -38,7 +39,8 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     # else up to 16 rows have both operands staged through LDS (k a multiple of 32) when the matrix has 16 M
     # elements, or rows of 2,048 columns and no activation behind it; what is left has the left operand staged from
     # 4 rows and 12 K elements
-    assert ops.skinny_variant(64, 1024, 3072) == 1 and ops.skinny_variant(17, 1024, 2048) == 1
+    assert ops.skinny_variant(64, 1024, 3072) == 6 and ops.skinny_variant(17, 1024, 2048) == 6   # few rows of the matrix
+    assert ops.skinny_variant(64, 2048, 2048) == 1 and ops.skinny_variant(48, 2048, 2048) == 6 and ops.skinny_variant(16, 1024, 2048) == 5
     assert ops.skinny_variant(16, 1024, 3072) == 5 and ops.skinny_variant(64, 4096, 1024) == 2
     assert ops.skinny_variant(4, 1024, 2048) == 5 and ops.skinny_variant(8, 4096, 1024) == 0
     assert ops.skinny_variant(16, 4096, 1024) == 2 and ops.skinny_variant(8, 6144, 2048, True) == 2
@@ -51,7 +53,7 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     assert ops.skinny_variant(1, 1024, 2048) == 5 and ops.skinny_variant(1, 4096, 4096) == 5
     assert ops.skinny_variant(3, 24576, 4096, True) == 5 and ops.skinny_variant(3, 6144, 2048, True) == 0
     assert ops.skinny_variant(8, 1024, 2000) == 2 and ops.skinny_variant(2, 1024, 2000) == 0
-    assert ops.skinny_variant(20, 1024, 1024) == 2 and ops.skinny_variant(4, 1024, 1000) == 0
+    assert ops.skinny_variant(20, 1024, 1024) == 6 and ops.skinny_variant(20, 4096, 1024) == 2 and ops.skinny_variant(4, 1024, 1000) == 0
     assert ops.skinny_variant(64, 2 * 1026, 4096, True) == 2 and ops.skinny_variant(64, 2 * 1028, 4096, True) == 1
     for p in ops.TUNE_ROWS:
       ops.set_product_choice(p, 4096, 4096, False, p > 8)

@@ -138,7 +138,7 @@ def test_decode_attention_at_long_contexts_with_the_engines_own_split_counts(len
   tile_keys, waves = ops.attn_decode_geometry(d)
   splits = decode_splits(B * nkv, max(lens), tile_keys, waves)
   print(f"decode attention: {B} requests of {lens} keys, {splits} key ranges, fused front {front}", flush=True)
-  assert splits == (32 if B == 1 else 8)
+  assert splits == ({8192: 32, 32768: 64}[lens[0]] if B == 1 else 8)
   g = torch.Generator().manual_seed(sum(lens))
   qs, kps, vps, rows, wants = [], [], [], [], []
   base = 0
