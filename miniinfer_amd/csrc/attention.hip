@@ -210,6 +210,187 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(
   }
 }
 
+// The same wave per (token, query heads of one kv head, key range) for 32-bit caches with head sizes in steps of 16
+// up to 128 and pages of 16 keys or more, with every load instruction of the wave covering whole lines of memory:
+// four lanes share a key.  Scores: lane (key = lane / 4, quarter = lane % 4) reads floats 16 i + 4 quarter .. + 3 of
+// its key's row for every i, so the four lanes read 64 bytes side by side and the wave 16 keys at a time; each lane's
+// partial score is one chain of fused multiply-adds over its dims in ascending order, the four are added as
+// (0 + 1) + (2 + 3), and four such passes give the tile's 64 scores, which are then moved to one key a lane.
+// Values: in the transposed pages a dim's 16 keys of a block are 64 bytes; lane (dim = lane / 4 + 16 c, quarter)
+// reads keys 4 quarter .. + 3 of the block and keeps its own sum for the dim, keys ascending; the four quarters' sums
+// are added once, at the end.  Blocks of 16 keys are aligned in the pages, so a tile that does not start on one (a
+// window's edge) and the last tile take their ragged blocks key by key.
+// DC = head size / 16 is a parameter of the build (64, 80, 96 and 128 are built), so that no branch stands between a
+// tile's loads.
+template <int REP, int DC>
+__global__ __launch_bounds__(256) void paged_attention_quad_kernel(
+    const float* __restrict__ q, int64_t q_row_stride, float* __restrict__ out, int64_t out_row_stride,
+    const float* __restrict__ k_pages, const float* __restrict__ v_pages, const int* __restrict__ block_table,
+    int table_width, const int* __restrict__ token_req, const int* __restrict__ cu_q, const int* __restrict__ kv_len,
+    int num_tokens, int nq, int nkv, int d, int page_shift, float scale, int window, int num_splits,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
+  extern __shared__ float smem[];
+  const int lane = threadIdx.x & (MI_WAVE - 1);
+  const int wave = threadIdx.x / MI_WAVE;
+  float* qs = smem + wave * REP * d;
+  const int groups = nq / REP;
+  const int64_t wid = (int64_t)blockIdx.x * (blockDim.x / MI_WAVE) + wave;
+  const bool live = wid < (int64_t)num_tokens * groups * num_splits;
+  int t = 0, h0 = 0, split = 0;
+  if (live) {
+    const int64_t tg = wid / num_splits;
+    split = (int)(wid - tg * num_splits);
+    t = (int)(tg / groups);
+    h0 = (int)(tg - (int64_t)t * groups) * REP;
+    const float* qr = q + (int64_t)t * q_row_stride + (int64_t)h0 * d;
+    for (int e = lane; e < REP * d; e += MI_WAVE) qs[e] = qr[e];
+  }
+  __syncthreads();
+  if (!live) return;
+
+  const int b = token_req[t];
+  const int q_begin = cu_q[b];
+  const int q_len = cu_q[b + 1] - q_begin;
+  const int pos = kv_len[b] - q_len + (t - q_begin);
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int g = h0 / (nq / nkv);
+  const int P = 1 << page_shift;
+  const int* bt = block_table + (int64_t)b * table_width;
+  const int quad = lane >> 2, quarter = lane & 3;
+
+  const int tiles = (pos - lo) / MI_WAVE + 1;
+  const int j_begin = lo + (int)((int64_t)split * tiles / num_splits) * MI_WAVE;
+  const int j_stop = (split + 1 == num_splits) ? pos + 1 : lo + (int)((int64_t)(split + 1) * tiles / num_splits) * MI_WAVE;
+
+  float m[REP], l[REP], acc[REP][DC];
+#pragma unroll
+  for (int x = 0; x < REP; ++x) {
+    m[x] = -INFINITY;
+    l[x] = 0.f;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) acc[x][c] = 0.f;
+  }
+
+  for (int j0 = j_begin; j0 < j_stop; j0 += MI_WAVE) {
+    // scores: four passes of 16 keys; a key past pos reads the row of pos and is masked below
+    float sc[4][REP];
+#pragma unroll        // all four passes' loads on their way together (one or two at a time: 39 against 31.5 us)
+    for (int pass = 0; pass < 4; ++pass) {
+      const int jk = min(j0 + pass * 16 + quad, pos);
+      const int64_t page = bt[jk >> page_shift];
+      const float* row = k_pages + ((page * nkv + g) * P + (jk & (P - 1))) * d + 4 * quarter;
+#pragma unroll
+      for (int x = 0; x < REP; ++x) sc[pass][x] = 0.f;
+#pragma unroll
+      for (int i = 0; i < DC; ++i) {
+        float kv[4];
+        load4(row + 16 * i, kv);
+#pragma unroll
+        for (int x = 0; x < REP; ++x) {
+          float qv[4];
+          load4(qs + x * d + 16 * i + 4 * quarter, qv);
+#pragma unroll
+          for (int y = 0; y < 4; ++y) sc[pass][x] = fmaf(qv[y], kv[y], sc[pass][x]);
+        }
+      }
+#pragma unroll
+      for (int x = 0; x < REP; ++x) {
+        sc[pass][x] += __shfl_xor(sc[pass][x], 1, MI_WAVE);
+        sc[pass][x] += __shfl_xor(sc[pass][x], 2, MI_WAVE);
+      }
+    }
+    // one key a lane: lane L takes key j0 + L, which pass L / 16 left in the lanes of quad L % 16
+    const int j = j0 + lane;
+    float s[REP], p[REP];
+#pragma unroll
+    for (int x = 0; x < REP; ++x) {
+      const int src = 4 * (lane & 15);
+      const float s0 = __shfl(sc[0][x], src, MI_WAVE), s1 = __shfl(sc[1][x], src, MI_WAVE);
+      const float s2 = __shfl(sc[2][x], src, MI_WAVE), s3 = __shfl(sc[3][x], src, MI_WAVE);
+      const int pass = lane >> 4;
+      const float v = pass == 0 ? s0 : (pass == 1 ? s1 : (pass == 2 ? s2 : s3));
+      s[x] = (j <= pos) ? v * scale : -INFINITY;
+    }
+#pragma unroll
+    for (int x = 0; x < REP; ++x) {
+      const float m_new = fmaxf(m[x], wave_max(s[x]));
+      p[x] = (j <= pos) ? expf(s[x] - m_new) : 0.f;
+      const float alpha = expf(m[x] - m_new);
+      l[x] = l[x] * alpha + wave_sum(p[x]);
+      m[x] = m_new;
+#pragma unroll
+      for (int c = 0; c < DC; ++c) acc[x][c] *= alpha;
+    }
+    // values: the aligned blocks of 16 keys that hold keys j0 .. j_end - 1
+    const int j_end = min(j0 + MI_WAVE, pos + 1);
+    for (int bs = j0 & ~15; bs < j_end; bs += 16) {
+      const int64_t page = bt[bs >> page_shift];
+      const float* vbase = v_pages + (page * nkv + g) * (int64_t)d * P + (bs & (P - 1)) + 4 * quarter;
+      const int k0 = bs + 4 * quarter;           // this lane's four keys of the block
+      if (bs >= j0 && bs + 16 <= j_end) {
+        float pk[REP][4];
+#pragma unroll
+        for (int x = 0; x < REP; ++x)
+#pragma unroll
+          for (int y = 0; y < 4; ++y) pk[x][y] = __shfl(p[x], k0 - j0 + y, MI_WAVE);
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+          float v4[4];
+          load4(vbase + (int64_t)(quad + 16 * c) * P, v4);
+#pragma unroll
+          for (int x = 0; x < REP; ++x)
+#pragma unroll
+            for (int y = 0; y < 4; ++y) acc[x][c] = fmaf(pk[x][y], v4[y], acc[x][c]);
+        }
+      } else {
+#pragma unroll
+        for (int y = 0; y < 4; ++y) {
+          const int key = k0 + y;
+          const bool inside = key >= j0 && key < j_end;
+          float pk[REP];
+#pragma unroll
+          for (int x = 0; x < REP; ++x) pk[x] = __shfl(p[x], inside ? key - j0 : 0, MI_WAVE);
+          if (inside) {
+#pragma unroll
+            for (int c = 0; c < DC; ++c) {
+              const float vv = vbase[(int64_t)(quad + 16 * c) * P + y];
+#pragma unroll
+              for (int x = 0; x < REP; ++x) acc[x][c] = fmaf(pk[x], vv, acc[x][c]);
+            }
+          }
+        }
+      }
+    }
+  }
+  // the four quarters' sums of a dim, added as (0 + 1) + (2 + 3); quarter u then stores the dims of blocks c = u mod 4
+#pragma unroll
+  for (int x = 0; x < REP; ++x) {
+#pragma unroll
+    for (int c = 0; c < DC; ++c) {
+      acc[x][c] += __shfl_xor(acc[x][c], 1, MI_WAVE);
+      acc[x][c] += __shfl_xor(acc[x][c], 2, MI_WAVE);
+    }
+    const int h = h0 + x;
+    if (num_splits > 1) {
+      const int64_t item = ((int64_t)t * nq + h) * num_splits + split;
+      float* po = part_o + item * d;
+#pragma unroll
+      for (int c = 0; c < DC; ++c)
+        if ((c & 3) == quarter) po[quad + 16 * c] = acc[x][c];
+      if (lane == 0) {
+        part_ml[item * 2] = m[x];
+        part_ml[item * 2 + 1] = l[x];
+      }
+    } else {
+      float* o = out + (int64_t)t * out_row_stride + (int64_t)h * d;
+      const float inv = 1.f / l[x];
+#pragma unroll
+      for (int c = 0; c < DC; ++c)
+        if ((c & 3) == quarter) o[quad + 16 * c] = acc[x][c] * inv;
+    }
+  }
+}
+
 // One workgroup per (token, head): out = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s with M = max_s m_s.
 // An empty part has m = -inf and l = 0 and adds nothing; the last part is never empty, so M is finite.
 // The parts' weights are made once, by the lanes side by side, and kept in LDS; then thread (group, dim) adds the
@@ -284,7 +465,13 @@ MI_EXPORT int mi_paged_attention(int dtype, const void* q, int64_t q_row_stride,
   while ((1 << shift) < page_size) ++shift;
   const int waves_per_block = 4;
   const int per_kv = nq / nkv;
-  const int rep = (per_kv == 2 || per_kv == 4 || per_kv == 8) ? per_kv : 1;
+  int rep = (per_kv == 2 || per_kv == 4 || per_kv == 8) ? per_kv : 1;
+  // the kernel with four lanes a key: 32-bit, head sizes it is built for, pages of whole blocks of 16 keys; it holds
+  // more of a tile in registers, so eight query heads of a kv head go to two waves of four
+  const bool quads = dtype == MI_DTYPE_F32 && (d == 64 || d == 80 || d == 96 || d == 128) && page_size >= 16 &&
+                     q_row_stride % 4 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
+                     (uintptr_t)v_pages % 16 == 0;
+  if (quads && rep == 8) rep = 4;
   const int64_t waves = (int64_t)num_tokens * (nq / rep) * num_splits;
   MI_REQUIRE(waves / waves_per_block < (int64_t)INT32_MAX, "paged_attention: too many (token, head, part) items");
   const int blocks = (int)((waves + waves_per_block - 1) / waves_per_block);
@@ -298,12 +485,28 @@ MI_EXPORT int mi_paged_attention(int dtype, const void* q, int64_t q_row_stride,
   else if (rep == 4) ATTN_GO(T, 4);                                                                                 \
   else if (rep == 2) ATTN_GO(T, 2);                                                                                 \
   else ATTN_GO(T, 1)
-  if (dtype == MI_DTYPE_F32) {
+#define ATTN_QUAD(REP, DC)                                                                                           \
+  paged_attention_quad_kernel<REP, DC><<<blocks, waves_per_block * MI_WAVE, lds, stream>>>(                         \
+      (const float*)q, q_row_stride, (float*)out, out_row_stride, (const float*)k_pages, (const float*)v_pages,     \
+      block_table, table_width, token_req, cu_q, kv_len, num_tokens, nq, nkv, d, shift, scale, window, num_splits,  \
+      part_o, part_ml)
+#define ATTN_QUAD_REP(DC)                                                                                            \
+  if (rep == 4) ATTN_QUAD(4, DC);                                                                                    \
+  else if (rep == 2) ATTN_QUAD(2, DC);                                                                               \
+  else ATTN_QUAD(1, DC)
+  if (quads) {
+    if (d == 64) { ATTN_QUAD_REP(4); }
+    else if (d == 80) { ATTN_QUAD_REP(5); }
+    else if (d == 96) { ATTN_QUAD_REP(6); }
+    else { ATTN_QUAD_REP(8); }
+  } else if (dtype == MI_DTYPE_F32) {
     ATTN_REP(float);
   } else if (dtype == MI_DTYPE_BF16) {
     ATTN_REP(bf16);
   } else
     MI_FAIL("paged_attention: unknown dtype %d", dtype);
+#undef ATTN_QUAD_REP
+#undef ATTN_QUAD
 #undef ATTN_REP
 #undef ATTN_GO
   MI_CHECK_LAUNCH("paged_attention");

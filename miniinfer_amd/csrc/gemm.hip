@@ -130,14 +130,16 @@ __global__ __launch_bounds__(512) void gemm_nt_stream_kernel(const TA* __restric
   const bool finisher = tid < R * MT;
   float tot = 0.f;
   for (int kb = 0; kb < K; kb += SCH * CHUNK_K) {
-    // this thread's weights of the block: all loads on their way before anything waits
+    // The block of A into LDS, rows beyond M as zeros: 8 loads of 16 bytes of a thread on their way at a time.  This
+    // thread's weights of the block are asked for behind the last of them and before anything waits: loads come back
+    // in the order they were asked for, so A (small, shared by every workgroup, from the caches) is staged and the
+    // first products run while the later weights are still on their way from memory.
     float wv[CHUNK_K / 4][4];
-#pragma unroll
-    for (int q = 0; q < CHUNK_K / 4; ++q) fetch4<TA, VEC>(wrow, kb + c * CHUNK_K + 4 * q, K, n_ok, wv[q]);
-    // the block of A into LDS, rows beyond M as zeros: 8 loads of 16 bytes of a thread on their way at a time
-    constexpr int ITEMS = MT * SCH * (CHUNK_K / 4);
-    for (int base = tid; base < ITEMS; base += 8 * blockDim.x) {
-      float v[8][4];
+    constexpr int ITEMS = MT * SCH * (CHUNK_K / 4);       // at least 4 a thread: MT >= 4, R <= 16
+    const int stride = 8 * blockDim.x;
+    const int last = tid + (ITEMS - 1 - tid) / stride * stride;      // where this thread's last batch begins
+    float v[8][4];
+    auto ask = [&](int base) {
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int idx = base + u * blockDim.x;
@@ -145,6 +147,8 @@ __global__ __launch_bounds__(512) void gemm_nt_stream_kernel(const TA* __restric
         const int m = idc / (SCH * (CHUNK_K / 4)), q = idc % (SCH * (CHUNK_K / 4));
         fetch4<TA, VEC>(A + (int64_t)(m < M ? m : 0) * lda, kb + 4 * q, K, m < M, v[u]);
       }
+    };
+    auto stage = [&](int base) {
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int idx = base + u * blockDim.x;
@@ -153,7 +157,15 @@ __global__ __launch_bounds__(512) void gemm_nt_stream_kernel(const TA* __restric
           store4(As + (m * SCH + q / (CHUNK_K / 4)) * SPAD + 4 * (q % (CHUNK_K / 4)), v[u]);
         }
       }
+    };
+    for (int base = tid; base < last; base += stride) {
+      ask(base);
+      stage(base);
     }
+    ask(last);
+#pragma unroll
+    for (int q = 0; q < CHUNK_K / 4; ++q) fetch4<TA, VEC>(wrow, kb + c * CHUNK_K + 4 * q, K, n_ok, wv[q]);
+    stage(last);
     __syncthreads();
     float acc[MT];
 #pragma unroll

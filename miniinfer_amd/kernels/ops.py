@@ -882,6 +882,19 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor], top_k: Opt
   return out
 
 
+def plain_attention_geometry(dtype: torch.dtype, nq: int, nkv: int, d: int, page_size: int) -> Tuple[int, int]:
+  """(query heads one wave of the plain kernel takes, waves that are resident on a compute unit at once) for these
+  sizes, as `mi_paged_attention` launches them: 32-bit caches with head sizes 64, 80, 96 or 128 and pages of 16 keys
+  or more go to the kernel with four lanes a key, which holds a whole tile's loads in registers (8 waves a unit, up
+  to 4 heads a wave); everything else to the kernel with one key a lane (16 waves, up to 8 heads)."""
+  per_kv = nq // nkv
+  quad = dtype == torch.float32 and d in (64, 80, 96, 128) and page_size >= 16
+  rep = per_kv if per_kv in (2, 4, 8) else 1
+  if quad and rep == 8:
+    rep = 4
+  return rep, (8 if quad else 16)
+
+
 # ----------------------------------------------------------------------------- attention on the matrix cores
 
 def mfma_attention_supported(dtype: torch.dtype, nq: int, nkv: int, d: int, page_size: int) -> bool:

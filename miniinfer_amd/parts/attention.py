@@ -125,10 +125,9 @@ class PagedAttention(Part):
     table = ctx.block_tables[cache.group]
     if not ops.mfma_attention_supported(qkv.dtype, nq, nkv, d, cache.page_size):
       T = qkv.shape[0]
-      per_kv = nq // nkv
-      waves = T * (nkv if per_kv in (2, 4, 8) else nq)      # the kernel takes such a group's heads in one wave
-      splits = plain_splits(waves, min(ctx.max_kv_len, window) if window else ctx.max_kv_len,
-                            16 * ops.compute_units())
+      heads_a_wave, waves_a_unit = ops.plain_attention_geometry(qkv.dtype, nq, nkv, d, cache.page_size)
+      splits = plain_splits(T * (nq // heads_a_wave), min(ctx.max_kv_len, window) if window else ctx.max_kv_len,
+                            waves_a_unit * ops.compute_units())
       part_o = part_ml = None
       if splits > 1:
         part_o = ctx.scratch("attn_part_o", T * nq * splits * d, torch.float32)
@@ -185,9 +184,11 @@ def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, wav
 
 def plain_splits(num_waves: int, max_keys: int, resident_waves: int = 4096) -> int:
   """Into how many key ranges the plain kernel (one wave per token and group of query heads) cuts each token's keys:
-  as many as fill the chip's wave slots (16 on each compute unit; the default is an MI355X's 16 x 256) once, each
-  range at least one tile of 64 keys, at most 64 ranges: a wave takes its tiles one after the other, so few tokens
-  over many keys are as quick as their longest range.  Prompt portions have waves enough and stay whole."""
+  as many as fill the chip's wave slots once (`resident_waves`: 8 or 16 on each compute unit, by the kernel that
+  runs, `ops.plain_attention_geometry`; the default is 16 x 256; one wave more than fit costs a second round: 40
+  against 31.5 us for 8 requests of 2,048 keys in 33 against 32 ranges), each range at least one tile of 64 keys, at
+  most 64 ranges: a wave takes its tiles one after the other, so few tokens over many keys are as quick as their
+  longest range.  Prompt portions have waves enough and stay whole."""
   want = resident_waves // max(1, num_waves)
   tiles = -(-max_keys // 64)
   return int(max(1, min(want, tiles, 64)))

@@ -211,9 +211,13 @@ def _attention_ref(q, k, v, scale, window):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("splits", [1, 2, 3, 7])
 @pytest.mark.parametrize("nq,nkv,d,P,window", [(6, 3, 48, 16, 0), (8, 2, 128, 8, 0), (4, 4, 16, 4, 0), (5, 1, 80, 32, 0),
-                                               (4, 2, 64, 16, 37), (16, 8, 256, 16, 0), (4, 2, 64, 16, 150)])
+                                               (4, 2, 64, 16, 37), (16, 8, 256, 16, 0), (4, 2, 64, 16, 150),
+                                               (8, 2, 128, 16, 0), (8, 1, 96, 64, 0), (16, 8, 128, 32, 101)])
 def test_paged_attention(dtype, nq, nkv, d, P, window, splits):
-  """Key ranges cut into parts (some of them empty for the short requests) give the same result as whole ones."""
+  """Key ranges cut into parts (some of them empty for the short requests) give the same result as whole ones.  In
+  32-bit the head sizes 64, 80, 96 and 128 with pages of 16 keys or more run on the kernel with four lanes a key (1,
+  2 and 4 query heads a wave, 8 as two waves of 4; windows whose edge is no multiple of 16), the others on the
+  kernel with a key a lane."""
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(5)
   # requests: (keys already cached, new tokens)
