@@ -7,6 +7,7 @@
 // chunks' sums are added one after the other, first chunk first.  So a row's result does not depend on what else
 // is in the batch, bit for bit, and the chunks are what the kernel for few rows works on side by side.
 #include "common.h"
+#include <type_traits>
 
 #define BM 64
 #define BN 64
@@ -193,6 +194,85 @@ __global__ __launch_bounds__(512) void gemm_nt_stream_kernel(const TA* __restric
   if (finisher && fm < M && fn < N) C[(int64_t)fm * ldc + fn] = from_float<TC>(tot);
 }
 
+// The same product for up to 8 rows of 32-bit A where all of k fits LDS beside R rows of W (k a multiple of 256) and
+// the row groups make at most one workgroup for every compute unit: both operands go straight from memory to LDS
+// (global_load_lds: lane i's 16 bytes land at base + 16 i), every load instruction of a wave covering 1 KB of one
+// row, which the per-thread loads of the kernel above do not (a thread there walks its own 256 bytes, so an
+// instruction touches 64 lines of memory: 2 TB/s).  A chunk's 16 pieces of 16 bytes are stored rotated by the
+// chunk's number (piece q of chunk c at place (q + c) mod 16), so that the threads of different chunks, which read
+// piece q at the same time, find theirs in different banks.  Thread (row pair, half of A's rows, chunk) then runs
+// the chunk chains of 2 rows of W against 4 rows of A (6 reads of LDS for 32 multiply-adds, where a thread with one
+// row of W and all rows of A needs 9), k ascending from zero as everywhere; the chunks' sums go through LDS to one
+// thread per result element, which adds them in order.  Rows of A beyond M repeat row M - 1 and rows of W beyond N
+// repeat row N - 1 (loads to LDS cannot be replaced by zeros); their results are not stored.
+#define LDS_MT 8
+__global__ __launch_bounds__(512) void gemm_nt_lds_kernel(const float* __restrict__ A, int64_t lda,
+                                                          const float* __restrict__ W, int64_t ldw,
+                                                          float* __restrict__ C, int64_t ldc, int M, int N, int K, int R) {
+  extern __shared__ float lds[];
+  const int SCH = K >> 6, UPR = SCH >> 2;      // chunks of a row; wave loads (1 KB: 4 chunks) of a row
+  float* Ws = lds;                             // [R][K]
+  float* As = lds + R * K;                     // [LDS_MT][K]
+  float* part = As + LDS_MT * K;               // [SCH][R][LDS_MT]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
+  const int n0 = blockIdx.x * R;
+  const int lc = lane >> 4, place = lane & 15;
+  // A first: it comes from the caches and is there when the weights arrive
+  for (int i = wave; i < LDS_MT * UPR; i += waves) {
+    const int m = i / UPR, c = (i - m * UPR) * 4 + lc;
+    const float* src = A + (int64_t)min(m, M - 1) * lda + c * 64 + ((place - c) & 15) * 4;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)(As + i * 256), 16, 0, 0);
+  }
+  for (int i = wave; i < R * UPR; i += waves) {
+    const int r = i / UPR, c = (i - r * UPR) * 4 + lc;
+    const float* src = W + (int64_t)min(n0 + r, N - 1) * ldw + c * 64 + ((place - c) & 15) * 4;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)(Ws + i * 256), 16, 0, 0);
+  }
+  // the compiler does not count the requests that write LDS: the wait is written out
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  const int c = tid % SCH, mh = (tid / SCH) & 1, rp = tid / (2 * SCH);
+  float acc[2][4];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) acc[a][m] = 0.f;
+  const float* w0 = Ws + (2 * rp) * K + c * 64;
+  const float* w1 = w0 + K;
+  const float* a0 = As + (4 * mh) * K + c * 64;
+#pragma unroll
+  for (int q = 0; q < CHUNK_K / 4; ++q) {
+    const int at = ((q + c) & 15) * 4;
+    float wa[4], wb[4];
+    load4(w0 + at, wa);
+    load4(w1 + at, wb);
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      float a[4];
+      load4(a0 + m * K + at, a);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[0][m] = fmaf(a[i], wa[i], acc[0][m]);
+        acc[1][m] = fmaf(a[i], wb[i], acc[1][m]);
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) part[(c * R + 2 * rp + a) * LDS_MT + 4 * mh + m] = acc[a][m];
+  __syncthreads();
+  for (int f = tid; f < R * LDS_MT; f += blockDim.x) {
+    const int fr = f / LDS_MT, fm = f - fr * LDS_MT;
+    float tot = 0.f;
+    for (int x = 0; x < SCH; ++x) tot += part[(x * R + fr) * LDS_MT + fm];
+    if (fm < M && n0 + fr < N) C[(int64_t)fm * ldc + n0 + fr] = tot;
+  }
+}
+
 static int gemm_compute_units() {
   static int cus = 0;
   if (cus == 0) {
@@ -220,6 +300,41 @@ static int launch_stream_instance(const void* A, int64_t lda, const void* W, int
   return 0;
 }
 
+// Launches gemm_nt_lds_kernel where it is the quicker one (0), or says that the case is not its own (1): up to 8 rows
+// of A, k a multiple of 256, 16-byte alignment, and a number of rows R of W per workgroup (16, 8 or 4: the most that
+// fit LDS and still make a workgroup for every other compute unit) with which the row groups do not exceed the
+// compute units (a second round of such workgroups would wait for the first: nothing overlaps inside one).
+// On an MI355X, 8 rows: [4096, 1024] 7.5 against 9.2 us, [1024, 2048] 7.2 against 9.7, [1024, 3072] 8.6 against 11.6;
+// [6144, 1024] (384 row groups) 12.1 against 11.3, which is why it stays with the kernel above.
+static int launch_lds(const float* A, int64_t lda, const float* W, int64_t ldw, float* C, int64_t ldc, int M, int N, int K,
+                      int cus, hipStream_t stream) {
+  if (M > LDS_MT || K % 256 != 0 || lda % 4 != 0 || ldw % 4 != 0 || (uintptr_t)A % 16 != 0 || (uintptr_t)W % 16 != 0) return 1;
+  const int sch = K / CHUNK_K;
+  int R = 0;
+  size_t lds = 0;
+  for (int r = 16; r >= 4; r /= 2) {
+    const size_t need = ((size_t)(r + LDS_MT) * K + (size_t)sch * r * LDS_MT) * sizeof(float);
+    const int threads = r * sch;           // (r / 2 row pairs) x 2 halves of A's rows x chunks
+    if (need <= 160 * 1024 && threads <= 512 && threads % 64 == 0 && ceil_div(N, r) >= cus / 2) {
+      R = r;
+      lds = need;
+      break;
+    }
+  }
+  if (R == 0 || ceil_div(N, R) > cus) return 1;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_lds_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      snprintf(g_mi_error, sizeof(g_mi_error), "gemm_nt: cannot raise the LDS allotment: %s", hipGetErrorString(e));
+      return -1;
+    }
+    raised = true;
+  }
+  gemm_nt_lds_kernel<<<ceil_div(N, R), R * sch, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, R);
+  return 0;
+}
+
 template <typename TA, typename TC>
 static int launch_stream(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
                          hipStream_t stream) {
@@ -229,6 +344,10 @@ static int launch_stream(const void* A, int64_t lda, const void* W, int64_t ldw,
   // one for every other unit, else 4 (every workgroup stages the rows of A once, so more rows mean fewer reads of
   // A; what fills the machine is the bytes on their way, 256 of them a thread), and never more than 512 threads.
   const int cus = gemm_compute_units();
+  if (std::is_same<TA, float>::value && std::is_same<TC, float>::value) {
+    const int rc = launch_lds((const float*)A, lda, (const float*)W, ldw, (float*)C, ldc, M, N, K, cus, stream);
+    if (rc <= 0) return -rc;      // 0: launched; negative: an error; 1: not its case
+  }
   const int mt = M <= 4 ? 4 : (M <= 8 ? 8 : 16);
   const int chunks = ceil_div(K, CHUNK_K);
   int sch = chunks <= 16 ? 16 : (chunks <= 32 || mt == 16 ? 32 : 48);

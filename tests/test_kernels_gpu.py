@@ -81,7 +81,8 @@ def test_silu_mul(dtype, M, I):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,N,K", [(1, 500, 80), (7, 130, 96), (65, 64, 17), (33, 1000, 1024), (128, 257, 300)])
+@pytest.mark.parametrize("M,N,K", [(1, 500, 80), (7, 130, 96), (65, 64, 17), (33, 1000, 1024), (128, 257, 300),
+                                   (5, 1100, 2048), (8, 2049, 512), (3, 4096, 1024)])
 def test_gemm_nt(dtype, M, N, K):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(3)
@@ -98,10 +99,12 @@ def test_gemm_nt(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("N,K", [(130, 96), (1000, 1030), (48, 17)])
+@pytest.mark.parametrize("N,K", [(130, 96), (1000, 1030), (48, 17), (1027, 1024), (4096, 768), (601, 3072)])
 def test_gemm_nt_rows_do_not_depend_on_the_batch(dtype, N, K):
-  """Few rows go to a kernel of their own (one result element per thread), many to the tiled one: both add a result
-  element's products in the same order, so a row's result is the same bits whichever kernel ran it."""
+  """Few rows go to kernels of their own, many to the tiled one: all add a result element's products in the same
+  order, so a row's result is the same bits whichever kernel ran it.  (Up to 8 rows in 32-bit with k a multiple of 256
+  and row groups for half to all of the compute units take both operands through LDS: the last three shapes, with 4,
+  16 and 4 rows of the matrix per workgroup and a last workgroup that is not full.)"""
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(4)
   a = torch.randn(40, K, generator=g).to(dtype).to(DEV)
