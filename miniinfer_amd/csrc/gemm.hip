@@ -301,26 +301,30 @@ static int launch_stream_instance(const void* A, int64_t lda, const void* W, int
 }
 
 // Launches gemm_nt_lds_kernel where it is the quicker one (0), or says that the case is not its own (1): up to 8 rows
-// of A, k a multiple of 256, 16-byte alignment, and a number of rows R of W per workgroup (16, 8 or 4: the most that
-// fit LDS and still make a workgroup for every other compute unit) with which the row groups do not exceed the
-// compute units (a second round of such workgroups would wait for the first: nothing overlaps inside one).
+// of A, k a multiple of 256, 16-byte alignment, and a number of rows R of W per workgroup that fits LDS and with which
+// the row groups do not exceed the compute units (a second round of such workgroups would wait for the first: nothing overlaps inside one).
 // On an MI355X, 8 rows: [4096, 1024] 7.5 against 9.2 us, [1024, 2048] 7.2 against 9.7, [1024, 3072] 8.6 against 11.6;
 // [6144, 1024] (384 row groups) 12.1 against 11.3, which is why it stays with the kernel above.
 static int launch_lds(const float* A, int64_t lda, const float* W, int64_t ldw, float* C, int64_t ldc, int M, int N, int K,
                       int cus, hipStream_t stream) {
   if (M > LDS_MT || K % 256 != 0 || lda % 4 != 0 || ldw % 4 != 0 || (uintptr_t)A % 16 != 0 || (uintptr_t)W % 16 != 0) return 1;
   const int sch = K / CHUNK_K;
+  // R: even, at least as many as leave no more row groups than compute units; 8 where fewer would do and 8 still
+  // make a group for every other unit (fewer workgroups read A less often: [1024, 2048] 7.2 against 7.6 us with 4);
+  // the first such R upwards whose workgroup is whole waves, up to 512 threads, and fits LDS, else the largest below
   int R = 0;
   size_t lds = 0;
-  for (int r = 16; r >= 4; r /= 2) {
-    const size_t need = ((size_t)(r + LDS_MT) * K + (size_t)sch * r * LDS_MT) * sizeof(float);
+  const int r_min = 2 * ceil_div(N, 2 * cus);
+  const int r_want = (r_min < 8 && ceil_div(N, 8) >= cus / 2) ? 8 : r_min;
+  auto fits = [&](int r, size_t* need) {
+    *need = ((size_t)(r + LDS_MT) * K + (size_t)sch * r * LDS_MT) * sizeof(float);
     const int threads = r * sch;           // (r / 2 row pairs) x 2 halves of A's rows x chunks
-    if (need <= 160 * 1024 && threads <= 512 && threads % 64 == 0 && ceil_div(N, r) >= cus / 2) {
-      R = r;
-      lds = need;
-      break;
-    }
-  }
+    return *need <= 160 * 1024 && threads <= 512 && threads % 64 == 0;
+  };
+  for (int r = r_want; r <= 32 && R == 0; r += 2)
+    if ((r == r_min || ceil_div(N, r) >= cus / 2) && fits(r, &lds)) R = r;
+  for (int r = r_want - 2; r >= r_min && r >= 2 && R == 0; r -= 2)
+    if (fits(r, &lds)) R = r;
   if (R == 0 || ceil_div(N, R) > cus) return 1;
   static bool raised = false;
   if (!raised) {
