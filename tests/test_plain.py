@@ -193,7 +193,7 @@ def test_layer_windows_follow_the_config_keys():
 
 def test_plain_attention_key_ranges():
   """The one-wave-per-head kernel's key ranges: whole for prompt portions and short contexts, cut for few tokens
-  over many keys, never shorter than two tiles, never more than 64."""
+  over many keys, never shorter than one tile, never more than 64."""
   from miniinfer_amd.parts.attention import plain_splits
   assert plain_splits(2048 * 16, 2048) == 1
   assert plain_splits(8 * 16, 100) == 2
@@ -201,3 +201,13 @@ def test_plain_attention_key_ranges():
   assert plain_splits(1, 700) == 11
   assert plain_splits(1, 1 << 20) == 64
   assert plain_splits(4096, 1 << 20) == 1
+  # the kernel with four lanes a key holds 8 waves a compute unit: 8 requests x 8 kv heads get 32 ranges of 2,100 keys'
+  # 33 tiles (a 33rd range would start a second round of waves), and it takes 8 query heads of a kv head as 2 waves
+  import torch
+  from miniinfer_amd.kernels import ops
+  assert ops.plain_attention_geometry(torch.float32, 16, 8, 128, 16) == (2, 8)
+  assert ops.plain_attention_geometry(torch.float32, 16, 2, 64, 32) == (4, 8)
+  assert ops.plain_attention_geometry(torch.float32, 16, 2, 48, 16) == (8, 16)      # head size without the kernel
+  assert ops.plain_attention_geometry(torch.float32, 16, 8, 128, 8) == (2, 16)      # pages too small for it
+  assert ops.plain_attention_geometry(torch.bfloat16, 15, 5, 128, 16) == (1, 16)
+  assert plain_splits(8 * 8, 2100, 8 * 256) == 32
