@@ -13,6 +13,15 @@
 // activation C[m, n] = silu(A W_gate^T)[m, n] * (A W_up^T)[m, n] (kernels/triton/silu_mul.py:33-37 of the
 // reference), made from the 32-bit sums of gate row n and up row n, which the same workgroup owns.
 #include "common.h"
+// SKINNY_NT: a second build of this file whose loads of W are nontemporal, for matrices that are read once a step
+// and are larger than what the caches keep until the next step (the caller chooses the build by the matrix's size).
+#ifdef SKINNY_NT
+#define W_LOAD(PTR) __builtin_nontemporal_load(PTR)
+#define W_LDS_AUX 2
+#else
+#define W_LOAD(PTR) (*(PTR))
+#define W_LDS_AUX 0
+#endif
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -174,7 +183,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         const bool kok = (s0 + c < s_end) && k < K;   // K is a multiple of 8: a lane's 8 elements are all in or all out
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
-          w[c][rb] = (kok && w_live) ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
+          w[c][rb] = (kok && w_live) ? W_LOAD(reinterpret_cast<const bf16x8*>(wrow[rb] + k)) : zero_bf16x8();
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
           const bool ok = kok && mok[mb];
@@ -238,7 +247,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
       for (int i = 0; i < NIW; ++i)
         if (w_stp[i] < n)
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wb + w_off[i]),
-                                           (__attribute__((address_space(3))) void*)(stage_w + 512 * i), 16, 0, 0);
+                                           (__attribute__((address_space(3))) void*)(stage_w + 512 * i), 16, 0, W_LDS_AUX);
       if (first) {
         first = false;
         SKINNY_NORM_PREFETCH()
@@ -341,7 +350,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const uint16_t* __res
         if (c < n) {
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb)
-            w[c][rb] = *reinterpret_cast<const u32x4*>(wb + woff[rb][WL ? c & 1 : 0] + (WL ? 128 * (c >> 1) : 64 * c));
+            w[c][rb] = W_LOAD(reinterpret_cast<const u32x4*>(wb + woff[rb][WL ? c & 1 : 0] + (WL ? 128 * (c >> 1) : 64 * c)));
           if constexpr (!STAGED) {
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
@@ -546,7 +555,7 @@ __global__ __launch_bounds__(512) void norm_gemm_kernel(const float* __restrict_
       const int k = 32 * (s0 + c) + 8 * (lane >> 4);
       const bool kok = (s0 + c < s_end) && k < K;
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) w[c][rb] = kok ? *reinterpret_cast<const bf16x8*>(wrow[rb] + k) : zero_bf16x8();
+      for (int rb = 0; rb < RB; ++rb) w[c][rb] = kok ? W_LOAD(reinterpret_cast<const bf16x8*>(wrow[rb] + k)) : zero_bf16x8();
       const bool ok = kok && mok;
       r0[c] = ok ? *reinterpret_cast<const f32x4*>(rrow + k) : f32x4{0.f, 0.f, 0.f, 0.f};
       r1[c] = ok ? *reinterpret_cast<const f32x4*>(rrow + k + 4) : f32x4{0.f, 0.f, 0.f, 0.f};
@@ -958,7 +967,7 @@ __global__ __launch_bounds__(64 * WN) void gemm_splitk_kernel(const uint16_t* __
     _Pragma("unroll") for (int s = 0; s < SK_STEPS; ++s) {                                                    \
       const int k = min(k0_ + 32 * s + 8 * (lane >> 4), K - 8);                                               \
       _Pragma("unroll") for (int rb = 0; rb < RB; ++rb)                                                       \
-        w[SLOT][rb][s] = *reinterpret_cast<const bf16x8*>(wrow_base[rb] + k);                                 \
+        w[SLOT][rb][s] = W_LOAD(reinterpret_cast<const bf16x8*>(wrow_base[rb] + k));                          \
     }                                                                                                         \
   }
 // zeroes what SK_FETCH read from outside the chunk's range (rows past M, columns past k_hi)

@@ -7,8 +7,8 @@ from . import jit
 # every shared object of the library: (source name, defines)
 # head sizes the MFMA attention is prebuilt for (others are built at a model's first use)
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
-ALL_MODULES = [("elementwise", ()), ("gemm", ()), ("gemm_skinny", ()), ("attention", ()), ("sampling", ()),
-               ("probes", ())] + \
+ALL_MODULES = [("elementwise", ()), ("gemm", ()), ("gemm_skinny", ()), ("gemm_skinny", (("SKINNY_NT", 1),)),
+               ("attention", ()), ("sampling", ()), ("probes", ())] + \
     [("attention_mfma", (("HEAD_DIM", d),)) for d in PREBUILT_HEAD_DIMS]
 
 

@@ -138,21 +138,24 @@ def cmd_decode_attention(args) -> int:
   part_ml = torch.empty(B * nq * splits * 2, device=DEV)
   turn = [0]
 
+  streams = ops.decode_streams_keys(B, nkv, d, L) if args.stream_keys == "auto" else args.stream_keys == "on"
+
   def plain():
     k, v = caches[turn[0] % copies]
     turn[0] += 1
-    ops.attn_decode(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0)
+    ops.attn_decode(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0, streams)
 
   def front():
     k, v = caches[turn[0] % copies]
     turn[0] += 1
     ops.attn_decode_front(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0,
-                          weight, weight, 1e-6, cos_sin, positions, slots)
+                          weight, weight, 1e-6, cos_sin, positions, slots, streams)
 
   calls = copies * max(1, args.calls // copies)
   for name, fn in (("attn_decode", plain), ("attn_decode_front", front)):
     t = graph_time_us(fn, calls)
-    print(f"{name}: {B} requests of {L} tokens, {nq}/{nkv} heads of {d}, {splits} splits, cache {cache_bytes / 1e6:.1f} MB: "
+    print(f"{name}: {B} requests of {L} tokens, {nq}/{nkv} heads of {d}, {splits} splits, "
+          f"{'nontemporal' if streams else 'ordinary'} loads, cache {cache_bytes / 1e6:.1f} MB: "
           f"{t:.1f} us with the merge, {cache_bytes / t / 1e6:.2f} TB/s")
   return 0
 
@@ -235,6 +238,8 @@ def main(argv=None) -> int:
   d.add_argument("--page-size", type=int, default=16)
   d.add_argument("--splits", type=int, default=0, help="key ranges per request (default: the engine's choice)")
   d.add_argument("--calls", type=int, default=24)
+  d.add_argument("--stream-keys", choices=["auto", "on", "off"], default="auto",
+                 help="nontemporal loads of the keys and values (auto: the engine's rule, ops.decode_streams_keys)")
   d.add_argument("--copies", type=int, default=0,
                  help="caches the calls cycle through, as a model's layers do (default: 2 to 8, 1.5 GB at most)")
   d.set_defaults(fn=cmd_decode_attention)

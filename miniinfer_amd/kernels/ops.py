@@ -97,10 +97,10 @@ _SIGS["attention_mfma"] = {
   "mi_attn_prefill": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                       c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
   "mi_attn_decode": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                     c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                     c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
   "mi_attn_decode_front": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                            c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int,
-                           c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
+                           c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
   "mi_attn_prefill_tokens_per_block": [c_int, c_int],
   "mi_attn_prefill_tokens_per_block_wide": [c_int, c_int],
 }
@@ -693,12 +693,26 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bo
     N //= 2
   if tuple(out.shape) != (M, N) or out.stride(1) != 1 or out.dtype not in (torch.bfloat16, torch.float32):
     raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit [{M}, {N}]")
-  lib = _lib("gemm_skinny")
+  lib = _skinny_lib(w)
   if variant is None:
     variant = skinny_variant(M, w.shape[0], K, gate_up)
   _skinny_call(lib, variant, out.dtype == torch.float32, gate_up, a, w, _ptr(out), out.stride(0) if M > 1 else N,
                M, N, K)
   return out
+
+
+# A matrix from this size on is read with nontemporal loads (a build of the kernels of its own): it is read once a
+# step and is larger than what the caches keep from one step to the next, so all it does there is push out what
+# could stay.  Measured on an MI355X, 8 rows: [151936, 1024] 56.4 -> 50.5 us, [151936, 4096] 213 -> 190,
+# gate|up [24576, 4096] 35.9 -> 31.9, [4096, 12288] 22.4 -> 20.4, gate|up [12288, 2048] 13.9 -> 12.9; matrices of
+# 34 MB and less lose (gate|up [6144, 1024] 5.4 -> 5.6, [4096, 4096] 8.5 -> 8.6, [8192, 2048] 9.8 -> 10.0).
+STREAMED_MATRIX_MIN_BYTES = 48 << 20
+
+
+def _skinny_lib(w: torch.Tensor):
+  if w.numel() * w.element_size() >= STREAMED_MATRIX_MIN_BYTES:
+    return _lib("gemm_skinny", (("SKINNY_NT", 1),))
+  return _lib("gemm_skinny")
 
 
 def gemm_skinny_waves(variant: int, num_rows: int, matrix_rows: int, k: int, gate_up: bool = False) -> int:
@@ -724,7 +738,7 @@ def gemm_skinny_scaled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_
     N //= 2
   if tuple(out.shape) != (M, N) or out.stride(1) != 1 or out.dtype not in (torch.bfloat16, torch.float32):
     raise KernelError(f"gemm_skinny: out {tuple(out.shape)} {out.dtype} does not fit [{M}, {N}]")
-  lib = _lib("gemm_skinny")
+  lib = _skinny_lib(w)
   ss_row = lib.mi_gemm_skinny_ss_row(M)
   if row_ss.dtype != torch.float32 or row_ss.dim() != 2 or row_ss.shape[1] != ss_row or not row_ss.is_contiguous():
     raise KernelError(f"gemm_skinny_scaled: row_ss must be a contiguous float32 [parts, {ss_row}] for {M} rows")
@@ -753,7 +767,7 @@ def gemm_skinny_into_norm(a: torch.Tensor, w: torch.Tensor, residual: torch.Tens
     raise KernelError("gemm_skinny_into_norm does not take these operands")
   M = a.shape[0]
   N, K = w.shape
-  lib = _lib("gemm_skinny")
+  lib = _skinny_lib(w)
   if variant is None:
     variant = skinny_variant(M, N, K)
   parts, _ = _skinny_plan(lib, variant, False, M, N, K)
@@ -797,7 +811,7 @@ def norm_gemm_skinny(residual: torch.Tensor, x: Optional[torch.Tensor], norm_wei
     if rows is not None or residual_out.shape != residual.shape or residual_out.dtype != torch.float32 \
         or not residual_out.is_contiguous() or residual_out.data_ptr() == residual.data_ptr():
       raise KernelError("norm_gemm_skinny: residual_out must be another float32 buffer of the residual's shape")
-  lib = _lib("gemm_skinny")
+  lib = _skinny_lib(w)
   _check(lib, lib.mi_norm_gemm_skinny(1 if gate_up else 0, _ptr(residual), _ptr(x), _ptr(residual_out),
                                       _ptr(norm_weight), _ptr(rows), float(eps), _ptr(w), w.stride(0), _ptr(out), N,
                                       M, N, K, _stream()))
@@ -972,13 +986,28 @@ def attn_prefill(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, 
                                   _PREFILL_VARIANTS[variant], _stream()))
 
 
+# A decode launch whose keys and values may come to this many bytes reads them with nontemporal loads: they are read
+# once a step and, with the weights, are many times what the caches hold, so ordinary loads only push out what could
+# stay.  Whole decode steps of the 0.6B shape (28 layers) at 2,048 tokens, nontemporal against ordinary loads: 8
+# requests (67 MB a layer) 1.325 against 1.304 ms, 16 the same, 24 (201 MB) 2.239 against 2.209, 32 (268 MB) 2.423
+# against 2.517, 48 3.172 against 3.335, 64 (537 MB) 3.68 against 4.08; one layer of 8 requests of 32,768 tokens
+# (1.07 GB) 178 against 194 us.  The caller's count of keys is an upper bound (a decode graph is made for tables of up
+# to twice the pages in use), hence a threshold of twice the size from which streaming pays.
+DECODE_STREAM_MIN_BYTES = 512 << 20
+
+
+def decode_streams_keys(num_entries: int, nkv: int, d: int, max_keys: int, element_size: int = 2) -> bool:
+  """Whether a decode attention launch over `num_entries` requests of up to `max_keys` keys should stream them."""
+  return 2 * num_entries * nkv * d * max_keys * element_size >= DECODE_STREAM_MIN_BYTES
+
+
 def attn_decode(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
                 v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor, kv_len: torch.Tensor,
                 first_entry: int, num_entries: int, num_splits: int, part_o: torch.Tensor, part_ml: torch.Tensor,
-                scale: float, window: int = 0) -> None:
+                scale: float, window: int = 0, stream_keys: bool = False) -> None:
   """MFMA split-key attention of entries first_entry .. first_entry + num_entries - 1, each of which brings exactly
   one token.  part_o float32 [>= num_entries * nq * num_splits * d], part_ml float32 [>= num_entries * nq *
-  num_splits * 2] are scratch."""
+  num_splits * 2] are scratch.  stream_keys: read the keys and values with nontemporal loads (`decode_streams_keys`)."""
   B = _attn_common("attn_decode", q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len)
   if first_entry < 0 or num_entries < 0 or first_entry + num_entries > B:
     raise KernelError(f"attn_decode: entries {first_entry}..{first_entry + num_entries} of {B}")
@@ -991,7 +1020,7 @@ def attn_decode(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k
   _check(lib, lib.mi_attn_decode(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages),
                                  _ptr(block_table), block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry,
                                  num_entries, num_splits, _ptr(part_o), _ptr(part_ml), nq, nkv, k_pages.shape[2],
-                                 float(scale), int(window), _stream()))
+                                 float(scale), int(window), 1 if stream_keys else 0, _stream()))
 
 
 def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
@@ -999,7 +1028,7 @@ def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.T
                       first_entry: int, num_entries: int, num_splits: int, part_o: torch.Tensor,
                       part_ml: torch.Tensor, scale: float, window: int, q_weight: Optional[torch.Tensor],
                       k_weight: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
-                      positions: torch.Tensor, slots: torch.Tensor) -> None:
+                      positions: torch.Tensor, slots: torch.Tensor, stream_keys: bool = False) -> None:
   """`attn_decode` for entries whose fused projection qkv [T, (nq + 2 nkv) d] (rows q | k | v) is still raw: the
   kernel does the per-head RMS norm of q and k (if weights), their rotation (if a table [max_pos, rotary_dim]) and
   the write of the new key and value to `slots`, as `qk_norm_rope_cache` would, and attends.  qkv is left as it is.
@@ -1030,8 +1059,8 @@ def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.T
   _check(lib, lib.mi_attn_decode_front(
     _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
     block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry, num_entries, num_splits, _ptr(part_o), _ptr(part_ml),
-    nq, nkv, k_pages.shape[2], float(scale), int(window), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos_sin),
-    rotary_dim, max_pos, _ptr(positions), _ptr(slots), _stream()))
+    nq, nkv, k_pages.shape[2], float(scale), int(window), 1 if stream_keys else 0, _ptr(q_weight), _ptr(k_weight),
+    float(eps), _ptr(cos_sin), rotary_dim, max_pos, _ptr(positions), _ptr(slots), _stream()))
 
 
 # ----------------------------------------------------------------------------- what the device delivers

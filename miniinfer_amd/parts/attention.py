@@ -156,13 +156,14 @@ class PagedAttention(Part):
     need = count * nq * splits
     part_o = ctx.scratch("attn_part_o", need * d, torch.float32)
     part_ml = ctx.scratch("attn_part_ml", need * 2, torch.float32)
+    streams = ops.decode_streams_keys(count, nkv, d, min(ctx.max_kv_len, window) if window else ctx.max_kv_len)
     if front is None:
       ops.attn_decode(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, first, count, splits,
-                      part_o, part_ml, self.scale, window)
+                      part_o, part_ml, self.scale, window, streams)
     else:
       ops.attn_decode_front(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, first, count, splits,
                             part_o, part_ml, self.scale, window, front[2], front[3], front[1], front[0],
-                            ctx.positions, ctx.slots[cache.group])
+                            ctx.positions, ctx.slots[cache.group], streams)
 
 
 def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, waves: int = 4,

@@ -343,6 +343,11 @@ def test_mfma_decode_attention_any_number_of_splits(nq, nkv, d, P, window, split
                   part_ml, d ** -0.5, window)
   torch.testing.assert_close(out.double().cpu()[5:], c["want"][5:], rtol=1.6e-2, atol=1e-2)
   assert float(out[:5].abs().sum()) == 0.0       # rows of the multi-token entries are not touched
+  # the keys and values read with nontemporal loads (as launches over many keys do): the same arithmetic
+  streamed = torch.zeros_like(out)
+  ops.attn_decode(c["q"], nq, nkv, d, streamed, c["kp"], c["vp"], c["table"], c["cu"], c["kv"], first, n, splits,
+                  part_o, part_ml, d ** -0.5, window, stream_keys=True)
+  assert torch.equal(streamed, out)
 
 
 @pytest.mark.parametrize("splits", [1, 5])
@@ -560,6 +565,11 @@ def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, win
                         cos_sin, pos.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV))
   torch.testing.assert_close(out.double().cpu(), want.double(), rtol=1.6e-2, atol=1e-2)
   assert torch.equal(c["q"], before)                     # the projection is read only
+  kp2, vp2, streamed = c["kp"].clone(), c["vp"].clone(), torch.zeros_like(out)
+  ops.attn_decode_front(c["q"], nq, nkv, d, streamed, kp2, vp2, c["table"], c["cu"], c["kv"], 0, B, splits, part_o,
+                        part_ml, d ** -0.5, window, qw.to(DEV) if with_norm else None, kw.to(DEV) if with_norm else None,
+                        eps, cos_sin, pos.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV), stream_keys=True)
+  assert torch.equal(streamed, out) and torch.equal(kp2, kp) and torch.equal(vp2, vp)   # nontemporal loads: same bits
   k_after, v_after = kp.float().cpu(), vp.float().cpu().transpose(2, 3)
   changed_k = (k_after != kc).any(-1)
   for b in range(B):
