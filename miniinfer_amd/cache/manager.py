@@ -211,6 +211,11 @@ class CacheManager:
     return sum(2 * n.num_kv_heads * n.head_dim * page_size * torch.empty((), dtype=n.dtype or dtype).element_size()
                for n in layer_needs if isinstance(n, PagedKV))
 
+  def token_bytes(self) -> int:
+    """Bytes of keys and values that one cached token holds in all layers (window groups counted like the others)."""
+    return sum(len(g.layers) * 2 * g.need.num_kv_heads * g.need.head_dim * torch.empty((), dtype=g.dtype).element_size()
+               for g in self.paged)
+
   def _allocate(self) -> None:
     for g in self.paged:
       n, h, d, P = len(g.layers), g.need.num_kv_heads, g.need.head_dim, g.page_size

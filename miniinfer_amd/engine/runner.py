@@ -163,6 +163,7 @@ class _DecodeGraph:
     ctx.future_tokens = runner.future_tokens
     self.ctx = ctx
     # every entry is padding while warming up and capturing: it reads and writes the scratch page only
+    runner.set_weight_streaming(B * W * cache.min_page_size)
     before, off_rule = ops.library_products_run(), ops.off_rule_products_run()
     self.graph, self.logits = self._capture(runner, ctx)
     self.ok = True
@@ -463,8 +464,14 @@ class ModelRunner:
             self._graphs[(b, w)] = _DecodeGraph(self, b, w)
     return len(self._graphs)
 
+  def set_weight_streaming(self, cached_tokens_bound: int) -> None:
+    """Says, for the step that follows, whether the weights are kept out of the last-level cache: they are where
+    the keys and values of the step's requests (at most `cached_tokens_bound` tokens) can stay there instead."""
+    self.choices.stream_weights = ops.weights_stream_past_cache(cached_tokens_bound * self.cache.token_bytes())
+
   def _step_eager(self, entries: Sequence[StepEntry]) -> torch.Tensor:
     ctx, order, kv_lens = self.build_context(entries)
+    self.set_weight_streaming(sum(kv_lens))
     logits = self.model.forward(ctx)
     if ctx._spare_used:                     # further copies out of the staging buffer were queued by the layers
       self._staging_done[self._staging_turn].record()

@@ -389,6 +389,7 @@ class ProductChoices:
     self.rule_only = bool(rule_only)
     self.own_only = False
     self.force: Optional[int] = None
+    self.stream_weights = False        # every matrix is read with nontemporal loads (set by the runner, step by step)
     self.library_products = [0, 0]     # (all, avoidable) products that went to the library
     self.off_rule = 0                  # products sent, by measurement, elsewhere than the rule would have
     self._outer: List["ProductChoices"] = []
@@ -708,9 +709,25 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate_up: bo
 # 34 MB and less lose (gate|up [6144, 1024] 5.4 -> 5.6, [4096, 4096] 8.5 -> 8.6, [8192, 2048] 9.8 -> 10.0).
 STREAMED_MATRIX_MIN_BYTES = 48 << 20
 
+# The last-level cache of an MI355X (256 MB) keeps the keys and values of a step for the next one if they fit and the
+# weights, which never do, are kept out of it: the current table's `stream_weights` then sends every matrix to the
+# nontemporal build.  Whole decode steps of the 0.6B shape, all weights nontemporal against only the large ones: one
+# request of 1,024 tokens (117 MB of keys and values in all layers) 0.992 against 1.036 ms, 2,048 tokens (235 MB) 1.010
+# against 1.050, 3,000 (344 MB) 1.035 against 1.050, 4,000 (459 MB) 1.066 against 1.050, 8,192 1.200 against 1.194;
+# 2 x 1,024 / 4 x 512 / 8 x 256 tokens 1.008 / 1.035 / 1.074 against 1.051 / 1.064 / 1.092; 2 x 2,048 1.077 against 1.067.
+# A step's count of cached tokens is an upper bound (decode graphs are made for tables of up to twice the pages in
+# use), so weights are streamed while the bound stays within twice the cache.
+LAST_LEVEL_CACHE_BYTES = 256 << 20
+
+
+def weights_stream_past_cache(cached_bytes_bound: int) -> bool:
+  """Whether a step that reads at most `cached_bytes_bound` bytes of keys and values (all layers) should keep its
+  weights out of the last-level cache, so that those keys and values are still there at the next step."""
+  return 0 < cached_bytes_bound <= 2 * LAST_LEVEL_CACHE_BYTES
+
 
 def _skinny_lib(w: torch.Tensor):
-  if w.numel() * w.element_size() >= STREAMED_MATRIX_MIN_BYTES:
+  if w.numel() * w.element_size() >= STREAMED_MATRIX_MIN_BYTES or _CURRENT[0].stream_weights:
     return _lib("gemm_skinny", (("SKINNY_NT", 1),))
   return _lib("gemm_skinny")
 

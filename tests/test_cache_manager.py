@@ -219,3 +219,21 @@ def test_random_orders_keep_the_books_of_unlike_groups(seed):
     m.release(r)
   m.check()
   assert m.all_pages_free() and m.num_free_slots() == 5
+
+
+def test_token_bytes_and_the_rule_that_keeps_weights_out_of_the_last_level_cache():
+  """A cached token's bytes over all layers; weights are streamed past the cache while a step's keys and values
+  (an upper bound) stay within twice its size, and never for a step without any."""
+  import torch
+  from miniinfer_amd.cache.manager import CacheManager
+  from miniinfer_amd.kernels import ops
+  from miniinfer_amd.parts import PagedKV
+  needs = [PagedKV(8, 128)] * 28
+  cm = CacheManager(needs, 16, 64, 4, 1024, torch.bfloat16, torch.device("cpu"), allocate=False)
+  assert cm.token_bytes() == 28 * 2 * 8 * 128 * 2 == 114688
+  mixed = CacheManager([PagedKV(2, 64), PagedKV(2, 64, window=32), PagedKV(4, 32, dtype=torch.float32)], 16, 64, 4,
+                       1024, torch.bfloat16, torch.device("cpu"), allocate=False)
+  assert mixed.token_bytes() == 2 * (2 * 2 * 64 * 2) + 2 * 4 * 32 * 4
+  tb = cm.token_bytes()
+  assert ops.weights_stream_past_cache(1 * 4096 * tb) and ops.weights_stream_past_cache(2 * 2048 * tb)
+  assert not ops.weights_stream_past_cache(4 * 2048 * tb) and not ops.weights_stream_past_cache(0)
