@@ -311,6 +311,9 @@ class ModelRunner:
     # future_tokens[r] as it is when the step's embedding kernel runs: whoever samples writes here, and may
     # launch the next step before reading the tokens back.
     self.future_tokens = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=self.device)
+    if self.device.type == "cuda":
+      from ..kernels import prepare
+      prepare(model.ctx.dtype, [g.need.head_dim for g in cache.paged])      # what is not built yet, side by side
 
   def graph_pool(self):
     if self._graph_pool is None:
