@@ -34,7 +34,14 @@ def _ptr(t: Optional[torch.Tensor]):
   return None if t is None else t.data_ptr()
 
 
+# the current stream's handle, asked for by every launch: torch's raw accessor where it has one (a tenth of the cost
+# of building a Stream object: a prompt's step of 28 layers asks 145 times)
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+  if _RAW_STREAM is not None:
+    return _RAW_STREAM(torch.cuda.current_device())
   return torch.cuda.current_stream().cuda_stream
 
 
