@@ -1040,6 +1040,118 @@ chunks_done:
   }
 }
 
+// The same workgroup (128 weight rows, a range of k, partials P[split][m][n]) for matrices that are streamed from
+// memory: both operands go straight to LDS (global_load_lds: lane i's 16 bytes land at base + 16 i) through a ring of
+// SR_NBUF stages of 128 k, a wave's load instruction covering 1 KB (4 rows x 256 bytes) of whole memory lines, where
+// the kernel above fetches the weights in the matrix cores' operand shape (16 rows x 64 bytes an instruction), which
+// streams at two thirds of the rate.  Stage i + 2 is asked for before stage i is multiplied; a wave waits for its
+// own loads of a stage by count (loads come back in the order they were asked for) and a barrier makes the stage
+// every wave's.  A row's 16 pieces of 16 bytes are stored with their places exchanged by the row's number (piece q
+// of row r at place q xor (r mod 16)), so that the 16 rows an operand read takes its pieces from lie in different
+// banks.  k and every split's range are multiples of 128 here; rows of W past N and of A past M repeat the last row
+// (loads to LDS cannot be replaced by zeros) and are never stored.
+constexpr int SR_NBUF = 3;
+constexpr int SR_WROWS = 128;
+template <int MB>
+__global__ __launch_bounds__(256) void gemm_splitk_ring_kernel(const uint16_t* __restrict__ A, int64_t lda,
+                                                               const uint16_t* __restrict__ W, int64_t ldw,
+                                                               float* __restrict__ P, int64_t ldp, void* __restrict__ C,
+                                                               int64_t ldc, int out_f32, int M, int N, int K, int kr) {
+  constexpr int AROWS = 16 * MB;
+  constexpr int STAGE = (SR_WROWS + AROWS) * SK_KC;      // elements of a stage: the weight rows, then the rows of A
+  constexpr int W_LOADS = SR_WROWS / 16;                 // wave loads (4 rows) of a stage that one of the 4 waves issues
+  constexpr int LW = W_LOADS + MB;                       // with its loads of A
+  extern __shared__ __attribute__((aligned(16))) uint16_t ring[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n0 = blockIdx.x * SR_WROWS;
+  const int split = blockIdx.y;
+  const int k_lo = split * kr;
+  const int k_hi = min(K, k_lo + kr);
+  const int nst = k_hi > k_lo ? (k_hi - k_lo) / SK_KC : 0;
+  // this lane's piece of every wave load: row rr of its 4 rows, place `at` of the row's 16
+  const int rr = lane >> 4, at = lane & 15;
+  const uint16_t* wsrc[W_LOADS];
+  const uint16_t* asrc[MB];
+#pragma unroll
+  for (int j = 0; j < W_LOADS; ++j) {
+    const int r = 4 * (wave + 4 * j) + rr;
+    wsrc[j] = W + (int64_t)min(n0 + r, N - 1) * ldw + k_lo + 8 * (at ^ (r & 15));
+  }
+#pragma unroll
+  for (int j = 0; j < MB; ++j) {
+    const int r = 4 * (wave + 4 * j) + rr;
+    asrc[j] = A + (int64_t)min(r, M - 1) * lda + k_lo + 8 * (at ^ (r & 15));
+  }
+  auto issue = [&](int st) {
+    uint16_t* base = ring + (st % SR_NBUF) * STAGE;
+    const int k0 = st * SK_KC;
+#pragma unroll
+    for (int j = 0; j < MB; ++j)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(asrc[j] + k0),
+                                       (__attribute__((address_space(3))) void*)(base + SR_WROWS * SK_KC + (wave + 4 * j) * 512),
+                                       16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < W_LOADS; ++j)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc[j] + k0),
+                                       (__attribute__((address_space(3))) void*)(base + (wave + 4 * j) * 512), 16, 0,
+                                       W_LDS_AUX);
+  };
+  f32x4 acc[2][MB];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int st = 0; st < SR_NBUF - 1 && st < nst; ++st) issue(st);
+  const int row = lane & 15, kg = lane >> 4;
+  for (int i = 0; i < nst; ++i) {
+    // the compiler does not count the loads that write LDS: the waits are written out
+    if (i + 1 < nst) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LW) : "memory");     // stage i + 1 may still be on its way
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // stage i is here; everyone is past stage i - 1
+    if (i + SR_NBUF - 1 < nst) issue(i + SR_NBUF - 1);                // into the buffer stage i - 1 was in
+    const uint16_t* wst = ring + (i % SR_NBUF) * STAGE;
+    const uint16_t* ast = wst + SR_WROWS * SK_KC;
+#pragma unroll
+    for (int s = 0; s < SK_STEPS; ++s) {
+      const int place = 8 * ((4 * s + kg) ^ row);
+      bf16x8 w[2];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+        w[rb] = *reinterpret_cast<const bf16x8*>(wst + (32 * wave + 16 * rb + row) * SK_KC + place);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(ast + (16 * mb + row) * SK_KC + place);
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+          acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[rb], a, acc[rb][mb], 0, 0, 0);
+      }
+    }
+  }
+  // lane holds C^T[n0 + 32 wave + 16 rb + 4 (lane / 16) + i][16 mb + lane % 16]
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    const int nb = n0 + 32 * wave + 16 * rb;
+    if (nb >= N) break;
+    const int n = nb + 4 * (lane >> 4);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = 16 * mb + (lane & 15);
+      if (m >= M) continue;
+      if (C) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) {
+            if (out_f32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n + i] = acc[rb][mb][i];
+            else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n + i] = float_to_bf16_bits(acc[rb][mb][i]);
+          }
+      } else {
+        *reinterpret_cast<f32x4*>(P + ((int64_t)split * M + m) * ldp + n) = acc[rb][mb];
+      }
+    }
+  }
+}
+
 // Adds the partials and finishes the product.  Grid (ceil(N / 256), ceil(M / waves)), 1 or 4 waves a workgroup (one
 // where that still leaves few workgroups): wave w takes row waves * blockIdx.y + w, a lane 4 columns.  N counts result columns; with gate_up the partials hold 2 N (gate | up).
 struct SplitkEnd {
@@ -1132,6 +1244,14 @@ struct SplitkPlan {
   int64_t ldp;
 };
 
+// for measurements: 0 keeps every k-split product on the kernel that fetches its weights into registers
+static int g_splitk_ring = 1;
+MI_EXPORT int mi_gemm_skinny_ring(int on) {
+  const int was = g_splitk_ring;
+  g_splitk_ring = on;
+  return was;
+}
+
 static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
   SplitkPlan p;
   // weight rows per workgroup: 128 for matrices of many rows, 32 for those of few (which need the workgroups)
@@ -1141,12 +1261,14 @@ static SplitkPlan splitk_plan(int M, int rows, int K, int want_splits) {
   const int tn = 16 * p.wn * p.rb;
   p.groups = (rows + tn - 1) / tn;
   // one workgroup for every compute unit: with twice as many (and half the k range each) every shape measured was
-  // slower, by 5 to 25%
+  // slower, by 5 to 25% (the ring kernel too: 64 rows of [4096, 12288] 27.4 us in 8 splits, 31 in 6 or 12, 39 in 2;
+  // gate|up [24576, 4096] 46 us in its 192 row groups unsplit, 52 to 87 in 2 to 16 splits, whose partials grow)
   const int target = compute_units();
   int s = want_splits > 0 ? want_splits : (target + p.groups / 2) / p.groups;
   if (s < 1) s = 1;
   if (s > 32) s = 32;
   int kr = ((K + s - 1) / s + 31) / 32 * 32;
+  if (K % SK_KC == 0) kr = (kr + SK_KC - 1) / SK_KC * SK_KC;      // whole stages of the ring kernel
   if (kr < 256) kr = 256;
   if (kr > SK_MAX_CHUNKS * SK_KC) kr = SK_MAX_CHUNKS * SK_KC;
   p.kr = kr;
@@ -1205,6 +1327,24 @@ MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void
              (long long)p.splits * M * p.ldp);
   const int MB = (M + 15) / 16;
   const dim3 grid(p.groups, p.splits);
+  // matrices of many rows, k in whole stages, 16-byte alignment: the kernel that takes both operands through LDS
+  if (g_splitk_ring && p.wn == 4 && K % SK_KC == 0 && p.kr % SK_KC == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
+    const size_t lds = (size_t)SR_NBUF * (SR_WROWS + 16 * MB) * SK_KC * sizeof(uint16_t);
+#define RING(mb)                                                                                                 \
+  {                                                                                                              \
+    static bool allowed = false;                                                                                 \
+    if (!allowed) {                                                                                              \
+      (void)hipFuncSetAttribute((const void*)gemm_splitk_ring_kernel<mb>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                160 * 1024);                                                                     \
+      allowed = true;                                                                                            \
+    }                                                                                                            \
+    gemm_splitk_ring_kernel<mb><<<grid, 256, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, ldw, scratch, \
+                                                            p.ldp, nullptr, ldc, out_f32, M, rows, K, p.kr);     \
+  }
+    if (MB == 1) RING(1) else if (MB == 2) RING(2) else if (MB == 3) RING(3) else RING(4)
+#undef RING
+    MI_CHECK_LAUNCH("gemm_skinny (k split, ring)");
+  } else {
 #define GO(mb, wn, rb, d)                                                                                       \
   gemm_splitk_kernel<mb, wn, rb, d><<<grid, 64 * wn, 0, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W,   \
                                                                   ldw, scratch, p.ldp, nullptr, ldc, out_f32, M, \
@@ -1222,6 +1362,7 @@ MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void
   }
 #undef GO
   MI_CHECK_LAUNCH("gemm_skinny (k split)");
+  }
   const SplitkEnd e{row_ss, ss_parts, SS_ROW(M), eps, residual, norm_weight, (uint16_t*)a_out, ss_out};
   const int red_waves = (int64_t)((N + 255) / 256) * M <= 2048 ? 1 : 4;
   splitk_reduce_kernel<<<dim3((N + 255) / 256, (M + red_waves - 1) / red_waves), 64 * red_waves, 0, stream>>>(
