@@ -1052,19 +1052,33 @@ chunks_done:
 // (loads to LDS cannot be replaced by zeros) and are never stored.
 constexpr int SR_NBUF = 3;
 constexpr int SR_WROWS = 128;
-template <int MB>
+// END: how a workgroup leaves its sums.  0: partials P[split][m][n] for the kernel below (any number of splits).
+// 1 (one split, nothing to do but store): the result itself.  2 (one split, a fused gate|up matrix of 2 N rows): the
+// workgroup takes 64 gate rows and the 64 up rows of the same result columns, so a wave holds both sums of its
+// columns and stores silu(gate) * up itself, the rows scaled first by rsqrt(sum_p row_ss[p][m] / K + eps) if row_ss
+// is given (N is then the number of result columns).
+struct RingEnd {
+  const float* row_ss;      // [ss_parts][ss_row] or null
+  int ss_parts;
+  int ss_row;
+  float eps;
+};
+template <int MB, int END>
 __global__ __launch_bounds__(256) void gemm_splitk_ring_kernel(const uint16_t* __restrict__ A, int64_t lda,
                                                                const uint16_t* __restrict__ W, int64_t ldw,
                                                                float* __restrict__ P, int64_t ldp, void* __restrict__ C,
-                                                               int64_t ldc, int out_f32, int M, int N, int K, int kr) {
+                                                               int64_t ldc, int out_f32, int M, int N, int K, int kr,
+                                                               RingEnd e) {
   constexpr int AROWS = 16 * MB;
   constexpr int STAGE = (SR_WROWS + AROWS) * SK_KC;      // elements of a stage: the weight rows, then the rows of A
   constexpr int W_LOADS = SR_WROWS / 16;                 // wave loads (4 rows) of a stage that one of the 4 waves issues
   constexpr int LW = W_LOADS + MB;                       // with its loads of A
+  constexpr int HALF = SR_WROWS / 2;
   extern __shared__ __attribute__((aligned(16))) uint16_t ring[];
+  __shared__ float ss_part[4][64];                       // END 2 with row_ss: the four waves' shares of the rows' sums
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n0 = blockIdx.x * SR_WROWS;
+  const int n0 = blockIdx.x * (END == 2 ? HALF : SR_WROWS);     // first weight row (END 2: first result column)
   const int split = blockIdx.y;
   const int k_lo = split * kr;
   const int k_hi = min(K, k_lo + kr);
@@ -1075,8 +1089,11 @@ __global__ __launch_bounds__(256) void gemm_splitk_ring_kernel(const uint16_t* _
   const uint16_t* asrc[MB];
 #pragma unroll
   for (int j = 0; j < W_LOADS; ++j) {
-    const int r = 4 * (wave + 4 * j) + rr;
-    wsrc[j] = W + (int64_t)min(n0 + r, N - 1) * ldw + k_lo + 8 * (at ^ (r & 15));
+    const int r = 4 * (wave + 4 * j) + rr;        // row of the stage
+    int64_t wr;
+    if (END == 2) wr = r < HALF ? min(n0 + r, N - 1) : N + min(n0 + r - HALF, N - 1);   // gate rows, then up rows
+    else wr = min(n0 + r, N - 1);
+    wsrc[j] = W + wr * ldw + k_lo + 8 * (at ^ (r & 15));
   }
 #pragma unroll
   for (int j = 0; j < MB; ++j) {
@@ -1103,7 +1120,15 @@ __global__ __launch_bounds__(256) void gemm_splitk_ring_kernel(const uint16_t* _
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int st = 0; st < SR_NBUF - 1 && st < nst; ++st) issue(st);
+  if (END == 2 && e.row_ss) {       // while the first stages are on their way: wave w adds parts w, w + 4, ... of row `lane`
+    float ssum = 0.f;
+    for (int p = wave; p < e.ss_parts; p += 4) ssum += e.row_ss[(int64_t)p * e.ss_row + min(lane, e.ss_row - 1)];
+    ss_part[wave][lane] = ssum;     // read after the loop's barriers (a product has at least one stage)
+  }
   const int row = lane & 15, kg = lane >> 4;
+  // LDS rows of this wave's two blocks of 16 weight rows
+  const int wrow0 = (END == 2 ? 16 * wave : 32 * wave) + row;
+  const int wrow1 = (END == 2 ? HALF + 16 * wave : 32 * wave + 16) + row;
   for (int i = 0; i < nst; ++i) {
     // the compiler does not count the loads that write LDS: the waits are written out
     if (i + 1 < nst) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LW) : "memory");     // stage i + 1 may still be on its way
@@ -1116,9 +1141,8 @@ __global__ __launch_bounds__(256) void gemm_splitk_ring_kernel(const uint16_t* _
     for (int s = 0; s < SK_STEPS; ++s) {
       const int place = 8 * ((4 * s + kg) ^ row);
       bf16x8 w[2];
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
-        w[rb] = *reinterpret_cast<const bf16x8*>(wst + (32 * wave + 16 * rb + row) * SK_KC + place);
+      w[0] = *reinterpret_cast<const bf16x8*>(wst + wrow0 * SK_KC + place);
+      w[1] = *reinterpret_cast<const bf16x8*>(wst + wrow1 * SK_KC + place);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(ast + (16 * mb + row) * SK_KC + place);
@@ -1127,6 +1151,28 @@ __global__ __launch_bounds__(256) void gemm_splitk_ring_kernel(const uint16_t* _
           acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[rb], a, acc[rb][mb], 0, 0, 0);
       }
     }
+  }
+  if (END == 2) {
+    // lane holds gate and up sums of result columns n0 + 16 wave + 4 (lane / 16) + i, row 16 mb + lane % 16
+    const int nb = n0 + 16 * wave;
+    if (nb >= N) return;
+    const int n = nb + 4 * (lane >> 4);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int m = 16 * mb + (lane & 15);
+      if (m >= M) continue;
+      float rstd = 1.f;
+      if (e.row_ss)
+        rstd = rsqrtf(((ss_part[0][m] + ss_part[1][m]) + (ss_part[2][m] + ss_part[3][m])) / (float)K + e.eps);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < N) {
+          const float v = silu_f(acc[0][mb][i] * rstd) * (acc[1][mb][i] * rstd);
+          if (out_f32) reinterpret_cast<float*>(C)[(int64_t)m * ldc + n + i] = v;
+          else reinterpret_cast<uint16_t*>(C)[(int64_t)m * ldc + n + i] = float_to_bf16_bits(v);
+        }
+    }
+    return;
   }
   // lane holds C^T[n0 + 32 wave + 16 rb + 4 (lane / 16) + i][16 mb + lane % 16]
 #pragma unroll
@@ -1138,7 +1184,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_ring_kernel(const uint16_t* _
     for (int mb = 0; mb < MB; ++mb) {
       const int m = 16 * mb + (lane & 15);
       if (m >= M) continue;
-      if (C) {
+      if (END == 1) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           if (n + i < N) {
@@ -1330,20 +1376,32 @@ MI_EXPORT int mi_gemm_skinny_v(int variant, int out_f32, int gate_up, const void
   // matrices of many rows, k in whole stages, 16-byte alignment: the kernel that takes both operands through LDS
   if (g_splitk_ring && p.wn == 4 && K % SK_KC == 0 && p.kr % SK_KC == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
     const size_t lds = (size_t)SR_NBUF * (SR_WROWS + 16 * MB) * SK_KC * sizeof(uint16_t);
-#define RING(mb)                                                                                                 \
+    // one split: no partials.  A fused gate|up matrix is taken 64 gate and 64 up rows to a workgroup, which stores
+    // the activation itself; a product with nothing to do at its end but store is stored by its workgroups.
+    const int end = p.splits == 1 ? (gate_up ? 2 : (!row_ss && !residual ? 1 : 0)) : 0;
+    const dim3 rgrid(end == 2 ? (N + SR_WROWS / 2 - 1) / (SR_WROWS / 2) : p.groups, p.splits);
+    const RingEnd re{row_ss, ss_parts, SS_ROW(M), eps};
+#define RING(mb, END)                                                                                            \
   {                                                                                                              \
     static bool allowed = false;                                                                                 \
     if (!allowed) {                                                                                              \
-      (void)hipFuncSetAttribute((const void*)gemm_splitk_ring_kernel<mb>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                160 * 1024);                                                                     \
+      /* what this instance needs, no more: its static LDS counts against the same 160 KB */                    \
+      const hipError_t err_ = hipFuncSetAttribute((const void*)gemm_splitk_ring_kernel<mb, END>,                 \
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);         \
+      MI_REQUIRE(err_ == hipSuccess, "gemm_skinny (k split, ring): %s", hipGetErrorString(err_));                \
       allowed = true;                                                                                            \
     }                                                                                                            \
-    gemm_splitk_ring_kernel<mb><<<grid, 256, lds, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W, ldw, scratch, \
-                                                            p.ldp, nullptr, ldc, out_f32, M, rows, K, p.kr);     \
+    gemm_splitk_ring_kernel<mb, END><<<rgrid, 256, lds, stream>>>(                                               \
+        (const uint16_t*)A, lda, (const uint16_t*)W, ldw, scratch, p.ldp, END ? C : nullptr, ldc, out_f32, M,     \
+        END == 2 ? N : rows, K, p.kr, re);                                                                       \
   }
-    if (MB == 1) RING(1) else if (MB == 2) RING(2) else if (MB == 3) RING(3) else RING(4)
+#define RING_MB(END)                                                                                             \
+  if (MB == 1) RING(1, END) else if (MB == 2) RING(2, END) else if (MB == 3) RING(3, END) else RING(4, END)
+    if (end == 2) { RING_MB(2) } else if (end == 1) { RING_MB(1) } else { RING_MB(0) }
+#undef RING_MB
 #undef RING
     MI_CHECK_LAUNCH("gemm_skinny (k split, ring)");
+    if (end) return 0;
   } else {
 #define GO(mb, wn, rb, d)                                                                                       \
   gemm_splitk_kernel<mb, wn, rb, d><<<grid, 64 * wn, 0, stream>>>((const uint16_t*)A, lda, (const uint16_t*)W,   \

@@ -313,7 +313,7 @@ class ModelRunner:
     self.future_tokens = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=self.device)
     if self.device.type == "cuda":
       from ..kernels import prepare
-      prepare(model.ctx.dtype, [g.need.head_dim for g in cache.paged])      # what is not built yet, side by side
+      prepare(cache.dtype, [g.need.head_dim for g in cache.paged])      # what is not built yet, side by side
 
   def graph_pool(self):
     if self._graph_pool is None:

@@ -402,7 +402,8 @@ def test_mfma_attention_finds_a_far_key_and_respects_the_window_edge():
                                    (3, 151936, 256), (33, 48, 2048), (5, 130, 88), (64, 1000, 40), (7, 2050, 64),
                                    (16, 1001, 512), (48, 1024, 4360), (64, 100, 12288), (20, 2064, 1000),
                                    (9, 1024, 2048), (13, 520, 3072), (30, 1000, 6144), (64, 272, 1024), (4, 2050, 4096),
-                                   (6, 600, 192), (16, 5120, 2560), (5, 300, 6400), (64, 40, 4224), (2, 2000, 128)])
+                                   (6, 600, 192), (16, 5120, 2560), (5, 300, 6400), (64, 40, 4224), (2, 2000, 128),
+                                   (64, 30001, 256)])
 def test_gemm_skinny(M, N, K, out_dtype, variant):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(9)
@@ -464,7 +465,8 @@ def test_gemm_skinny_drawn_shapes():
 
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("M,I,K", [(8, 3072, 1024), (1, 112, 80), (40, 160, 96), (64, 100, 256), (33, 1028, 2200),
-                                   (8, 1536, 4096), (16, 516, 2048), (48, 260, 1024), (3, 200, 5120), (20, 36, 448)])
+                                   (8, 1536, 4096), (16, 516, 2048), (48, 260, 1024), (3, 200, 5120), (20, 36, 448),
+                                   (64, 12288, 512), (5, 11012, 256)])      # k split: unsplit, the kernel's own ending
 def test_gemm_skinny_gate_up_activation(M, I, K, variant):
   from miniinfer_amd.kernels import ops
   g = torch.Generator().manual_seed(10)
@@ -583,7 +585,7 @@ def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, win
 @pytest.mark.parametrize("M,N,K,N2,gate_up", [(8, 1024, 2048, 6144, True), (1, 80, 96, 112, False), (16, 1024, 3072, 4096, False),
                                                (40, 136, 264, 200, True), (64, 1024, 2048, 3072, False), (5, 88, 40, 24, False),
                                                (12, 2056, 96, 160, True), (64, 1024, 3072, 4096, False),
-                                               (33, 520, 2304, 132, True)])
+                                               (33, 520, 2304, 132, True), (40, 1024, 256, 11008, True)])
 @pytest.mark.parametrize("variants", [(0, 0), (1, 0), (0, 1), (1, 1), (2, 2), (2, 1), (4, 3), (3, 4), (5, 5), (6, 6), (6, 1)])
 def test_norm_split_between_two_products(M, N, K, N2, gate_up, variants):
   """residual += a W1^T; y = rmsnorm(residual) * w; out = y W2^T (or the gated activation of it), the add and the
