@@ -82,3 +82,30 @@ def test_product_kernel_choice_falls_back_to_the_rule_and_obeys_measurements():
     assert ops.product_choice_known(4096, 4096, False) and not ops.product_choice_known(4096, 4096, True)
   finally:
     ops.clear_product_choices()
+
+
+def test_what_a_decode_step_reads_past_the_caches():
+  """Keys and values of a launch are streamed (nontemporal loads) from 512 MB on, counted with the upper bound of keys a
+  decode graph is made for; matrices from 48 MB on go to the nontemporal build of the product kernels, and every matrix
+  does while the table in use says so (the runner does, for steps whose keys and values fit the last-level cache)."""
+  import torch
+  from miniinfer_amd.kernels import ops
+  # Qwen3-0.6B shape: 8 kv heads of 128, bfloat16: 4 KB a token and layer
+  assert not ops.decode_streams_keys(8, 8, 128, 4096) and not ops.decode_streams_keys(24, 8, 128, 4096)
+  assert ops.decode_streams_keys(32, 8, 128, 4096) and ops.decode_streams_keys(64, 8, 128, 2048)
+  assert ops.decode_streams_keys(8, 8, 128, 32768) and not ops.decode_streams_keys(1, 8, 128, 32768)
+  assert ops.decode_streams_keys(16, 8, 128, 4096, element_size=4)
+  small = torch.empty(1024, 2048, dtype=torch.bfloat16, device="meta")
+  head = torch.empty(151936, 1024, dtype=torch.bfloat16, device="meta")
+  picked = []
+  real = ops._lib
+  ops._lib = lambda name, defines=(): picked.append(defines) or defines
+  try:
+    table = ops.ProductChoices()
+    with table:
+      assert ops._skinny_lib(small) == () and ops._skinny_lib(head) == (("SKINNY_NT", 1),)
+      table.stream_weights = True
+      assert ops._skinny_lib(small) == (("SKINNY_NT", 1),)
+    assert ops._skinny_lib(small) == ()          # another table is in use again: its own switch counts
+  finally:
+    ops._lib = real
