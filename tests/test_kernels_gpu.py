@@ -428,6 +428,28 @@ def test_gemm_skinny(M, N, K, out_dtype, variant):
       assert variant == 5 and (M, N, K) == (16, 5120, 2560)
 
 
+@pytest.mark.parametrize("M,N,K,gate_up", [(8, 4096, 1024, False), (64, 3072, 1024, True), (40, 1000, 2048, False),
+                                          (33, 12288, 512, True), (16, 5120, 2560, False)])
+def test_gemm_skinny_nontemporal_build_gives_the_same_bits(M, N, K, gate_up):
+  """The build of the product kernels whose weight loads are nontemporal (for matrices too large to stay in the caches,
+  and for every matrix while the table in use says `stream_weights`) does the same arithmetic: equal results in every
+  form."""
+  from miniinfer_amd.kernels import ops
+  g = torch.Generator().manual_seed(12)
+  a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+  w = (torch.randn(2 * N if gate_up else N, K, generator=g) * 0.1).bfloat16().to(DEV)
+  table = ops.ProductChoices()
+  for variant in (0, 1, 2, 3, 4, 5, 6):
+    plain = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    streamed = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_skinny(a, w, plain, gate_up=gate_up, variant=variant)
+    with table:
+      table.stream_weights = True
+      ops.gemm_skinny(a, w, streamed, gate_up=gate_up, variant=variant)
+    assert torch.equal(plain, streamed), variant
+  assert ("gemm_skinny", (("SKINNY_NT", 1),)) in ops._libs and ("gemm_skinny", ()) in ops._libs
+
+
 def test_gemm_skinny_drawn_shapes():
   """Every form of the weight-streaming product on shapes drawn at random (rows 1 to 64, k a multiple of 8 from 8 to
   6,400, 1 to 5,000 columns, left operands with a row stride of their own, a third of them gate|up), against 64-bit
