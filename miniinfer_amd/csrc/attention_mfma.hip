@@ -572,7 +572,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
 // combines the partials with the log-sum-exp rule.  (Merging inside this kernel, by the workgroup that
 // finishes last, was measured: the device-wide fences it needs cost many times the second launch.)
 // Partials: part_o [entries, nq, num_splits, D], part_ml [entries, nq, num_splits, 2] (max in base-2 units).
+// A launch whose key ranges make two such workgroups or more for every compute unit runs with workgroups of twice
+// the waves and half the ranges instead (WAVES = DECODE_WAVES_WIDE): half as many workgroups to hand out, fewer
+// heads a wave for the norms and the rotation, half the partials for the merge (8 requests of 2,048 tokens: 19.1
+// against 20.5 us with the merge, 16 requests 30.0 against 32.7; one request, whose 64 workgroups are few enough
+// already, 12.8 against 11.5, so the caller says which).
 constexpr int DECODE_WAVES = D > 128 ? 2 : 4;
+constexpr int DECODE_WAVES_WIDE = 2 * DECODE_WAVES;
 
 // With FRONT, the kernel also does what precedes attention for a decoded token (fused_qwen3.py:98-107 of the
 // reference): `q` is then the raw fused projection [tokens, (nq + 2 nkv) D] with rows q | k | v.  Every workgroup
@@ -594,16 +600,16 @@ struct DecodeFront {
 
 __device__ __forceinline__ float bf16_at(const uint16_t* p) { return __uint_as_float((uint32_t)(*p) << 16); }
 
-template <bool FRONT, bool STREAM>
-__global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_kernel(
+template <bool FRONT, bool STREAM, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) DECODE_OCCUPANCY void decode_kernel(
     const uint16_t* __restrict__ q, int64_t q_row_stride, uint16_t* __restrict__ out, int64_t out_row_stride,
     const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_len, int first_entry,
     float* __restrict__ part_o, float* __restrict__ part_ml, int nq, int nkv, int page_shift, float scale,
     int window, DecodeFront front) {
-  __shared__ float lds_o[DECODE_WAVES][DBLK][64][4];
-  __shared__ float lds_m[DECODE_WAVES][16];
-  __shared__ float lds_l[DECODE_WAVES][16];
+  __shared__ float lds_o[WAVES][DBLK][64][4];
+  __shared__ float lds_m[WAVES][16];
+  __shared__ float lds_l[WAVES][16];
   __shared__ __attribute__((aligned(16))) uint16_t lds_q[FRONT ? 16 * D : 8];   // normed, rotated queries of the group
   __shared__ __attribute__((aligned(16))) uint16_t lds_k[FRONT ? D : 8];        // and the new key
   const int lane = threadIdx.x & 63;
@@ -662,10 +668,10 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_ker
     // straight-line code.  So everything the norm and the rotation read is asked for first, without branches
     // (absent operands read a stand-in address and are replaced afterwards), in two dependent rounds (the
     // position, then its angles); the first macro tile is asked for after that, and the arithmetic runs while the
-    // tile is on its way.  Wave w takes heads w, w + DECODE_WAVES, ... of the group's query heads followed by
+    // tile is on its way.  Wave w takes heads w, w + WAVES, ... of the group's query heads followed by
     // its key head; a lane takes the rotation pairs (j, j + D/2), j = lane + 64 c.  Without a rotation table
     // the pairs are "rotated" by the angle 0.
-    constexpr int HPW = (17 + DECODE_WAVES - 1) / DECODE_WAVES;
+    constexpr int HPW = (17 + WAVES - 1) / WAVES;
     constexpr int HALF = D / 2;
     constexpr int NP = (HALF + 63) / 64;
     const uint16_t* row = q + (int64_t)token * q_row_stride;
@@ -676,7 +682,7 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_ker
     float xa[HPW][NP], xb[HPW][NP];
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
-      const int hh = wave + DECODE_WAVES * i;
+      const int hh = wave + WAVES * i;
       const uint16_t* src = row + (int64_t)(hh < G ? g * G + hh : nq + g) * D;
 #pragma unroll
       for (int cc = 0; cc < NP; ++cc) {
@@ -716,7 +722,7 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_ker
     }
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
-      const int hh = wave + DECODE_WAVES * i;
+      const int hh = wave + WAVES * i;
       if (hh <= G) {                           // the same for every lane of the wave
         const bool is_key = hh == G;
         uint16_t* dst = is_key ? lds_k : lds_q + hh * D;
@@ -754,7 +760,7 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_ker
     softmax_update<1>(st, s, p, c, j0, pos_lo, pos_hi);
 #pragma unroll
     for (int t = 0; t < MT; t += 2) tile_values<1>(st, va[t], va[t + 1], p[t], p[t + 1]);
-    mt += DECODE_WAVES;
+    mt += WAVES;
     if (mt < t1) DECODE_FETCH(mt)
   }
 #undef DECODE_FETCH
@@ -816,11 +822,11 @@ __global__ __launch_bounds__(64 * DECODE_WAVES) DECODE_OCCUPANCY void decode_ker
     if (col >= G) continue;
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < DECODE_WAVES; ++w) M = fmaxf(M, lds_m[w][col]);
+    for (int w = 0; w < WAVES; ++w) M = fmaxf(M, lds_m[w][col]);
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float L = 0.f;
 #pragma unroll
-    for (int w = 0; w < DECODE_WAVES; ++w) {
+    for (int w = 0; w < WAVES; ++w) {
       const float mw = lds_m[w][col];
       const float wt = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - M);
       const f32x4 v = *reinterpret_cast<const f32x4*>(&lds_o[w][blk][slot][0]);
@@ -1067,6 +1073,7 @@ MI_EXPORT int mi_attn_macro_tile_keys() { return MKEYS; }
 
 // Waves per workgroup of the decode kernel.
 MI_EXPORT int mi_attn_decode_waves() { return DECODE_WAVES; }
+MI_EXPORT int mi_attn_decode_waves_wide() { return DECODE_WAVES_WIDE; }
 
 // Query tokens per work item (a workgroup of 4 waves, 16 * PREFILL_NB columns each) of the prefill launch.
 MI_EXPORT int mi_attn_prefill_tokens_per_block(int nq, int nkv) {
@@ -1129,11 +1136,12 @@ MI_EXPORT int mi_attn_prefill(const void* q, int64_t q_row_stride, void* out, in
 // Entries first_entry .. first_entry + num_entries - 1 must each bring exactly one token.
 // part_o: float [num_entries * nq * num_splits * D]; part_ml: float [num_entries * nq * num_splits * 2].
 // stream_keys: read the keys and values with nontemporal loads (for launches that read many times the caches' size).
+// wide: workgroups of mi_attn_decode_waves_wide() waves instead of mi_attn_decode_waves().
 MI_EXPORT int mi_attn_decode(const void* q, int64_t q_row_stride, void* out, int64_t out_row_stride, const void* k_pages,
                              const void* v_pages, const int* block_table, int table_width, const int* cu_q,
                              const int* kv_len, int first_entry, int num_entries, int num_splits, float* part_o,
                              float* part_ml, int nq, int nkv, int page_size, float scale, int window,
-                             int stream_keys, hipStream_t stream) {
+                             int stream_keys, int wide, hipStream_t stream) {
   if (check_common("attn_decode", nq, nkv, page_size, q_row_stride, out_row_stride, table_width)) return 1;
   if (check_scale("attn_decode", scale)) return 1;
   MI_REQUIRE(num_entries >= 0 && first_entry >= 0 && window >= 0, "attn_decode: bad entry range or window");
@@ -1142,13 +1150,18 @@ MI_EXPORT int mi_attn_decode(const void* q, int64_t q_row_stride, void* out, int
   MI_REQUIRE(num_splits == 1 || (part_o && part_ml), "attn_decode: no partial buffers");
   if (num_entries == 0) return 0;
   dim3 grid(num_splits, nkv, num_entries);
-#define DECODE_GO(FRONT, STREAM, Q, QS, F)                                                                          \
-  decode_kernel<FRONT, STREAM><<<grid, 64 * DECODE_WAVES, 0, stream>>>(                                             \
+#define DECODE_GO_W(FRONT, STREAM, WV, Q, QS, F)                                                                   \
+  decode_kernel<FRONT, STREAM, WV><<<grid, 64 * WV, 0, stream>>>(                                                   \
       (const uint16_t*)(Q), QS, (uint16_t*)out, out_row_stride, (const uint16_t*)k_pages, (const uint16_t*)v_pages, \
       block_table, table_width, cu_q, kv_len, first_entry, part_o, part_ml, nq, nkv, log2_of(page_size), scale,     \
       window, F)
-  if (stream_keys) DECODE_GO(false, true, q, q_row_stride, DecodeFront{});
-  else DECODE_GO(false, false, q, q_row_stride, DecodeFront{});
+#define DECODE_GO(FRONT, STREAM, Q, QS, F)                                                                          \
+  {                                                                                                                  \
+    if (wide) DECODE_GO_W(FRONT, STREAM, DECODE_WAVES_WIDE, Q, QS, F);                                               \
+    else DECODE_GO_W(FRONT, STREAM, DECODE_WAVES, Q, QS, F);                                                         \
+  }
+  if (stream_keys) DECODE_GO(false, true, q, q_row_stride, DecodeFront{})
+  else DECODE_GO(false, false, q, q_row_stride, DecodeFront{})
   MI_CHECK_LAUNCH("attn_decode");
   if (num_splits > 1) {
     launch_decode_merge(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q, first_entry, num_entries, nq, num_splits,
@@ -1165,7 +1178,7 @@ MI_EXPORT int mi_attn_decode_front(const void* qkv, int64_t qkv_row_stride, void
                                    void* k_pages, void* v_pages, const int* block_table, int table_width,
                                    const int* cu_q, const int* kv_len, int first_entry, int num_entries, int num_splits,
                                    float* part_o, float* part_ml, int nq, int nkv, int page_size, float scale,
-                                   int window, int stream_keys, const float* q_weight, const float* k_weight,
+                                   int window, int stream_keys, int wide, const float* q_weight, const float* k_weight,
                                    float eps, const float* cos_sin, int rotary_dim, int max_pos,
                                    const int* positions, const int* slots, hipStream_t stream) {
   if (check_common("attn_decode_front", nq, nkv, page_size, qkv_row_stride, out_row_stride, table_width)) return 1;
@@ -1184,9 +1197,10 @@ MI_EXPORT int mi_attn_decode_front(const void* qkv, int64_t qkv_row_stride, void
   DecodeFront front{q_weight, k_weight, eps, cos_sin, rotary_dim, max_pos, positions, slots, (uint16_t*)k_pages,
                     (uint16_t*)v_pages};
   dim3 grid(num_splits, nkv, num_entries);
-  if (stream_keys) DECODE_GO(true, true, qkv, qkv_row_stride, front);
-  else DECODE_GO(true, false, qkv, qkv_row_stride, front);
+  if (stream_keys) DECODE_GO(true, true, qkv, qkv_row_stride, front)
+  else DECODE_GO(true, false, qkv, qkv_row_stride, front)
 #undef DECODE_GO
+#undef DECODE_GO_W
   MI_CHECK_LAUNCH("attn_decode_front");
   if (num_splits > 1) {
     launch_decode_merge(part_o, part_ml, (uint16_t*)out, out_row_stride, cu_q, first_entry, num_entries, nq, num_splits,
@@ -1244,5 +1258,5 @@ MI_EXPORT int mi_attn_decode_static(const void* q, int64_t q_row_stride, void* o
   if (static_scratch(&base)) return 1;
   return mi_attn_decode(q, q_row_stride, out, out_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len,
                         first_entry, num_entries, num_splits, base, base + ml_offset, nq, nkv, page_size, scale, window,
-                        0, stream);
+                        0, 0, stream);
 }

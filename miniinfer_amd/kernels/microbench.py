@@ -110,7 +110,7 @@ def cmd_prefill_attention(args) -> int:
 
 
 def cmd_decode_attention(args) -> int:
-  from ..parts.attention import decode_splits
+  from ..parts.attention import decode_launch, decode_splits
   nq, nkv, d, P, B, L = args.heads, args.kv_heads, args.head_dim, args.page_size, args.batch, args.context
   if not ops.mfma_attention_supported(torch.bfloat16, nq, nkv, d, P):
     print("these sizes go to the plain attention kernel, which this command does not time", file=sys.stderr)
@@ -133,7 +133,12 @@ def cmd_decode_attention(args) -> int:
   cos_sin = torch.cat([angles.cos(), angles.sin()], dim=1).contiguous()
   out = torch.empty(B, nq * d, dtype=torch.bfloat16, device=DEV)
   tile_keys, waves = ops.attn_decode_geometry(d)
-  splits = args.splits or decode_splits(B * nkv, L, tile_keys, waves)
+  splits, wide = decode_launch(B * nkv, L, tile_keys, waves, 2 * ops.compute_units())
+  if args.wide != "auto":
+    wide = args.wide == "on"
+    splits = decode_splits(B * nkv, L, tile_keys, waves, 2 * ops.compute_units())
+    splits = (splits + 1) // 2 if wide and splits >= 2 else splits
+  splits = args.splits or splits
   part_o = torch.empty(B * nq * splits * d, device=DEV)
   part_ml = torch.empty(B * nq * splits * 2, device=DEV)
   turn = [0]
@@ -143,18 +148,19 @@ def cmd_decode_attention(args) -> int:
   def plain():
     k, v = caches[turn[0] % copies]
     turn[0] += 1
-    ops.attn_decode(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0, streams)
+    ops.attn_decode(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0, streams, wide)
 
   def front():
     k, v = caches[turn[0] % copies]
     turn[0] += 1
     ops.attn_decode_front(qkv, nq, nkv, d, out, k, v, table, cu, kv, 0, B, splits, part_o, part_ml, d ** -0.5, 0,
-                          weight, weight, 1e-6, cos_sin, positions, slots, streams)
+                          weight, weight, 1e-6, cos_sin, positions, slots, streams, wide)
 
   calls = copies * max(1, args.calls // copies)
   for name, fn in (("attn_decode", plain), ("attn_decode_front", front)):
     t = graph_time_us(fn, calls)
     print(f"{name}: {B} requests of {L} tokens, {nq}/{nkv} heads of {d}, {splits} splits, "
+          f"{ops.attn_decode_geometry(d, wide)[1]} waves a workgroup, "
           f"{'nontemporal' if streams else 'ordinary'} loads, cache {cache_bytes / 1e6:.1f} MB: "
           f"{t:.1f} us with the merge, {cache_bytes / t / 1e6:.2f} TB/s")
   return 0
@@ -238,6 +244,8 @@ def main(argv=None) -> int:
   d.add_argument("--page-size", type=int, default=16)
   d.add_argument("--splits", type=int, default=0, help="key ranges per request (default: the engine's choice)")
   d.add_argument("--calls", type=int, default=24)
+  d.add_argument("--wide", choices=["auto", "on", "off"], default="auto",
+                 help="workgroups of twice the waves and half the key ranges (auto: the engine's rule, decode_launch)")
   d.add_argument("--stream-keys", choices=["auto", "on", "off"], default="auto",
                  help="nontemporal loads of the keys and values (auto: the engine's rule, ops.decode_streams_keys)")
   d.add_argument("--copies", type=int, default=0,

@@ -104,10 +104,10 @@ _SIGS["attention_mfma"] = {
   "mi_attn_prefill": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                       c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
   "mi_attn_decode": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                     c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+                     c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void_p],
   "mi_attn_decode_front": [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                            c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int,
-                           c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
+                           c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
   "mi_attn_prefill_tokens_per_block": [c_int, c_int],
   "mi_attn_prefill_tokens_per_block_wide": [c_int, c_int],
 }
@@ -962,10 +962,11 @@ def attn_prefill_wide_pays(q_lens, nq: int, nkv: int, d: int) -> int:
   return tpb if items * nkv >= PREFILL_WIDE_WORKGROUPS_PER_UNIT * compute_units() else 0
 
 
-def attn_decode_geometry(d: int):
-  """(keys per macro tile, waves per workgroup) of the decode kernel for this head size."""
+def attn_decode_geometry(d: int, wide: bool = False):
+  """(keys per macro tile, waves per workgroup) of the decode kernel for this head size; wide: of its launch with
+  workgroups of twice the waves."""
   lib = _lib("attention_mfma", (("HEAD_DIM", d),))
-  return lib.mi_attn_macro_tile_keys(), lib.mi_attn_decode_waves()
+  return lib.mi_attn_macro_tile_keys(), (lib.mi_attn_decode_waves_wide() if wide else lib.mi_attn_decode_waves())
 
 
 def _attn_common(what, q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len):
@@ -1028,10 +1029,11 @@ def decode_streams_keys(num_entries: int, nkv: int, d: int, max_keys: int, eleme
 def attn_decode(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
                 v_pages: torch.Tensor, block_table: torch.Tensor, cu_q: torch.Tensor, kv_len: torch.Tensor,
                 first_entry: int, num_entries: int, num_splits: int, part_o: torch.Tensor, part_ml: torch.Tensor,
-                scale: float, window: int = 0, stream_keys: bool = False) -> None:
+                scale: float, window: int = 0, stream_keys: bool = False, wide: bool = False) -> None:
   """MFMA split-key attention of entries first_entry .. first_entry + num_entries - 1, each of which brings exactly
   one token.  part_o float32 [>= num_entries * nq * num_splits * d], part_ml float32 [>= num_entries * nq *
-  num_splits * 2] are scratch.  stream_keys: read the keys and values with nontemporal loads (`decode_streams_keys`)."""
+  num_splits * 2] are scratch.  stream_keys: read the keys and values with nontemporal loads (`decode_streams_keys`);
+  wide: workgroups of twice the waves (`attn_decode_geometry(d, wide=True)`; see `decode_launch` of the attention part)."""
   B = _attn_common("attn_decode", q, out, nq, nkv, d, k_pages, v_pages, block_table, cu_q, kv_len)
   if first_entry < 0 or num_entries < 0 or first_entry + num_entries > B:
     raise KernelError(f"attn_decode: entries {first_entry}..{first_entry + num_entries} of {B}")
@@ -1044,7 +1046,7 @@ def attn_decode(q: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k
   _check(lib, lib.mi_attn_decode(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages),
                                  _ptr(block_table), block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry,
                                  num_entries, num_splits, _ptr(part_o), _ptr(part_ml), nq, nkv, k_pages.shape[2],
-                                 float(scale), int(window), 1 if stream_keys else 0, _stream()))
+                                 float(scale), int(window), 1 if stream_keys else 0, 1 if wide else 0, _stream()))
 
 
 def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.Tensor, k_pages: torch.Tensor,
@@ -1052,7 +1054,8 @@ def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.T
                       first_entry: int, num_entries: int, num_splits: int, part_o: torch.Tensor,
                       part_ml: torch.Tensor, scale: float, window: int, q_weight: Optional[torch.Tensor],
                       k_weight: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
-                      positions: torch.Tensor, slots: torch.Tensor, stream_keys: bool = False) -> None:
+                      positions: torch.Tensor, slots: torch.Tensor, stream_keys: bool = False,
+                      wide: bool = False) -> None:
   """`attn_decode` for entries whose fused projection qkv [T, (nq + 2 nkv) d] (rows q | k | v) is still raw: the
   kernel does the per-head RMS norm of q and k (if weights), their rotation (if a table [max_pos, rotary_dim]) and
   the write of the new key and value to `slots`, as `qk_norm_rope_cache` would, and attends.  qkv is left as it is.
@@ -1083,7 +1086,8 @@ def attn_decode_front(qkv: torch.Tensor, nq: int, nkv: int, d: int, out: torch.T
   _check(lib, lib.mi_attn_decode_front(
     _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
     block_table.shape[1], _ptr(cu_q), _ptr(kv_len), first_entry, num_entries, num_splits, _ptr(part_o), _ptr(part_ml),
-    nq, nkv, k_pages.shape[2], float(scale), int(window), 1 if stream_keys else 0, _ptr(q_weight), _ptr(k_weight),
+    nq, nkv, k_pages.shape[2], float(scale), int(window), 1 if stream_keys else 0, 1 if wide else 0, _ptr(q_weight),
+    _ptr(k_weight),
     float(eps), _ptr(cos_sin), rotary_dim, max_pos, _ptr(positions), _ptr(slots), _stream()))
 
 

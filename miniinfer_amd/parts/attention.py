@@ -151,19 +151,19 @@ class PagedAttention(Part):
     nq, nkv, d, window = self.nq, self.nkv, self.d, self.window or 0
     table = ctx.block_tables[cache.group]
     tile_keys, waves = ops.attn_decode_geometry(d)
-    splits = decode_splits(count * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len, tile_keys, waves,
-                           2 * ops.compute_units())
+    splits, wide = decode_launch(count * nkv, min(ctx.max_kv_len, window) if window else ctx.max_kv_len, tile_keys,
+                                 waves, 2 * ops.compute_units())
     need = count * nq * splits
     part_o = ctx.scratch("attn_part_o", need * d, torch.float32)
     part_ml = ctx.scratch("attn_part_ml", need * 2, torch.float32)
     streams = ops.decode_streams_keys(count, nkv, d, min(ctx.max_kv_len, window) if window else ctx.max_kv_len)
     if front is None:
       ops.attn_decode(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, first, count, splits,
-                      part_o, part_ml, self.scale, window, streams)
+                      part_o, part_ml, self.scale, window, streams, wide)
     else:
       ops.attn_decode_front(qkv, nq, nkv, d, out, cache.k, cache.v, table, ctx.cu_q, ctx.kv_len, first, count, splits,
                             part_o, part_ml, self.scale, window, front[2], front[3], front[1], front[0],
-                            ctx.positions, ctx.slots[cache.group], streams)
+                            ctx.positions, ctx.slots[cache.group], streams, wide)
 
 
 def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, waves: int = 4,
@@ -181,6 +181,24 @@ def decode_splits(num_head_entries: int, max_keys: int, tile_keys: int = 64, wav
   if want == 1 and n < resident_workgroups and 5 * n <= 4 * resident_workgroups:
     want = 2
   return int(max(1, min(want, max(1, tiles // waves), 64)))
+
+
+def decode_launch(num_head_entries: int, max_keys: int, tile_keys: int = 64, waves: int = 4,
+                  resident_workgroups: int = 512):
+  """(key ranges, wide) of a decode launch: `decode_splits`' ranges with workgroups of `waves` waves, or half the
+  ranges with workgroups of twice the waves (`wide`): half as many workgroups to hand out, fewer heads a wave for the
+  norms and the rotation, half the partials to merge or none at all.  Wide workgroups pay where they are a single
+  round of one a compute unit and still half a round (or, where they need no merge, a quarter): requests x us with
+  the merge, 2,048 keys each, wide against not: 4 x 14.1 / 14.5, 8 x 19.2 / 20.5, 16 x 30.1 / 32.4, 24 x 40.0 / 46.0,
+  32 x 50.2 / 53.8; 512 keys each: 8 x 10.5 / 12.3, 32 x 17.1 / 21.5; but 1 x 12.8 / 11.5 (too few workgroups), 12 x
+  33.8 / 26.6 and 48 x 82.1 / 77.4 (a second round)."""
+  splits = decode_splits(num_head_entries, max_keys, tile_keys, waves, resident_workgroups)
+  units = resident_workgroups // 2
+  half = (splits + 1) // 2
+  groups = max(1, num_head_entries) * half
+  if splits >= 2 and groups <= units and (2 * groups >= units or (half == 1 and 4 * groups >= units)):
+    return half, True
+  return splits, False
 
 
 def plain_splits(num_waves: int, max_keys: int, resident_waves: int = 4096) -> int:

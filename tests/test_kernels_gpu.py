@@ -348,6 +348,13 @@ def test_mfma_decode_attention_any_number_of_splits(nq, nkv, d, P, window, split
   ops.attn_decode(c["q"], nq, nkv, d, streamed, c["kp"], c["vp"], c["table"], c["cu"], c["kv"], first, n, splits,
                   part_o, part_ml, d ** -0.5, window, stream_keys=True)
   assert torch.equal(streamed, out)
+  # workgroups of twice the waves (as launches of many workgroups get): the macro tiles go to other waves, so the
+  # sums are rounded elsewhere; held to the same reference
+  wide = torch.zeros_like(out)
+  ops.attn_decode(c["q"], nq, nkv, d, wide, c["kp"], c["vp"], c["table"], c["cu"], c["kv"], first, n, splits, part_o,
+                  part_ml, d ** -0.5, window, wide=True)
+  torch.testing.assert_close(wide.double().cpu()[5:], c["want"][5:], rtol=1.6e-2, atol=1e-2)
+  assert float(wide[:5].abs().sum()) == 0.0
 
 
 @pytest.mark.parametrize("splits", [1, 5])
@@ -594,6 +601,12 @@ def test_mfma_decode_with_fused_norm_rotation_and_cache_write(nq, nkv, d, P, win
                         part_ml, d ** -0.5, window, qw.to(DEV) if with_norm else None, kw.to(DEV) if with_norm else None,
                         eps, cos_sin, pos.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV), stream_keys=True)
   assert torch.equal(streamed, out) and torch.equal(kp2, kp) and torch.equal(vp2, vp)   # nontemporal loads: same bits
+  kp3, vp3, wide = c["kp"].clone(), c["vp"].clone(), torch.zeros_like(out)          # workgroups of twice the waves
+  ops.attn_decode_front(c["q"], nq, nkv, d, wide, kp3, vp3, c["table"], c["cu"], c["kv"], 0, B, splits, part_o,
+                        part_ml, d ** -0.5, window, qw.to(DEV) if with_norm else None, kw.to(DEV) if with_norm else None,
+                        eps, cos_sin, pos.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV), wide=True)
+  torch.testing.assert_close(wide.double().cpu(), want.double(), rtol=1.6e-2, atol=1e-2)
+  assert torch.equal(kp3, kp) and torch.equal(vp3, vp)                                # the same cache writes
   k_after, v_after = kp.float().cpu(), vp.float().cpu().transpose(2, 3)
   changed_k = (k_after != kc).any(-1)
   for b in range(B):

@@ -19,6 +19,19 @@ def test_decode_key_ranges_fill_one_round_and_stay_few():
   assert decode_splits(8 * 8, 2048) == 8 and decode_splits(12 * 8, 2048) == 5 and decode_splits(24 * 8, 2048) == 2
   assert decode_splits(48 * 8, 2048) == 2 and decode_splits(64 * 8, 2048) == 1
   assert decode_splits(8, 8192) == 32 and decode_splits(8, 32768) == 64 and decode_splits(8, 2048) == 8
+  # launches that fill a round of two workgroups a compute unit with two ranges or more take workgroups of twice the
+  # waves and half the ranges; few workgroups and unsplit launches stay as they are
+  from miniinfer_amd.parts.attention import decode_launch
+  assert decode_launch(8 * 8, 2048) == (4, True) and decode_launch(16 * 8, 2048) == (2, True)
+  assert decode_launch(32 * 8, 2048) == (1, True) and decode_launch(24 * 8, 2048) == (1, True)
+  assert decode_launch(4 * 8, 2048) == (4, True) and decode_launch(8 * 8, 512) == (1, True)
+  assert decode_launch(8, 2048) == (8, False) and decode_launch(2 * 8, 2048) == (8, False)       # too few workgroups
+  assert decode_launch(12 * 8, 2048) == (5, False) and decode_launch(48 * 8, 2048) == (2, False)  # a second round
+  assert decode_launch(64 * 8, 2048) == (1, False) and decode_launch(8, 32768) == (32, True)
+  for n in (1, 8, 64, 100, 256, 384, 512):
+    for keys in (100, 2048, 32768):
+      s, wide = decode_launch(n, keys)
+      assert s >= 1 and s * (8 if wide else 4) <= max(8 if wide else 4, -(-keys // 64)), (n, keys, s, wide)
   assert decode_splits(16, 32768) == 32 and decode_splits(1, 1 << 20) == 64
   assert decode_splits(8 * 4, 2048, 32, 2) == 16 and decode_splits(64 * 4, 2048, 32, 2) == 2
 

@@ -25,7 +25,7 @@ def _load(d=D):
   common = [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int,
             c_int, c_int]
   tail = [c_int, c_int, c_int, c_float, c_int, c_void_p]
-  lib.mi_attn_decode.argtypes = common + [c_void_p, c_void_p] + tail[:-1] + [c_int, c_void_p]   # + stream_keys
+  lib.mi_attn_decode.argtypes = common + [c_void_p, c_void_p] + tail[:-1] + [c_int, c_int, c_void_p]   # + stream_keys, wide
   lib.mi_attn_decode_static.argtypes = common + tail
   for f in (lib.mi_attn_decode, lib.mi_attn_decode_static, lib.mi_attn_static_scratch_floats):
     f.restype = c_int
@@ -65,7 +65,7 @@ def _run(lib, c, entries, nq, nkv, P, splits, static, D=D, window=0, first=0):
     need = (entries - first) * nq * splits
     part_o = torch.empty(need * D, dtype=torch.float32, device=out.device)
     part_ml = torch.empty(need * 2, dtype=torch.float32, device=out.device)
-    rc = lib.mi_attn_decode(*args, part_o.data_ptr(), part_ml.data_ptr(), *tail[:-1], 0, stream)
+    rc = lib.mi_attn_decode(*args, part_o.data_ptr(), part_ml.data_ptr(), *tail[:-1], 0, 0, stream)
   assert rc == 0, lib.mi_last_error().decode()
   torch.cuda.synchronize()
   return out
