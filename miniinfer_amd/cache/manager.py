@@ -38,6 +38,9 @@ class CacheError(RuntimeError):
   pass
 
 
+SPREAD_EVERY = 33
+
+
 class PagePool:
   """Free list of page ids 1..num_pages (page 0 is a scratch page that is never handed out).
   Pages freed last are handed out first, so reuse shows early."""
@@ -46,7 +49,14 @@ class PagePool:
     if num_pages <= 0:
       raise ValueError("a page pool needs at least one page")
     self.num_pages = num_pages
-    self._free: List[int] = list(range(num_pages, 0, -1))
+    # Ascending, but every SPREAD_EVERY-th page only after all the others: requests of the same power-of-two length
+    # (benchmarks love 2,048 tokens) would otherwise lie a power of two apart in memory, and the workgroups of a
+    # decode step, which walk their requests' pages side by side, would ask the same few memory channels at the same
+    # time (64 requests of 2,048 tokens of the 0.6B shape: 17,300 -> 17,830 tok/s with 33, 17,600 with 17, 17,700 with
+    # 129; the attention kernel over the engine's own tables 96.3 us a layer, 91.5 with their pages shuffled).
+    first = [p for p in range(1, num_pages + 1) if p % SPREAD_EVERY]
+    last = [p for p in range(1, num_pages + 1) if p % SPREAD_EVERY == 0]
+    self._free: List[int] = (first + last)[::-1]
     self._held = bytearray(num_pages + 1)
 
   @property
