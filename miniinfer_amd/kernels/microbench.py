@@ -122,7 +122,14 @@ def cmd_decode_attention(args) -> int:
   g = torch.Generator(device=DEV).manual_seed(0)
   caches = [(torch.randn(pages + 1, nkv, P, d, device=DEV, generator=g).bfloat16(),
              torch.randn(pages + 1, nkv, d, P, device=DEV, generator=g).bfloat16()) for _ in range(copies)]
-  table = (torch.randperm(pages, device=DEV, generator=g) + 1).to(torch.int32).view(B, per_req)
+  if args.pages == "ascending":        # request after request, as a free list in plain ascending order would hand them out
+    table = (torch.arange(pages, device=DEV) + 1).to(torch.int32).view(B, per_req)
+  elif args.pages == "pool":           # as the engine's page pool hands them out
+    from ..cache.manager import PagePool
+    pool = PagePool(pages)
+    table = torch.tensor([pool.alloc(per_req) for _ in range(B)], dtype=torch.int32, device=DEV)
+  else:
+    table = (torch.randperm(pages, device=DEV, generator=g) + 1).to(torch.int32).view(B, per_req)
   qkv = torch.randn(B, (nq + 2 * nkv) * d, device=DEV, generator=g).bfloat16()
   cu = torch.arange(B + 1, dtype=torch.int32, device=DEV)
   kv = torch.full((B,), L, dtype=torch.int32, device=DEV)
@@ -244,6 +251,9 @@ def main(argv=None) -> int:
   d.add_argument("--page-size", type=int, default=16)
   d.add_argument("--splits", type=int, default=0, help="key ranges per request (default: the engine's choice)")
   d.add_argument("--calls", type=int, default=24)
+  d.add_argument("--pages", choices=["shuffled", "ascending", "pool"], default="shuffled",
+                 help="which pages the requests hold: a random choice, request after request in ascending order, or "
+                      "as the engine's page pool hands them out")
   d.add_argument("--wide", choices=["auto", "on", "off"], default="auto",
                  help="workgroups of twice the waves and half the key ranges (auto: the engine's rule, decode_launch)")
   d.add_argument("--stream-keys", choices=["auto", "on", "off"], default="auto",
